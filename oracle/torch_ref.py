@@ -1,0 +1,72 @@
+"""TEST INFRASTRUCTURE ONLY -- torch-on-CPU restatement of the reference's Python path.
+
+Second, independent formulation of the three operators, built from library
+``transpose`` / ``flip`` / ``einsum`` the way the reference's torch fallbacks
+are.  It serves two purposes: (1) it cross-checks the C oracle (two
+formulations written differently must agree), (2) it is the "reference torch
+CPU path" that the benchmark times on the host cores as ``cpu_baseline``.
+
+Follows, without importing them:
+  cross_scan   classification/models/csm_triton.py:22-29 and :532-541
+  cross_merge  classification/models/csm_triton.py:56-62 and :543-551
+  selective_scan  kernels/selective_scan/test_selective_scan.py:168-234
+                  (selective_scan_ref; same arithmetic as csms6s.py:25-68 but
+                  the bias add and softplus happen after the widening to fp32,
+                  as in the device kernel, selective_scan_fwd_kernel_oflex.cuh:123-127)
+"""
+import torch
+import torch.nn.functional as F
+
+
+def cross_scan(x):
+    B, C, H, W = x.shape
+    row_major = x.reshape(B, C, H * W)
+    col_major = x.transpose(2, 3).reshape(B, C, H * W)
+    return torch.stack([row_major, col_major, row_major.flip(-1), col_major.flip(-1)], dim=1)
+
+
+def cross_merge(ys):
+    B, K, C, H, W = ys.shape
+    y = ys.reshape(B, K, C, H * W)
+    both = y[:, 0:2] + y[:, 2:4].flip(-1)            # (y0 + flip y2), (y1 + flip y3)
+    col = both[:, 1].reshape(B, C, W, H).transpose(2, 3).reshape(B, C, H * W)
+    return both[:, 0] + col
+
+
+def cross_merge_left_to_right(ys):
+    """Add order of the Triton kernel, csm_triton.py:362-370: ((y0+y1')+y2')+y3'."""
+    B, K, C, H, W = ys.shape
+    y = ys.reshape(B, K, C, H * W)
+    t = lambda v: v.reshape(B, C, W, H).transpose(2, 3).reshape(B, C, H * W)
+    return ((y[:, 0] + t(y[:, 1])) + y[:, 2].flip(-1)) + t(y[:, 3].flip(-1))
+
+
+def selective_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
+                   return_last_state=False):
+    dtype_in = u.dtype
+    batch, dim, L = u.shape
+    G, N = B.shape[1], B.shape[2]
+    u32, dl = u.float(), delta.float()
+    if delta.shape[1] != dim:                       # delta-group broadcast, oflex.h dim_deltagroups_ratio
+        rep = dim // delta.shape[1]
+        dl = dl.repeat_interleave(rep, dim=1)
+        if delta_bias is not None:
+            delta_bias = delta_bias.repeat_interleave(rep)
+    if delta_bias is not None:
+        dl = dl + delta_bias.float()[None, :, None]
+    if delta_softplus:
+        dl = F.softplus(dl)
+    Bf = B.float().repeat_interleave(dim // G, dim=1)  # (batch, dim, N, L)
+    Cf = C.float().repeat_interleave(dim // G, dim=1)
+    decay = torch.exp(torch.einsum("bdl,dn->bdln", dl, A.float()))
+    drive = torch.einsum("bdl,bdnl,bdl->bdln", dl, Bf, u32)
+    h = torch.zeros(batch, dim, N, dtype=torch.float32)
+    ys = []
+    for t in range(L):
+        h = decay[:, :, t] * h + drive[:, :, t]
+        ys.append(torch.einsum("bdn,bdn->bd", h, Cf[..., t]))
+    y = torch.stack(ys, dim=2) if L > 0 else torch.zeros(batch, dim, 0)
+    if D is not None:
+        y = y + u32 * D.float()[None, :, None]
+    out = y if out_float else y.to(dtype_in)
+    return (out, h) if return_last_state else out

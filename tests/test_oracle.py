@@ -1,0 +1,251 @@
+"""Pins the CPU oracle (oracle/ss2d_oracle.c and oracle/torch_ref.py) without the reference.
+
+Every check is chosen so that a plausible slip (a transposed index, a dropped flip, a wrong
+add order, a missing bias, the wrong group for B/C) fails at least one of them.
+"""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+from oracle import ss2d_oracle as orc
+from oracle import torch_ref
+
+
+@pytest.fixture(scope="module")
+def kat(golden_dir):
+    with open(os.path.join(golden_dir, "cross_scan_kat.json")) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="module")
+def scan_golden(golden_dir):
+    with open(os.path.join(golden_dir, "selective_scan_f64.json")) as f:
+        return json.load(f)
+
+
+# ---------------------------------------------------------------- cross scan
+@pytest.mark.parametrize("impl", [orc.cross_scan, torch_ref.cross_scan])
+def test_cross_scan_known_answers(kat, impl):
+    for case in kat["scan"]:
+        H, W = case["H"], case["W"]
+        x = torch.tensor(case["x"], dtype=torch.float32).view(1, 1, H, W)
+        y = impl(x)
+        assert y.shape == (1, 4, 1, H * W)
+        assert y.view(4, -1).tolist() == [[float(v) for v in row] for row in case["y"]]
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 3, 3, 5), (1, 2, 7, 7), (2, 2, 14, 14), (1, 3, 56, 57), (1, 2, 57, 58)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.int64, torch.uint8])
+def test_cross_scan_brute_force_and_second_formulation(shape, dtype):
+    B, C, H, W = shape
+    g = torch.Generator().manual_seed(1)
+    x = torch.randint(0, 250, shape, generator=g).to(dtype)
+    y = orc.cross_scan(x)
+    assert torch.equal(y, torch_ref.cross_scan(x))
+    L = H * W
+    for b in range(B):
+        for c in range(C):
+            for h in range(0, H, max(1, H // 5)):
+                for w in range(0, W, max(1, W // 5)):
+                    v = x[b, c, h, w]
+                    assert y[b, 0, c, h * W + w] == v
+                    assert y[b, 1, c, w * H + h] == v
+                    assert y[b, 2, c, L - 1 - (h * W + w)] == v
+                    assert y[b, 3, c, L - 1 - (w * H + h)] == v
+    # each direction is a permutation of the map
+    for k in range(4):
+        assert torch.equal(y[:, k].float().sort(-1).values, x.reshape(B, C, L).float().sort(-1).values)
+
+
+def test_cross_scan_empty():
+    assert orc.cross_scan(torch.zeros(0, 3, 4, 4)).shape == (0, 4, 3, 16)
+    assert orc.cross_scan(torch.zeros(2, 0, 4, 4)).shape == (2, 4, 0, 16)
+
+
+# --------------------------------------------------------------- cross merge
+@pytest.mark.parametrize("impl", [orc.cross_merge, torch_ref.cross_merge])
+def test_cross_merge_known_answer(kat, impl):
+    m = kat["merge"]
+    ys = torch.tensor(m["ys"], dtype=torch.float32).view(1, 4, 1, m["H"], m["W"])
+    assert impl(ys).view(-1).tolist() == [float(v) for v in m["out"]]
+    for case in kat["scan"]:
+        ys = torch.tensor(case["y"], dtype=torch.float32).view(1, 4, 1, case["H"], case["W"])
+        assert impl(ys).view(-1).tolist() == [float(v) for v in case["merged"]]
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 3, 5), (1, 2, 7, 7), (1, 3, 56, 57), (1, 2, 57, 58)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cross_merge_matches_second_formulation_bitwise(shape, dtype):
+    B, C, H, W = shape
+    g = torch.Generator().manual_seed(2)
+    ys = torch.randn((B, 4, C, H, W), generator=g).to(dtype)
+    assert torch.equal(orc.cross_merge(ys), torch_ref.cross_merge(ys))
+    assert torch.equal(orc.cross_merge(ys, order=1), torch_ref.cross_merge_left_to_right(ys))
+
+
+def test_cross_merge_add_order_is_observable():
+    # values chosen so that fp32 rounding separates the two association orders
+    y = torch.zeros(1, 4, 1, 1, 1)
+    y[0, 0], y[0, 1], y[0, 2], y[0, 3] = 1.0, 2.0 ** -24, -1.0, 2.0 ** -24
+    # torch order: (1 + -1) + (2^-24 + 2^-24) = 2^-23 ; left-to-right: ((1+2^-24)+-1)+2^-24 = 2^-24
+    assert orc.cross_merge(y).item() == 2.0 ** -23
+    assert orc.cross_merge(y, order=1).item() == 2.0 ** -24
+    # bf16: each pairwise sum is rounded to bf16
+    yb = torch.zeros(1, 4, 1, 1, 1, dtype=torch.bfloat16)
+    yb[0, 0], yb[0, 1], yb[0, 2], yb[0, 3] = 1.0, 2.0 ** -9, -1.0, 2.0 ** -9
+    assert orc.cross_merge(yb).item() == 2.0 ** -8
+    assert orc.cross_merge(yb, order=1).item() == 2.0 ** -9
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 3, 5), (2, 4, 14, 14), (1, 2, 57, 58)])
+def test_merge_of_scan_is_four_x_and_adjoint(shape):
+    B, C, H, W = shape
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(shape, generator=g)
+    for order in (0, 1):
+        assert torch.equal(orc.cross_merge(orc.cross_scan(x).view(B, 4, C, H, W), order=order).view(shape), 4 * x)
+    # <scan(x), y> == <x, merge(y)> (how the reference defines the backward, csm_triton.py:208-225)
+    xi = torch.randint(-8, 8, shape, generator=g).float()
+    yi = torch.randint(-8, 8, (B, 4, C, H, W), generator=g).float()
+    lhs = (orc.cross_scan(xi).view(-1) * yi.view(-1)).sum()
+    rhs = (xi.view(-1) * orc.cross_merge(yi).view(-1)).sum()
+    assert lhs == rhs
+
+
+# ------------------------------------------------------------ selective scan
+def _t(v, dtype=torch.float32):
+    return None if v is None else torch.tensor(v, dtype=dtype)
+
+
+def _case_tensors(case):
+    return dict(u=_t(case["u"]), delta=_t(case["delta"]), A=_t(case["A"]), B=_t(case["B"]), C=_t(case["C"]),
+                D=_t(case["D"]), delta_bias=_t(case["delta_bias"]), delta_softplus=case["delta_softplus"])
+
+
+@pytest.mark.parametrize("idx", range(5))
+def test_scan_golden_float64_vectors(scan_golden, idx):
+    case = scan_golden[idx]
+    kw = _case_tensors(case)
+    want = torch.tensor(case["out"], dtype=torch.float64)
+    wide = orc.selective_scan(**kw, wide=True)
+    assert torch.allclose(wide, want, rtol=1e-12, atol=1e-12)
+    got, xst = orc.selective_scan(**kw, return_x=True)
+    assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-5)
+    last = torch.tensor(case["last_state"], dtype=torch.float64)
+    assert torch.allclose(xst[:, :, -1, 1::2].double(), last, rtol=1e-4, atol=1e-5)
+    ref, h = torch_ref.selective_scan(**kw, return_last_state=True)
+    assert torch.allclose(ref.double(), want, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(h.double(), last, rtol=1e-4, atol=1e-5)
+
+
+def _rand_inputs(seed, batch, dim, G, N, L, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    # distributions of the reference's own test, test_selective_scan.py:414-444
+    A = -0.5 * torch.rand(dim, N, generator=g)
+    B = torch.randn(batch, G, N, L, generator=g).to(dtype)
+    C = torch.randn(batch, G, N, L, generator=g).to(dtype)
+    D = torch.randn(dim, generator=g)
+    bias = 0.5 * torch.rand(dim, generator=g)
+    u = torch.randn(batch, dim, L, generator=g).to(dtype)
+    delta = (0.5 * torch.rand(batch, dim, L, generator=g)).to(dtype)
+    return u, delta, A, B, C, D, bias
+
+
+@pytest.mark.parametrize("N,L", [(1, 64), (1, 300), (8, 129), (16, 40)])
+@pytest.mark.parametrize("softplus", [False, True])
+def test_scan_c_oracle_vs_torch_restatement(N, L, softplus):
+    u, delta, A, B, C, D, bias = _rand_inputs(5, 2, 8, 2, N, L)
+    a = orc.selective_scan(u, delta, A, B, C, D, bias, softplus)
+    b = torch_ref.selective_scan(u, delta, A, B, C, D, bias, softplus)
+    assert torch.allclose(a, b, rtol=1e-5, atol=1e-5)
+    w = orc.selective_scan(u, delta, A, B, C, D, bias, softplus, wide=True)
+    assert torch.allclose(a.double(), w, rtol=1e-4, atol=1e-4)
+
+
+def test_scan_length_one_closed_form():
+    u, delta, A, B, C, D, bias = _rand_inputs(6, 3, 4, 2, 3, 1)
+    out = orc.selective_scan(u, delta, A, B, C, D, bias, True)
+    dl = torch.nn.functional.softplus(delta + bias[None, :, None])
+    Bf, Cf = B.repeat_interleave(2, 1), C.repeat_interleave(2, 1)
+    want = (Cf * Bf).sum(2) * dl * u + D[None, :, None] * u      # y = C.B dl u + D u
+    assert torch.allclose(out, want, rtol=1e-5, atol=1e-6)
+
+
+def test_scan_zero_A_is_cumsum():
+    u, delta, A, B, C, D, bias = _rand_inputs(7, 2, 4, 4, 1, 200)
+    out = orc.selective_scan(u, delta, torch.zeros_like(A), B, C, None, None, False)
+    h = torch.cumsum((delta * B[:, :, 0] * u).double(), dim=-1)
+    assert torch.allclose(out.double(), h * C[:, :, 0].double(), rtol=1e-4, atol=1e-4)
+
+
+def test_scan_geometric_series():
+    L, dl, Av = 500, 0.05, -0.7
+    one = torch.ones(1, 1, L)
+    out = orc.selective_scan(one, dl * one, torch.tensor([[Av]]), one.view(1, 1, 1, L), one.view(1, 1, 1, L))
+    a = math.exp(dl * Av)
+    want = torch.tensor([dl * (1 - a ** (t + 1)) / (1 - a) for t in range(L)], dtype=torch.float64)
+    assert torch.allclose(out.view(-1).double(), want, rtol=1e-4)
+
+
+def test_scan_zero_B_is_skip_path_and_output_dtype():
+    u, delta, A, B, C, D, bias = _rand_inputs(8, 2, 4, 2, 2, 50, dtype=torch.bfloat16)
+    out = orc.selective_scan(u, delta, A, torch.zeros_like(B), C, D, bias, True)
+    assert out.dtype == torch.float32 and torch.equal(out, u.float() * D[None, :, None])
+    out_in = orc.selective_scan(u, delta, A, torch.zeros_like(B), C, D, bias, True, out_float=False)
+    assert out_in.dtype == torch.bfloat16 and torch.equal(out_in, (u.float() * D[None, :, None]).bfloat16())
+
+
+def test_scan_softplus_threshold_and_bias():
+    # delta+bias > 20 passes through unchanged (fwd_kernel_oflex.cuh:126); softplus(0)=ln 2
+    one = torch.ones(1, 1, 1)
+    k = dict(A=torch.zeros(1, 1), B=one.view(1, 1, 1, 1), C=one.view(1, 1, 1, 1))
+    assert orc.selective_scan(one, 20.0 * one, delta_bias=torch.tensor([5.0]), delta_softplus=True, **k).item() == 25.0
+    got = orc.selective_scan(one, -3.0 * one, delta_bias=torch.tensor([3.0]), delta_softplus=True, **k).item()
+    assert abs(got - math.log(2.0)) < 1e-6
+    assert orc.selective_scan(one, -3.0 * one, delta_bias=torch.tensor([3.5]), delta_softplus=False, **k).item() == 0.5
+
+
+def test_scan_group_broadcast_uses_floor_division():
+    # channel d reads B[:, d // (dim/G)] (csms6s.py:53 == fwd_kernel_oflex.cuh:90)
+    batch, dim, G, L = 1, 6, 3, 5
+    u, dl = torch.ones(batch, dim, L), torch.ones(batch, dim, L)
+    B = torch.arange(1, G + 1).float().view(1, G, 1, 1).expand(1, G, 1, L).contiguous()
+    C = torch.ones(1, G, 1, L)
+    out = orc.selective_scan(u, dl, torch.zeros(dim, 1), B, C)
+    assert out[0, :, 0].tolist() == [1.0, 1.0, 2.0, 2.0, 3.0, 3.0]
+    # delta groups: delta (batch, 2, L) shared by dim/2 channels each (test_selective_scan.py:446-450)
+    dl2 = torch.tensor([1.0, 3.0]).view(1, 2, 1).expand(1, 2, L).contiguous()
+    out = orc.selective_scan(u, dl2, torch.zeros(dim, 1), torch.ones(1, 1, 1, L), torch.ones(1, 1, 1, L))
+    assert out[0, :, 0].tolist() == [1.0, 1.0, 1.0, 3.0, 3.0, 3.0]
+
+
+def test_scan_chunk_states_layout():
+    # x[b,d,c,2n] = running product of a since t=0, x[b,d,c,2n+1] = h at chunk end (chunks of 2048)
+    L = 2048 + 700
+    u, delta, A, B, C, D, bias = _rand_inputs(9, 1, 2, 1, 2, L)
+    out, xst = orc.selective_scan(u, delta, A, B, C, D, bias, True, return_x=True)
+    assert xst.shape == (1, 2, 2, 4)
+    _, h_end = torch_ref.selective_scan(u, delta, A, B, C, D, bias, True, return_last_state=True)
+    assert torch.allclose(xst[:, :, -1, 1::2], h_end, rtol=1e-4, atol=1e-5)
+    _, h_mid = torch_ref.selective_scan(u[..., :2048], delta[..., :2048], A, B[..., :2048], C[..., :2048], D, bias, True,
+                                        return_last_state=True)
+    assert torch.allclose(xst[:, :, 0, 1::2], h_mid, rtol=1e-4, atol=1e-5)
+    dl = torch.nn.functional.softplus(delta + bias[None, :, None]).double()
+    aprod = torch.exp((dl.sum(-1)[..., None] * A.double()[None]))
+    assert torch.allclose(xst[:, :, -1, 0::2].double(), aprod, rtol=1e-3, atol=1e-30)
+
+
+def test_scan_split_invariance():
+    # scanning [0,s) then [s,L) with the carried state equals one scan: the state after s steps is
+    # recovered from the outputs with C=1, N=1
+    L, s = 90, 37
+    u, delta, A, B, C, D, bias = _rand_inputs(10, 1, 3, 1, 1, L)
+    ones = torch.ones_like(C)
+    h = orc.selective_scan(u, delta, A, B, ones, None, bias, True)            # h_t itself
+    h2 = orc.selective_scan(u[..., s:], delta[..., s:], A, B[..., s:], ones[..., s:], None, bias, True)
+    dl = torch.nn.functional.softplus(delta + bias[None, :, None])
+    decay = torch.exp(torch.cumsum(dl[..., s:] * A[None, :, 0, None], -1))
+    assert torch.allclose(h[..., s:], h2 + decay * h[..., s - 1:s], rtol=1e-4, atol=1e-5)
