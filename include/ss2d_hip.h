@@ -1,0 +1,124 @@
+/*
+ * ss2d_hip.h -- C ABI of libss2d_hip.so: the SS2D inference hot path of VMamba
+ * (CrossScan -> selective-scan forward -> CrossMerge) as hand-written HIP
+ * kernels for gfx950 (MI355X).
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes, no framework types; every pointer is DEVICE memory
+ *     on the device that is current for the calling thread;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is
+ *     enqueued on it and the call returns without synchronising;
+ *   - nothing is allocated, freed or synchronised inside the library; outputs are
+ *     caller-allocated, inputs are only read;
+ *   - re-entrant: there is no global state, so concurrent calls on different
+ *     streams are independent;
+ *   - the return value is SS2D_OK or a negative SS2D_E* code (errno numbering); on
+ *     error nothing has been launched.  No exception crosses this boundary.
+ *
+ * Each entry point replaces one native piece of the reference (file:line are paths
+ * inside MzeroMiko/VMamba).
+ */
+#ifndef SS2D_HIP_H
+#define SS2D_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SS2D_ABI_VERSION 1
+
+/* element types */
+#define SS2D_F32 0
+#define SS2D_BF16 1
+#define SS2D_F16 2
+
+/* status codes */
+#define SS2D_OK 0
+#define SS2D_EINVAL (-22)  /* bad shape, stride, pointer or flag            */
+#define SS2D_ENOTSUP (-95) /* valid request this build has no kernel for    */
+#define SS2D_ELAUNCH (-5)  /* the HIP runtime refused the launch            */
+
+/* CrossMerge association orders */
+#define SS2D_MERGE_PAIRWISE 0      /* (y0 + flip y2) + T(y1 + flip y3): cross_merge_fwd,
+                                      classification/models/csm_triton.py:61-62           */
+#define SS2D_MERGE_LEFT_TO_RIGHT 1 /* ((y0 + T y1) + flip y2) + T flip y3: the Triton
+                                      kernel, classification/models/csm_triton.py:362-370 */
+
+/* Chunk length of the `x` (chunk-end state) output of the scan:
+ * kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:206 */
+#define SS2D_SCAN_CHUNK 2048
+
+int ss2d_abi_version(void);
+const char *ss2d_strerror(int code);
+
+/*
+ * CrossScan, scans=0, channel-first in and out, not one-by-one.
+ * Replaces the Triton launch CrossScanTritonF.forward
+ * (classification/models/csm_triton.py:405-433, kernel :278-361); semantics of
+ * cross_scan_fwd (csm_triton.py:22-29).
+ *   x (B,C,H,W) contiguous  ->  y (B,4,C,H*W) contiguous, same element size:
+ *   y[b,0,c,h*W+w] = y[b,1,c,w*H+h] = y[b,2,c,L-1-(h*W+w)] = y[b,3,c,L-1-(w*H+h)] = x[b,c,h,w]
+ * elem_bytes in {1,2,4,8}; a pure permutation, bit-exact for any payload.
+ * Empty tensors (any of B,C,H,W zero) are a no-op returning SS2D_OK.
+ */
+int ss2d_cross_scan(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, void *stream);
+
+/*
+ * CrossMerge, scans=0, channel-first in and out, not one-by-one.
+ * Replaces CrossMergeTritonF.forward (csm_triton.py:458-481, kernel :362-370);
+ * default semantics and rounding order of cross_merge_fwd (csm_triton.py:56-62).
+ *   ys (B,4,C,H,W) contiguous -> out (B,C,H*W) contiguous, dtype in {F32,BF16,F16};
+ *   every pairwise add is rounded to `dtype` (round-to-nearest-even), in the
+ *   association order selected by `order`.
+ */
+int ss2d_cross_merge(const void *ys, void *out, int B, int C, int H, int W, int dtype, int order,
+                     void *stream);
+
+/*
+ * Selective-scan forward ("oflex" flavour: output may be fp32 whatever the input).
+ * Replaces selective_scan_fwd + selective_scan_fwd_kernel
+ * (kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:143-231,
+ *  .../selective_scan_fwd_kernel_oflex.cuh:67-212); the struct mirrors SSMParamsBase
+ * (.../selective_scan_oflex.h:26-61).  Strides are in ELEMENTS; the innermost
+ * (sequence) stride of u, delta, B, C, out is 1.
+ *
+ *   u      (batch, dim, seqlen)              in_dtype
+ *   delta  (batch, delta_dim, seqlen)        in_dtype; dim % delta_dim == 0, channel d reads
+ *                                            row d / (dim/delta_dim)
+ *   A      (dim, dstate)                     fp32
+ *   B, C   (batch, n_groups, dstate, seqlen) in_dtype; dim % n_groups == 0, channel d reads
+ *                                            group d / (dim/n_groups)
+ *   D      (dim) fp32 or NULL;  delta_bias (delta_dim) fp32 or NULL
+ *   out    (batch, dim, seqlen)              out_dtype: SS2D_F32 or in_dtype
+ *   x      (batch, dim, n_chunks, 2*dstate)  fp32 contiguous or NULL (skip);
+ *          n_chunks = ceil(seqlen / SS2D_SCAN_CHUNK); x[..,2n] = product of a since t=0,
+ *          x[..,2n+1] = h_n, both at the end of the chunk (last state = x[:,:,-1,1::2])
+ *
+ *   dl = delta + delta_bias;  if delta_softplus: dl = dl > 20 ? dl : log1p(exp(dl))
+ *   h_n[t] = exp(dl*A[d,n]) * h_n[t-1] + dl*B[n,t]*u[t];   out[t] = sum_n C[n,t]*h_n[t] + D[d]*u[t]
+ * State and arithmetic are fp32.  dstate <= 256 (selective_scan_oflex.cpp:180).
+ */
+typedef struct ss2d_scan_params {
+    int32_t batch, dim, seqlen, dstate, n_groups, delta_dim;
+    int32_t in_dtype, out_dtype;
+    int32_t delta_softplus;
+    int32_t reserved;
+    const void *u, *delta, *A, *B, *C, *D, *delta_bias;
+    void *out;
+    void *x;
+    int64_t u_batch_stride, u_d_stride;
+    int64_t delta_batch_stride, delta_d_stride;
+    int64_t A_d_stride, A_dstate_stride;
+    int64_t B_batch_stride, B_group_stride, B_dstate_stride;
+    int64_t C_batch_stride, C_group_stride, C_dstate_stride;
+    int64_t out_batch_stride, out_d_stride;
+} ss2d_scan_params;
+
+int ss2d_selective_scan_fwd(const ss2d_scan_params *params, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SS2D_HIP_H */

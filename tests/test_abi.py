@@ -1,0 +1,93 @@
+"""CPU-only checks of the C ABI: the library loads, exports what include/ss2d_hip.h declares,
+and validates arguments before touching the GPU (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from vmamba_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "ss2d_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ss2d_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS), names
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_version_and_strerror():
+    assert _lib.lib().ss2d_abi_version() == _lib.ABI_VERSION
+    text = open(os.path.join(ROOT, "include", "ss2d_hip.h")).read()
+    assert f"#define SS2D_ABI_VERSION {_lib.ABI_VERSION}" in text
+    assert _lib.strerror(0) == "ok"
+    assert "invalid" in _lib.strerror(_lib.SS2D_EINVAL)
+    assert "unknown" in _lib.strerror(12345)
+
+
+def test_struct_layout_matches_header():
+    # 10 int32 + 9 pointers + 14 int64, no padding surprises
+    assert ctypes.sizeof(_lib.ScanParams) == 10 * 4 + 9 * 8 + 14 * 8
+    assert _lib.ScanParams.u.offset == 40 and _lib.ScanParams.u_batch_stride.offset == 40 + 72
+
+
+def test_cross_scan_argument_validation():
+    L = _lib.lib()
+    assert L.ss2d_cross_scan(None, None, 0, 3, 4, 4, 4, None) == _lib.SS2D_OK          # empty: no-op
+    assert L.ss2d_cross_scan(None, None, 2, 3, 0, 4, 2, None) == _lib.SS2D_OK
+    assert L.ss2d_cross_scan(None, None, 1, 1, 1, 1, 4, None) == _lib.SS2D_EINVAL      # null pointers
+    assert L.ss2d_cross_scan(None, None, 1, 1, 1, 1, 3, None) == _lib.SS2D_EINVAL      # element size
+    assert L.ss2d_cross_scan(None, None, -1, 1, 1, 1, 4, None) == _lib.SS2D_EINVAL
+
+
+def test_cross_merge_argument_validation():
+    L = _lib.lib()
+    assert L.ss2d_cross_merge(None, None, 0, 3, 4, 4, _lib.SS2D_F32, 0, None) == _lib.SS2D_OK
+    assert L.ss2d_cross_merge(None, None, 1, 1, 1, 1, _lib.SS2D_F32, 0, None) == _lib.SS2D_EINVAL
+    assert L.ss2d_cross_merge(None, None, 1, 1, 1, 1, 7, 0, None) == _lib.SS2D_EINVAL   # dtype
+    assert L.ss2d_cross_merge(None, None, 1, 1, 1, 1, _lib.SS2D_F32, 2, None) == _lib.SS2D_EINVAL  # order
+
+
+def test_scan_argument_validation():
+    L = _lib.lib()
+    assert L.ss2d_selective_scan_fwd(None, None) == _lib.SS2D_EINVAL
+    p = _lib.ScanParams()
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups, p.delta_dim = 0, 8, 16, 1, 4, 8
+    p.in_dtype, p.out_dtype = _lib.SS2D_BF16, _lib.SS2D_F32
+    assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_OK               # empty batch
+    p.batch = 2
+    assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_EINVAL           # null pointers
+    p.dstate = 257
+    assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_EINVAL           # dstate > 256
+    p.dstate, p.n_groups = 1, 3
+    assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_EINVAL           # dim % n_groups
+    p.n_groups, p.out_dtype = 4, _lib.SS2D_F16
+    assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_EINVAL           # out dtype neither f32 nor input
+
+
+def test_host_api_rejects_cpu_tensors_and_unsupported_modes():
+    import torch
+    import vmamba_amd as va
+    x = torch.zeros(1, 2, 3, 3)
+    with pytest.raises(NotImplementedError):
+        va.cross_scan_fn(x)
+    with pytest.raises(NotImplementedError):
+        va.cross_merge_fn(torch.zeros(1, 4, 2, 3, 3))
+    with pytest.raises(NotImplementedError):
+        va.cross_scan_fn(x, scans=1)
+    with pytest.raises(NotImplementedError):
+        va.cross_scan_fn(x, force_torch=True)
+    u = torch.zeros(1, 4, 8)
+    with pytest.raises(RuntimeError):
+        va.selective_scan_fn(u, u, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8))
+    with pytest.raises(NotImplementedError):
+        va.selective_scan_fn(u, u, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8), backend="torch")

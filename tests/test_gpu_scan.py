@@ -1,0 +1,217 @@
+"""GPU parity of the selective-scan forward against the CPU oracle (selective_scan_ref semantics).
+
+Tolerances: fp32 output (fp32 or exact-widened 16-bit inputs): rtol 1e-3, atol 1e-4 -- the
+north-star bound "1e-3 relative in fp32"; 16-bit output: rtol 2e-2, atol 2e-2.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import ss2d_oracle as orc
+import vmamba_amd as va
+from vmamba_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL32 = dict(rtol=1e-3, atol=1e-4)
+TOL16 = dict(rtol=2e-2, atol=2e-2)
+
+
+def _announce(*what):
+    print("CASE", *what, flush=True)
+
+
+def make_inputs(seed, batch, dim, G, N, L, dtype, delta_dim=None, ss2d_like=False):
+    g = torch.Generator().manual_seed(seed)
+    delta_dim = dim if delta_dim is None else delta_dim
+    if ss2d_like:
+        # BASELINE config 0 recipe: dt log-uniform in [1e-3, 0.1], bias = inverse softplus, A = -(1..N)
+        dt = torch.exp(torch.rand(delta_dim, generator=g) * (torch.log(torch.tensor(0.1)) - torch.log(torch.tensor(1e-3)))
+                       + torch.log(torch.tensor(1e-3)))
+        bias = dt + torch.log(-torch.expm1(-dt))
+        A = -torch.arange(1, N + 1, dtype=torch.float32).repeat(dim, 1)
+        delta = torch.randn(batch, delta_dim, L, generator=g)
+        D = torch.ones(dim)
+    else:
+        # the reference's own test distributions, test_selective_scan.py:414-444
+        A = -0.5 * torch.rand(dim, N, generator=g)
+        bias = 0.5 * torch.rand(delta_dim, generator=g)
+        delta = 0.5 * torch.rand(batch, delta_dim, L, generator=g)
+        D = torch.randn(dim, generator=g)
+    B = torch.randn(batch, G, N, L, generator=g)
+    C = torch.randn(batch, G, N, L, generator=g)
+    u = torch.randn(batch, dim, L, generator=g)
+    return u.to(dtype), delta.to(dtype), A, B.to(dtype), C.to(dtype), D, bias
+
+
+def run_gpu(u, delta, A, B, C, D, bias, softplus, out_float=True):
+    dev = lambda t: None if t is None else t.to(DEV)
+    out, x = va.selective_scan_fwd(dev(u), dev(delta), dev(A), dev(B), dev(C), dev(D), dev(bias), softplus, 1, out_float)
+    torch.cuda.synchronize()
+    return out.cpu(), x.cpu()
+
+
+def check(u, delta, A, B, C, D, bias, softplus, out_float=True):
+    want, xw = orc.selective_scan(u, delta, A, B, C, D, bias, softplus, out_float=out_float, return_x=True)
+    got, xg = run_gpu(u, delta, A, B, C, D, bias, softplus, out_float)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    tol = TOL32 if out_float or u.dtype == torch.float32 else TOL16
+    err = (got.float() - want.float()).abs().max().item()
+    assert torch.allclose(got.float(), want.float(), **tol), f"max abs err {err}"
+    assert torch.allclose(xg[..., 1::2], xw[..., 1::2], **TOL32), "chunk-end states"
+    assert torch.allclose(xg[..., 0::2], xw[..., 0::2], rtol=1e-3, atol=1e-30), "chunk-end decay products"
+
+
+@pytest.fixture(scope="module")
+def scan_golden(golden_dir):
+    with open(os.path.join(golden_dir, "selective_scan_f64.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("idx", range(5))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_golden_float64_vectors(scan_golden, idx, dtype):
+    case = scan_golden[idx]
+    _announce("golden", idx, dtype)
+    t = lambda v, dt=torch.float32: None if v is None else torch.tensor(v, dtype=dt)
+    got, x = run_gpu(t(case["u"], dtype), t(case["delta"], dtype), t(case["A"]), t(case["B"], dtype), t(case["C"], dtype),
+                     t(case["D"]), t(case["delta_bias"]), case["delta_softplus"])
+    want = torch.tensor(case["out"], dtype=torch.float64)
+    assert torch.allclose(got.double(), want, **TOL32)
+    assert torch.allclose(x[:, :, -1, 1::2].double(), torch.tensor(case["last_state"], dtype=torch.float64), **TOL32)
+
+
+# batch, dim, G, N, L
+GRID = [
+    (2, 8, 4, 1, 1), (2, 8, 4, 1, 7), (2, 16, 4, 1, 49), (2, 8, 4, 1, 64), (2, 16, 4, 1, 196), (1, 8, 2, 1, 512),
+    (2, 8, 4, 1, 784), (1, 8, 4, 1, 1000), (1, 8, 4, 1, 2048), (1, 4, 4, 1, 2049), (2, 12, 4, 1, 3136),
+    (1, 4, 2, 1, 4097), (1, 4, 1, 1, 9000),
+    (1, 8, 4, 16, 49), (1, 8, 4, 16, 520), (1, 4, 2, 16, 3136), (2, 6, 2, 2, 100), (1, 6, 3, 5, 777), (1, 4, 1, 8, 2500),
+    (1, 2, 1, 64, 300),
+]
+
+
+@pytest.mark.parametrize("batch,dim,G,N,L", GRID)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_scan_matches_oracle(batch, dim, G, N, L, dtype):
+    _announce("scan", batch, dim, G, N, L, dtype)
+    check(*make_inputs(21, batch, dim, G, N, L, dtype), True)
+
+
+@pytest.mark.parametrize("batch,dim,G,N,L", [(2, 8, 4, 1, 3136), (1, 8, 4, 16, 784), (2, 16, 4, 1, 49), (1, 4, 4, 1, 333)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_scan_ss2d_init_recipe(batch, dim, G, N, L, dtype):
+    _announce("scan-ss2d", batch, dim, G, N, L, dtype)
+    check(*make_inputs(22, batch, dim, G, N, L, dtype, ss2d_like=True), True)
+
+
+@pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False), (True, True, False)])
+@pytest.mark.parametrize("L", [130, 2304])
+def test_scan_optional_arguments(has_D, has_bias, softplus, L):
+    _announce("scan-opt", has_D, has_bias, softplus, L)
+    u, delta, A, B, C, D, bias = make_inputs(23, 2, 8, 2, 1, L, torch.float32)
+    check(u, delta, A, B, C, D if has_D else None, bias if has_bias else None, softplus)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L", [49, 3136])
+def test_scan_output_in_input_dtype(dtype, L):
+    _announce("scan-out16", dtype, L)
+    check(*make_inputs(24, 2, 8, 4, 1, L, dtype), True, out_float=False)
+
+
+@pytest.mark.parametrize("L", [64, 2560])
+def test_scan_delta_group_broadcast(L):
+    # delta (batch, dim1, L) shared by dim/dim1 channels, test_selective_scan.py:392, 446-450
+    _announce("scan-deltagroup", L)
+    check(*make_inputs(25, 2, 24, 2, 1, L, torch.float32, delta_dim=6), True)
+
+
+def test_scan_many_rows_long_sequence_uses_one_wave_per_row():
+    # >= 16384 rows with L > 2048: the unsplit kernel carries state across 2048-chunks in registers
+    _announce("scan-manyrows")
+    check(*make_inputs(26, 4, 4096, 4, 1, 2560, torch.bfloat16), True)
+
+
+def test_scan_strided_views_of_the_projection():
+    """B, C and delta handed over as views into one x_dbl buffer (no .contiguous()), as the SS2D
+    core could do with the output of x_proj (vmamba.py:606)."""
+    _announce("scan-strided")
+    batch, K, Dn, N, R, L = 2, 4, 6, 2, 3, 392
+    g = torch.Generator().manual_seed(27)
+    x_dbl = torch.randn(batch, K, R + 2 * N, L, generator=g)
+    dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
+    big = torch.randn(batch, K * Dn + 5, L, generator=g) * 0.5
+    u_view, delta_view = big[:, 2:2 + K * Dn], (big * 0.3)[:, 5:]
+    A = -0.5 * torch.rand(K * Dn, N, generator=g)
+    want = orc.selective_scan(u_view, delta_view, A, Bs, Cs, None, None, True)
+    xd = x_dbl.to(DEV)
+    _, Bd, Cd = torch.split(xd, [R, N, N], dim=2)
+    bigd = big.to(DEV)
+    dview = (bigd * 0.3)[:, 5:]
+    assert not Bd.is_contiguous() and not bigd[:, 2:2 + K * Dn].is_contiguous()
+    got = va.selective_scan_fn(bigd[:, 2:2 + K * Dn], dview, A.to(DEV), Bd, Cd, None, None, True)
+    assert torch.allclose(got.cpu(), want, **TOL32)
+
+
+def test_scan_softplus_threshold_and_extremes():
+    _announce("scan-softplus")
+    L = 64
+    delta = torch.linspace(-30.0, 30.0, L).view(1, 1, L).repeat(1, 2, 1)
+    u = torch.ones(1, 2, L)
+    A = torch.zeros(2, 1)
+    one = torch.ones(1, 1, 1, L)
+    # with A=0, B=C=1, u=1, D=None the output is cumsum(softplus(delta))
+    got, _ = run_gpu(u, delta, A, one, one, None, None, True)
+    want = torch.cumsum(torch.nn.functional.softplus(delta.double()), -1)
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-7)
+    inc = got[0, 0, 1:] - got[0, 0, :-1]
+    assert torch.allclose(inc[-10:].double(), delta[0, 0, -10:].double(), rtol=1e-5)  # > 20: identity
+
+
+def test_scan_errors_from_host_api():
+    u = torch.zeros(1, 4, 8, device=DEV)
+    A = torch.zeros(4, 1, device=DEV)
+    Bm = torch.zeros(1, 4, 1, 8, device=DEV)
+    with pytest.raises(RuntimeError):
+        va.selective_scan_fn(u, u.double(), A, Bm, Bm)                  # dtype mismatch
+    with pytest.raises(RuntimeError):
+        va.selective_scan_fn(u, u, A, torch.zeros(1, 3, 1, 8, device=DEV), Bm)   # dim % n_groups
+    with pytest.raises(RuntimeError):
+        va.selective_scan_fn(u, u, A.half(), Bm, Bm)                    # A must be fp32
+    with pytest.raises(RuntimeError):
+        va.selective_scan_fn(u.transpose(1, 2).contiguous().transpose(1, 2), u, A, Bm, Bm)  # last stride != 1
+    assert va.selective_scan_fn(u[:0], u[:0], A, Bm[:0], Bm[:0]).shape == (0, 4, 8)
+    out = va.selective_scan_fn(u.requires_grad_(), u, A, Bm, Bm)
+    with pytest.raises(NotImplementedError):
+        out.sum().backward()
+
+
+@pytest.mark.parametrize("cfg", ["stage1", "stage3", "stage4", "n16"])
+def test_full_size_properties(cfg):
+    """BASELINE configs at full size: exact scaling linearity in u, exact skip path with B=0, and a
+    slice of rows against the oracle."""
+    _announce("scan-full", cfg)
+    batch, Dn, L, N = dict(stage1=(128, 96, 3136, 1), stage3=(128, 384, 196, 1), stage4=(128, 768, 49, 1),
+                           n16=(16, 192, 3136, 16))[cfg]
+    K = 4
+    g = torch.Generator(device=DEV).manual_seed(28)
+    rn = lambda *s: torch.randn(*s, generator=g, device=DEV)
+    u, delta = rn(batch, K * Dn, L).bfloat16(), (rn(batch, K * Dn, L) * 0.5 - 3.0).bfloat16()
+    Bm, Cm = rn(batch, K, N, L).bfloat16(), rn(batch, K, N, L).bfloat16()
+    A = -torch.arange(1, N + 1, device=DEV, dtype=torch.float32).repeat(K * Dn, 1)
+    D = torch.ones(K * Dn, device=DEV)
+    bias = torch.rand(K * Dn, generator=g, device=DEV) - 1.0
+    y = va.selective_scan_fn(u, delta, A, Bm, Cm, D, bias, True)
+    y2 = va.selective_scan_fn(u * 2, delta, A, Bm, Cm, D, bias, True)
+    assert torch.equal(y2, 2 * y)                       # power-of-two scaling commutes with every rounding
+    y0 = va.selective_scan_fn(u, delta, A, torch.zeros_like(Bm), Cm, D, bias, True)
+    assert torch.equal(y0, u.float() * D[None, :, None])
+    for b in (0, batch - 1):
+        rows = slice(Dn * 3 - 5, Dn * 3 + 4)             # straddles directions 2 and 3
+        want = orc.selective_scan(u[b:b + 1].cpu(), delta[b:b + 1].cpu(), A.cpu(), Bm[b:b + 1].cpu(), Cm[b:b + 1].cpu(),
+                                  D.cpu(), bias.cpu(), True)
+        assert torch.allclose(y[b:b + 1, rows].cpu(), want[:, rows], **TOL32)

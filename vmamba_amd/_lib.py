@@ -1,0 +1,72 @@
+"""ctypes binding of libss2d_hip.so (the C ABI declared in include/ss2d_hip.h).
+
+There is no CPU fallback: if the library has not been built, loading fails loudly.
+"""
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libss2d_hip.so")
+
+SS2D_F32, SS2D_BF16, SS2D_F16 = 0, 1, 2
+SS2D_OK, SS2D_EINVAL, SS2D_ENOTSUP, SS2D_ELAUNCH = 0, -22, -95, -5
+MERGE_PAIRWISE, MERGE_LEFT_TO_RIGHT = 0, 1
+SCAN_CHUNK = 2048
+ABI_VERSION = 1
+
+EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd")
+
+
+class ScanParams(ctypes.Structure):
+    """struct ss2d_scan_params (include/ss2d_hip.h)."""
+    _fields_ = (
+        [(n, ctypes.c_int32) for n in ("batch", "dim", "seqlen", "dstate", "n_groups", "delta_dim",
+                                       "in_dtype", "out_dtype", "delta_softplus", "reserved")]
+        + [(n, ctypes.c_void_p) for n in ("u", "delta", "A", "B", "C", "D", "delta_bias", "out", "x")]
+        + [(n, ctypes.c_int64) for n in ("u_batch_stride", "u_d_stride", "delta_batch_stride", "delta_d_stride",
+                                         "A_d_stride", "A_dstate_stride",
+                                         "B_batch_stride", "B_group_stride", "B_dstate_stride",
+                                         "C_batch_stride", "C_group_stride", "C_dstate_stride",
+                                         "out_batch_stride", "out_d_stride")]
+    )
+
+
+class Ss2dError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what}: {strerror(code)} (ss2d status {code})")
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build the HIP library first (python -m vmamba_amd.build). "
+                "vmamba_amd has no CPU or PyTorch fallback for its kernels.")
+        L = ctypes.CDLL(LIB_PATH)
+        L.ss2d_abi_version.restype = ctypes.c_int
+        L.ss2d_strerror.restype = ctypes.c_char_p
+        L.ss2d_strerror.argtypes = [ctypes.c_int]
+        L.ss2d_cross_scan.restype = ctypes.c_int
+        L.ss2d_cross_scan.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+        L.ss2d_cross_merge.restype = ctypes.c_int
+        L.ss2d_cross_merge.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 6 + [ctypes.c_void_p]
+        L.ss2d_selective_scan_fwd.restype = ctypes.c_int
+        L.ss2d_selective_scan_fwd.argtypes = [ctypes.POINTER(ScanParams), ctypes.c_void_p]
+        if L.ss2d_abi_version() != ABI_VERSION:
+            raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
+        _lib = L
+    return _lib
+
+
+def strerror(code):
+    return lib().ss2d_strerror(int(code)).decode()
+
+
+def check(code, what):
+    if code != SS2D_OK:
+        raise Ss2dError(code, what)

@@ -1,0 +1,102 @@
+"""Selective-scan operator API, mirroring classification/models/csms6s.py:71-126.
+
+``selective_scan_fn(u, delta, A, B, C, D, delta_bias, delta_softplus, oflex, backend)`` keeps
+the reference's positional signature.  The forward runs the HIP scan in libss2d_hip.so; there
+is no torch or CPU implementation here, so ``backend="torch"`` and CPU tensors raise.  The
+argument checks are those of selective_scan_fwd
+(kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:152-204) and fail
+with RuntimeError as the reference's TORCH_CHECKs do.
+"""
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.SS2D_F32, torch.bfloat16: _lib.SS2D_BF16, torch.float16: _lib.SS2D_F16}
+MAX_DSTATE = 256
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def selective_scan_fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, nrows=1, out_float=True,
+                       want_x=True):
+    """Python twin of ``selective_scan_cuda_oflex.fwd``: returns [out, x].
+
+    out (batch, dim, L) is fp32 when ``out_float`` else u.dtype; x (batch, dim, n_chunks, 2N)
+    holds the chunk-end states (None when ``want_x`` is False).  ``nrows`` is accepted and
+    ignored, as in the reference (selective_scan_oflex.cpp:224-226).
+    """
+    _check(u.dtype in _DTYPE_CODE, f"selective_scan_fwd not implemented for input type '{u.dtype}'")
+    _check(A.dtype == torch.float32, "A must be float32")
+    _check(delta.dtype == u.dtype and B.dtype == u.dtype and C.dtype == u.dtype, "delta, B, C must have u's dtype")
+    for name, t in (("u", u), ("delta", delta), ("A", A), ("B", B), ("C", C)):
+        _check(t.is_cuda, f"{name} must be a GPU tensor: vmamba_amd has no CPU path")
+    _check(u.dim() == 3 and delta.dim() == 3 and A.dim() == 2 and B.dim() == 4 and C.dim() == 4, "bad tensor ranks")
+    _check(u.stride(-1) == 1 or u.size(-1) == 1, "u must be contiguous in its last dimension")
+    _check(delta.stride(-1) == 1 or delta.size(-1) == 1, "delta must be contiguous in its last dimension")
+    batch, dim, seqlen = u.shape
+    dstate, n_groups, delta_dim = A.size(1), B.size(1), delta.size(1)
+    _check(dim % n_groups == 0, "dims should be dividable by n_groups")
+    _check(dim % delta_dim == 0, "dims should be dividable by delta_dim")
+    _check(dstate <= MAX_DSTATE, "selective_scan only supports state dimension <= 256")
+    _check(tuple(delta.shape) == (batch, delta_dim, seqlen), "delta must have shape (batch_size, delta_dim, seqlen)")
+    _check(tuple(A.shape) == (dim, dstate), "A must have shape (dim, dstate)")
+    _check(tuple(B.shape) == (batch, n_groups, dstate, seqlen), "B must have shape (batch_size, n_groups, dstate, seqlen)")
+    _check(tuple(C.shape) == (batch, n_groups, dstate, seqlen), "C must have shape (batch_size, n_groups, dstate, seqlen)")
+    _check(B.stride(-1) == 1 or B.size(-1) == 1, "B must be contiguous in its last dimension")
+    _check(C.stride(-1) == 1 or C.size(-1) == 1, "C must be contiguous in its last dimension")
+    if D is not None:
+        _check(D.dtype == torch.float32 and D.is_cuda, "D must be a float32 GPU tensor")
+        _check(tuple(D.shape) == (dim,), "D must have shape (dim)")
+        D = D.contiguous()
+    if delta_bias is not None:
+        _check(delta_bias.dtype == torch.float32 and delta_bias.is_cuda, "delta_bias must be a float32 GPU tensor")
+        _check(tuple(delta_bias.shape) == (delta_dim,), "delta_bias must have shape (delta_dim)")
+        delta_bias = delta_bias.contiguous()
+
+    n_chunks = (seqlen + _lib.SCAN_CHUNK - 1) // _lib.SCAN_CHUNK
+    out = torch.empty((batch, dim, seqlen), device=u.device, dtype=torch.float32 if out_float else u.dtype)
+    x = torch.empty((batch, dim, n_chunks, dstate * 2), device=u.device, dtype=torch.float32) if want_x else None
+
+    p = _lib.ScanParams()
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups, p.delta_dim = batch, dim, seqlen, dstate, n_groups, delta_dim
+    p.in_dtype, p.out_dtype = _DTYPE_CODE[u.dtype], _DTYPE_CODE[out.dtype]
+    p.delta_softplus = int(bool(delta_softplus))
+    p.u, p.delta, p.A, p.B, p.C = u.data_ptr(), delta.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
+    p.D = D.data_ptr() if D is not None else None
+    p.delta_bias = delta_bias.data_ptr() if delta_bias is not None else None
+    p.out = out.data_ptr()
+    p.x = x.data_ptr() if x is not None else None
+    p.u_batch_stride, p.u_d_stride = u.stride(0), u.stride(1)
+    p.delta_batch_stride, p.delta_d_stride = delta.stride(0), delta.stride(1)
+    p.A_d_stride, p.A_dstate_stride = A.stride(0), A.stride(1)
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = B.stride(0), B.stride(1), B.stride(2)
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = C.stride(0), C.stride(1), C.stride(2)
+    p.out_batch_stride, p.out_d_stride = out.stride(0), out.stride(1)
+    with torch.cuda.device(u.device):
+        rc = _lib.lib().ss2d_selective_scan_fwd(p, torch.cuda.current_stream(u.device).cuda_stream)
+    _lib.check(rc, "ss2d_selective_scan_fwd")
+    return [out, x]
+
+
+class SelectiveScanHip(torch.autograd.Function):
+    """Forward-only counterpart of SelectiveScanCuda (csms6s.py:71-109)."""
+
+    @staticmethod
+    def forward(ctx, u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, oflex=True, backend=None):
+        needs_grad = any(isinstance(t, torch.Tensor) and t.requires_grad for t in (u, delta, A, B, C, D, delta_bias))
+        out, _ = selective_scan_fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, 1, oflex, want_x=needs_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        raise NotImplementedError("vmamba_amd implements the inference forward only; the selective-scan backward is not built")
+
+
+def selective_scan_fn(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=True, oflex=True, backend=None):
+    # u, delta: (B, K*C, L); A: (K*C, N); B, C: (B, K, N, L); D, delta_bias: (K*C)
+    if backend not in (None, "oflex"):
+        raise NotImplementedError(f"selective_scan_fn: backend={backend!r} is not available; this package ships the HIP 'oflex' forward only")
+    return SelectiveScanHip.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, oflex, backend)

@@ -1,0 +1,177 @@
+// CrossMerge (scans=0, channel-first): ys (B,4,C,L) -> out (B,C,L), the summing inverse of
+// CrossScan.  With r = h*W+w (row-major) and t = w*H+h (column-major):
+//   pairwise order:       out[r] = (y0[r] + y2[L-1-r]) + (y1[t] + y3[L-1-t])
+//   left-to-right order:  out[r] = ((y0[r] + y1[t]) + y2[L-1-r]) + y3[L-1-t]
+// Each add is rounded to the tensor dtype (fp32 adds are exact IEEE adds; bf16/f16 adds are
+// done in fp32 and rounded to nearest even), so the result is bit-identical to elementwise
+// torch arithmetic in the same order.
+//
+// HBM-bound: 4 reads + 1 write per element.  The column-major operands are read
+// lane-contiguously in THEIR order, combined, and transposed through LDS (odd pitch, so the
+// strided writes are conflict-free); the row-major operands and the output are then
+// lane-contiguous as well.  No strided global access anywhere.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+constexpr int kMTile = 64;
+constexpr int kMTilePitch = kMTile + 1;
+constexpr int kMergeLdsBytes = 32 * 1024;
+constexpr int kMergeTargetElems = 4096;
+
+template <typename T> __device__ __forceinline__ T add_rn(T a, T b) { return from_f32<T>(to_f32(a) + to_f32(b)); }
+
+template <typename T, int kOrder>
+__global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__restrict__ ys, T *__restrict__ out, int C,
+                                                                  int H, int W, int G, int groups_per_image,
+                                                                  FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *lds = reinterpret_cast<T *>(smem_raw);
+
+    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const uint32_t b = wg / (uint32_t)groups_per_image;
+    const uint32_t c0 = (wg - b * groups_per_image) * (uint32_t)G;
+    const uint32_t g = min((uint32_t)G, (uint32_t)C - c0);
+    const uint32_t L = divL.d;
+    const uint32_t n = g * L;
+    const uint32_t Lp = (uint32_t)H * (uint32_t)Wp;
+    const uint32_t lds_dir = (uint32_t)G * Lp;     // second LDS plane (left-to-right order only)
+
+    const size_t CL = (size_t)C * L;
+    const T *y0 = ys + ((size_t)b * 4 + 0) * CL + (size_t)c0 * L;
+    const T *y1 = y0 + CL;
+    const T *y2 = y1 + CL;
+    const T *y3 = y2 + CL;
+    T *o = out + ((size_t)b * C + c0) * L;
+
+    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
+        uint32_t m, t, h, w;
+        divmod(e, divL, m, t);
+        divmod(t, divH, w, h);
+        const T a = y1[e];
+        const T c = y3[m * L + (L - 1 - t)];
+        if (kOrder == SS2D_MERGE_PAIRWISE) {
+            lds[m * Lp + h * Wp + w] = add_rn(a, c);
+        } else {
+            lds[m * Lp + h * Wp + w] = a;
+            lds[lds_dir + m * Lp + h * Wp + w] = c;
+        }
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
+        uint32_t m, r, h, w;
+        divmod(e, divL, m, r);
+        divmod(r, divW, h, w);
+        const T a = y0[e];
+        const T c = y2[m * L + (L - 1 - r)];
+        const uint32_t li = m * Lp + h * Wp + w;
+        if (kOrder == SS2D_MERGE_PAIRWISE) {
+            o[e] = add_rn(add_rn(a, c), lds[li]);
+        } else {
+            o[e] = add_rn(add_rn(add_rn(a, lds[li]), c), lds[lds_dir + li]);
+        }
+    }
+}
+
+template <typename T, int kOrder>
+__global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__restrict__ ys, T *__restrict__ out, int C,
+                                                                  int H, int W, int tiles_h, int tiles_w) {
+    __shared__ T lds[(kOrder == SS2D_MERGE_PAIRWISE ? 1 : 2) * kMTile * kMTilePitch];
+    constexpr uint32_t kPlane = kMTile * kMTilePitch;
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    uint32_t wg = blockIdx.x;
+    const uint32_t tw = wg % tiles_w; wg /= tiles_w;
+    const uint32_t th = wg % tiles_h; wg /= tiles_h;
+    const uint32_t c = wg % C, b = wg / C;
+    const uint32_t h0 = th * kMTile, w0 = tw * kMTile;
+    const size_t L = (size_t)H * W, CL = (size_t)C * L;
+
+    const T *y0 = ys + ((size_t)b * 4 + 0) * CL + (size_t)c * L;
+    const T *y1 = y0 + CL;
+    const T *y2 = y1 + CL;
+    const T *y3 = y2 + CL;
+    T *o = out + ((size_t)b * C + c) * L;
+
+    for (uint32_t cc = wave; cc < kMTile; cc += kBlock / kWave) {
+        const uint32_t w = w0 + cc, h = h0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t t = (size_t)w * H + h;
+            const T a = y1[t];
+            const T d = y3[L - 1 - t];
+            if (kOrder == SS2D_MERGE_PAIRWISE) {
+                lds[lane * kMTilePitch + cc] = add_rn(a, d);
+            } else {
+                lds[lane * kMTilePitch + cc] = a;
+                lds[kPlane + lane * kMTilePitch + cc] = d;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t rr = wave; rr < kMTile; rr += kBlock / kWave) {
+        const uint32_t h = h0 + rr, w = w0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t r = (size_t)h * W + w;
+            const T a = y0[r];
+            const T d = y2[L - 1 - r];
+            const uint32_t li = rr * kMTilePitch + lane;
+            if (kOrder == SS2D_MERGE_PAIRWISE) {
+                o[r] = add_rn(add_rn(a, d), lds[li]);
+            } else {
+                o[r] = add_rn(add_rn(add_rn(a, lds[li]), d), lds[kPlane + li]);
+            }
+        }
+    }
+}
+
+template <typename T, int kOrder>
+static int launch_cross_merge(const void *ys, void *out, int B, int C, int H, int W, hipStream_t stream) {
+    const int64_t L = (int64_t)H * W;
+    const int Wp = W | 1;
+    const int planes = kOrder == SS2D_MERGE_PAIRWISE ? 1 : 2;
+    const int64_t map_lds = (int64_t)planes * H * Wp * (int64_t)sizeof(T);
+    if (map_lds <= kMergeLdsBytes) {
+        int G = (int)((kMergeTargetElems + L - 1) / L);
+        G = G < 1 ? 1 : G;
+        G = G > C ? C : G;
+        const int64_t cap = kMergeLdsBytes / map_lds;
+        G = G > cap ? (int)cap : G;
+        const int groups = (C + G - 1) / G;
+        const int64_t n_wg = (int64_t)B * groups;
+        if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+        hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder>), dim3((uint32_t)n_wg), dim3(kBlock),
+                           (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
+                           make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+    } else {
+        const int tiles_h = (H + kMTile - 1) / kMTile, tiles_w = (W + kMTile - 1) / kMTile;
+        const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;
+        if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+        hipLaunchKernelGGL((cross_merge_tile_kernel<T, kOrder>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                           (const T *)ys, (T *)out, C, H, W, tiles_h, tiles_w);
+    }
+    return launch_status();
+}
+
+template <typename T>
+static int dispatch_order(const void *ys, void *out, int B, int C, int H, int W, int order, hipStream_t s) {
+    return order == SS2D_MERGE_PAIRWISE ? launch_cross_merge<T, SS2D_MERGE_PAIRWISE>(ys, out, B, C, H, W, s)
+                                        : launch_cross_merge<T, SS2D_MERGE_LEFT_TO_RIGHT>(ys, out, B, C, H, W, s);
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_cross_merge(const void *ys, void *out, int B, int C, int H, int W, int dtype, int order,
+                                void *stream) {
+    using namespace ss2d;
+    if (B < 0 || C < 0 || H < 0 || W < 0) return SS2D_EINVAL;
+    if (order != SS2D_MERGE_PAIRWISE && order != SS2D_MERGE_LEFT_TO_RIGHT) return SS2D_EINVAL;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!ys || !out) return SS2D_EINVAL;
+    if ((int64_t)H * W > 0x3fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case SS2D_F32: return dispatch_order<float>(ys, out, B, C, H, W, order, s);
+        case SS2D_BF16: return dispatch_order<bf16_t>(ys, out, B, C, H, W, order, s);
+        default: return dispatch_order<f16_t>(ys, out, B, C, H, W, order, s);
+    }
+}

@@ -1,0 +1,146 @@
+// CrossScan (scans=0, channel-first): x (B,C,H,W) -> y (B,4,C,L), a pure permutation.
+//
+// HBM-bound: 1 read + 4 writes per element.  Directions 0/2 (row-major and its reversal) are
+// written straight from the loaded registers; directions 1/3 (column-major and its reversal)
+// go through an LDS transpose so that both the global read and the global writes are
+// lane-contiguous.  LDS rows are padded to an odd pitch so the strided side is conflict-free.
+//
+// Two shapes of workgroup:
+//   maps kernel  - small maps (<= kMapsLdsBytes): a workgroup takes G whole maps of one image;
+//                  7x7 .. 90x90 feature maps land here.
+//   tile kernel  - large maps: a workgroup takes one 64x64 tile of one map.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+constexpr int kTile = 64;
+constexpr int kTilePitch = kTile + 1;
+constexpr int kMapsLdsBytes = 32 * 1024;   // per-workgroup LDS budget of the maps kernel
+constexpr int kMapsTargetElems = 4096;     // elements a maps-workgroup aims to move per direction
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__restrict__ x, T *__restrict__ y, int C,
+                                                                 int H, int W, int G, int groups_per_image,
+                                                                 FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *lds = reinterpret_cast<T *>(smem_raw);
+
+    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const uint32_t b = wg / (uint32_t)groups_per_image;
+    const uint32_t c0 = (wg - b * groups_per_image) * (uint32_t)G;
+    const uint32_t g = min((uint32_t)G, (uint32_t)C - c0);
+    const uint32_t L = divL.d;
+    const uint32_t n = g * L;
+    const uint32_t Lp = (uint32_t)H * (uint32_t)Wp;
+
+    const size_t CL = (size_t)C * L;
+    const T *xin = x + ((size_t)b * C + c0) * L;
+    T *y0 = y + ((size_t)b * 4 + 0) * CL + (size_t)c0 * L;
+    T *y1 = y0 + CL;
+    T *y2 = y1 + CL;
+    T *y3 = y2 + CL;
+
+    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
+        uint32_t m, j, h, w;
+        divmod(e, divL, m, j);
+        divmod(j, divW, h, w);
+        const T v = xin[e];
+        lds[m * Lp + h * Wp + w] = v;
+        y0[e] = v;
+        y2[m * L + (L - 1 - j)] = v;
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
+        uint32_t m, t, h, w;
+        divmod(e, divL, m, t);
+        divmod(t, divH, w, h);          // t = w*H + h
+        const T v = lds[m * Lp + h * Wp + w];
+        y1[e] = v;
+        y3[m * L + (L - 1 - t)] = v;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cross_scan_tile_kernel(const T *__restrict__ x, T *__restrict__ y, int C,
+                                                                 int H, int W, int tiles_h, int tiles_w) {
+    __shared__ T lds[kTile * kTilePitch];
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    uint32_t wg = blockIdx.x;
+    const uint32_t tw = wg % tiles_w; wg /= tiles_w;
+    const uint32_t th = wg % tiles_h; wg /= tiles_h;
+    const uint32_t c = wg % C, b = wg / C;
+    const uint32_t h0 = th * kTile, w0 = tw * kTile;
+    const size_t L = (size_t)H * W, CL = (size_t)C * L;
+
+    const T *xm = x + ((size_t)b * C + c) * L;
+    T *y0 = y + ((size_t)b * 4 + 0) * CL + (size_t)c * L;
+    T *y1 = y0 + CL;
+    T *y2 = y1 + CL;
+    T *y3 = y2 + CL;
+
+    for (uint32_t rr = wave; rr < kTile; rr += kBlock / kWave) {
+        const uint32_t h = h0 + rr, w = w0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t r = (size_t)h * W + w;
+            const T v = xm[r];
+            lds[rr * kTilePitch + lane] = v;
+            y0[r] = v;
+            y2[L - 1 - r] = v;
+        }
+    }
+    __syncthreads();
+    for (uint32_t cc = wave; cc < kTile; cc += kBlock / kWave) {
+        const uint32_t w = w0 + cc, h = h0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t t = (size_t)w * H + h;
+            const T v = lds[lane * kTilePitch + cc];
+            y1[t] = v;
+            y3[L - 1 - t] = v;
+        }
+    }
+}
+
+template <typename T>
+static int launch_cross_scan(const void *x, void *y, int B, int C, int H, int W, hipStream_t stream) {
+    const int64_t L = (int64_t)H * W;
+    const int Wp = W | 1;
+    const int64_t map_lds = (int64_t)H * Wp * (int64_t)sizeof(T);
+    if (map_lds <= kMapsLdsBytes) {
+        int G = (int)((kMapsTargetElems + L - 1) / L);
+        G = G < 1 ? 1 : G;
+        G = G > C ? C : G;
+        const int64_t cap = kMapsLdsBytes / map_lds;
+        G = G > cap ? (int)cap : G;
+        const int groups = (C + G - 1) / G;
+        const int64_t n_wg = (int64_t)B * groups;
+        if (n_wg > 0x7fffffff || (int64_t)G * L > 0x7fffffff) return SS2D_ENOTSUP;
+        hipLaunchKernelGGL(cross_scan_maps_kernel<T>, dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds), stream,
+                           (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
+                           make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+    } else {
+        const int tiles_h = (H + kTile - 1) / kTile, tiles_w = (W + kTile - 1) / kTile;
+        const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;
+        if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+        hipLaunchKernelGGL(cross_scan_tile_kernel<T>, dim3((uint32_t)n_wg), dim3(kBlock), 0, stream, (const T *)x,
+                           (T *)y, C, H, W, tiles_h, tiles_w);
+    }
+    return launch_status();
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_cross_scan(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, void *stream) {
+    using namespace ss2d;
+    if (B < 0 || C < 0 || H < 0 || W < 0) return SS2D_EINVAL;
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return SS2D_EINVAL;
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    if ((int64_t)H * W > 0x3fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (elem_bytes) {
+        case 1: return launch_cross_scan<uint8_t>(x, y, B, C, H, W, s);
+        case 2: return launch_cross_scan<uint16_t>(x, y, B, C, H, W, s);
+        case 4: return launch_cross_scan<uint32_t>(x, y, B, C, H, W, s);
+        default: return launch_cross_scan<uint64_t>(x, y, B, C, H, W, s);
+    }
+}

@@ -1,0 +1,401 @@
+// Selective-scan forward for gfx950: a chunked linear-recurrence scan written for 64-lane
+// wavefronts.
+//
+//   dl_t  = softplus(delta_t + bias)                     (fused into the load)
+//   h_n,t = exp(dl_t A_n) h_n,t-1 + dl_t B_n,t u_t       (fp32 state)
+//   y_t   = sum_n C_n,t h_n,t + D u_t
+//
+// The recurrence is the scan of pairs (a,b) under (a1,b1) o (a0,b0) = (a1 a0, a1 b0 + b1).
+// A wavefront covers 512 consecutive positions per pass: every lane scans its 8 consecutive
+// items in registers, the 64 lane totals are scanned with DPP row shifts / row broadcasts (no
+// LDS, no barrier), and the running state is carried from pass to pass in a register.
+//
+//   row kernel   one wavefront per (batch, channel) row, 4 rows per workgroup.
+//   row4 kernel  long rows with few of them: the 4 wavefronts of a workgroup split each
+//                2048-position chunk of one row and exchange their totals through LDS.
+//
+// I/O is 16-byte vectors per lane whenever pointers, strides and the row length allow
+// (kVec); otherwise element-wise with bounds checks.  Positions past the end of a row are fed
+// as dl = 0, u = 0, i.e. the identity pair (1, 0), so the state at the end of the last pass is
+// the state at the last real position.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+constexpr int kItems = 8;                    // consecutive positions per lane per pass
+constexpr int kPass = kWave * kItems;        // 512 positions per wavefront pass
+constexpr int kWavesPerWg = kBlock / kWave;  // 4
+constexpr int kPassesPerChunk = SS2D_SCAN_CHUNK / kPass;  // 4
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct ScanArgs {
+    const void *u, *delta, *B, *C;
+    const float *A, *D, *bias;
+    void *out;
+    float *x;
+    int32_t batch, dim, L, N, dim_per_group, dim_per_delta, n_chunks, softplus;
+    int64_t u_bs, u_ds, dl_bs, dl_ds, A_ds, A_ns, B_bs, B_gs, B_ns, C_bs, C_gs, C_ns, o_bs, o_ds;
+    int32_t rows;
+};
+
+// ---- 8-wide loads / stores ------------------------------------------------------------
+template <typename T, bool kVec>
+__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems]) {
+    if constexpr (kVec) {
+        // the host guarantees 16-byte alignment and L % (16/sizeof(T)) == 0, so a vector is either
+        // entirely inside the row or entirely outside
+        if constexpr (sizeof(T) == 2) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (pos < L) raw = *reinterpret_cast<const uint4 *>(row + pos);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = to_f32(T{(uint16_t)(w[i] & 0xffffu)});
+                v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
+            }
+        } else {
+            float4 lo = make_float4(0, 0, 0, 0), hi = make_float4(0, 0, 0, 0);
+            if (pos < L) lo = *reinterpret_cast<const float4 *>(row + pos);
+            if (pos + 4 < L) hi = *reinterpret_cast<const float4 *>(row + pos + 4);
+            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+            v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) v[i] = (pos + i < L) ? to_f32(row[pos + i]) : 0.0f;
+    }
+}
+
+template <typename T, bool kVec>
+__device__ __forceinline__ void store_items(T *__restrict__ row, int pos, int L, const float (&v)[kItems]) {
+    if constexpr (kVec) {
+        if constexpr (sizeof(T) == 2) {
+            if (pos < L) {
+                uint32_t w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    w[i] = (uint32_t)from_f32<T>(v[2 * i]).bits | ((uint32_t)from_f32<T>(v[2 * i + 1]).bits << 16);
+                *reinterpret_cast<uint4 *>(row + pos) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        } else {
+            if (pos < L) *reinterpret_cast<float4 *>(row + pos) = make_float4(v[0], v[1], v[2], v[3]);
+            if (pos + 4 < L) *reinterpret_cast<float4 *>(row + pos + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kItems; ++i)
+            if (pos + i < L) row[pos + i] = from_f32<T>(v[i]);
+    }
+}
+
+// softplus(x) = log1p(exp(x)) with two hardware transcendentals; for small exp(x) the series
+// t - t^2/2 + t^3/3 replaces log(1+t), whose rounding of 1+t would otherwise dominate.
+__device__ __forceinline__ float softplus_f32(float x) {
+    const float t = __builtin_amdgcn_exp2f(fminf(x, 20.0f) * kLog2e);
+    const float series = t * (1.0f - t * (0.5f - t * 0.33333334f));
+    const float full = kLn2 * __builtin_amdgcn_logf(1.0f + t);
+    const float sp = t < 0.015625f ? series : full;
+    return x > 20.0f ? x : sp;
+}
+
+// Inclusive scan of (a,h) over the 64 lanes; returns this lane's EXCLUSIVE prefix in
+// (a_ex,h_ex) and the wave total, uniform, in (a_tot,h_tot).
+__device__ __forceinline__ void wave_scan_pairs(float a, float h, float &a_ex, float &h_ex, float &a_tot,
+                                                float &h_tot) {
+#define SS2D_SCAN_STEP(CTRL, MASK)                        \
+    {                                                     \
+        const float ap = dpp_move<CTRL, MASK>(1.0f, a);   \
+        const float hp = dpp_move<CTRL, MASK>(0.0f, h);   \
+        h = fmaf(a, hp, h);                               \
+        a = a * ap;                                       \
+    }
+    SS2D_SCAN_STEP(kDppRowShr1, 0xF)
+    SS2D_SCAN_STEP(kDppRowShr2, 0xF)
+    SS2D_SCAN_STEP(kDppRowShr4, 0xF)
+    SS2D_SCAN_STEP(kDppRowShr8, 0xF)
+    SS2D_SCAN_STEP(kDppRowBcast15, 0xA)
+    SS2D_SCAN_STEP(kDppRowBcast31, 0xC)
+#undef SS2D_SCAN_STEP
+    a_ex = dpp_move<kDppWaveShr1>(1.0f, a);
+    h_ex = dpp_move<kDppWaveShr1>(0.0f, h);
+    a_tot = read_lane(a, kWave - 1);
+    h_tot = read_lane(h, kWave - 1);
+}
+
+// One state of one pass: lane-local scan of its 8 items, wave scan of the lane totals, then
+// the state entering the lane (from `carry`, the state entering the pass) is pushed through
+// the items and C*h is accumulated into y.  Returns the pass totals.
+__device__ __forceinline__ void scan_state_pass(const float (&dl)[kItems], const float (&du)[kItems],
+                                                const float (&Bv)[kItems], const float (&Cv)[kItems], float A_log2e,
+                                                float carry, float (&y)[kItems], float &a_tot, float &h_tot) {
+    float ac[kItems], hh[kItems];
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        const float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
+        const float b = Bv[i] * du[i];
+        ac[i] = i == 0 ? a : ac[i - 1] * a;
+        hh[i] = i == 0 ? b : fmaf(a, hh[i - 1], b);
+    }
+    float a_ex, h_ex;
+    wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+    const float s_in = fmaf(a_ex, carry, h_ex);
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
+}
+
+template <typename in_t, bool kVec>
+__device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_row, int pos, int L, float bias,
+                                             float Dv, bool softplus, float (&dl)[kItems], float (&du)[kItems],
+                                             float (&y)[kItems]) {
+    float uv[kItems];
+    load_items<in_t, kVec>(u_row, pos, L, uv);
+    load_items<in_t, kVec>(dl_row, pos, L, dl);
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        float d = dl[i] + bias;
+        if (softplus) d = softplus_f32(d);
+        d = (pos + i < L) ? d : 0.0f;     // identity pair past the end of the row (u is 0 there)
+        dl[i] = d;
+        du[i] = d * uv[i];
+        y[i] = Dv * uv[i];
+    }
+}
+
+// ---- one wavefront per row ------------------------------------------------------------
+// kN > 0: dstate known at compile time, states live in registers.
+// kN == 0: any dstate; the per-wave states live in LDS (2*dstate floats per wave).
+template <typename in_t, typename out_t, int kN, bool kVec>
+__global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
+    extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int row = (int)(wg * kWavesPerWg) + wave;
+    if (row >= p.rows) return;           // whole wavefront leaves; this kernel has no barrier
+
+    const int N = kN > 0 ? kN : p.N;
+    const int b = row / p.dim, d = row - b * p.dim;
+    const int grp = d / p.dim_per_group, dg = d / p.dim_per_delta;
+    const in_t *u_row = reinterpret_cast<const in_t *>(p.u) + b * p.u_bs + d * p.u_ds;
+    const in_t *dl_row = reinterpret_cast<const in_t *>(p.delta) + b * p.dl_bs + dg * p.dl_ds;
+    const in_t *B_row = reinterpret_cast<const in_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
+    const in_t *C_row = reinterpret_cast<const in_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+    out_t *o_row = reinterpret_cast<out_t *>(p.out) + b * p.o_bs + d * p.o_ds;
+    const float *A_row = p.A + d * p.A_ds;
+    float *x_row = p.x ? p.x + (size_t)row * p.n_chunks * 2 * N : nullptr;
+    const float Dv = p.D ? p.D[d] : 0.0f;
+    const float bias = p.bias ? p.bias[dg] : 0.0f;
+    const bool softplus = p.softplus != 0;
+    const int L = p.L;
+
+    float h_reg[kN > 0 ? kN : 1], ap_reg[kN > 0 ? kN : 1], A_reg[kN > 0 ? kN : 1];
+    float *st = dyn_state + (size_t)wave * 2 * N;
+    if constexpr (kN > 0) {
+#pragma unroll
+        for (int n = 0; n < kN; ++n) { h_reg[n] = 0.0f; ap_reg[n] = 1.0f; A_reg[n] = A_row[n * p.A_ns] * kLog2e; }
+    } else {
+        for (int n = lane; n < N; n += kWave) { st[2 * n] = 1.0f; st[2 * n + 1] = 0.0f; }
+    }
+
+    const int n_pass = (L + kPass - 1) / kPass;
+    for (int pass = 0; pass < n_pass; ++pass) {
+        const int pos = pass * kPass + lane * kItems;
+        float dl[kItems], du[kItems], y[kItems];
+        load_delta_u<in_t, kVec>(u_row, dl_row, pos, L, bias, Dv, softplus, dl, du, y);
+        const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || pass == n_pass - 1);
+        float *x_out = chunk_end ? x_row + (size_t)(pass / kPassesPerChunk) * 2 * N : nullptr;
+
+        if constexpr (kN > 0) {
+#pragma unroll
+            for (int n = 0; n < kN; ++n) {
+                float Bv[kItems], Cv[kItems], a_tot, h_tot;
+                load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+                load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                scan_state_pass(dl, du, Bv, Cv, A_reg[n], h_reg[n], y, a_tot, h_tot);
+                h_reg[n] = fmaf(a_tot, h_reg[n], h_tot);
+                ap_reg[n] *= a_tot;
+                if (chunk_end && lane == 0) { x_out[2 * n] = ap_reg[n]; x_out[2 * n + 1] = h_reg[n]; }
+            }
+        } else {
+            for (int n = 0; n < N; ++n) {
+                float Bv[kItems], Cv[kItems], a_tot, h_tot;
+                load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+                load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                const float ap = st[2 * n], h0 = st[2 * n + 1];
+                scan_state_pass(dl, du, Bv, Cv, A_row[n * p.A_ns] * kLog2e, h0, y, a_tot, h_tot);
+                const float h1 = fmaf(a_tot, h0, h_tot), ap1 = ap * a_tot;
+                if (lane == 0) {
+                    st[2 * n] = ap1; st[2 * n + 1] = h1;
+                    if (chunk_end) { x_out[2 * n] = ap1; x_out[2 * n + 1] = h1; }
+                }
+            }
+        }
+        store_items<out_t, kVec>(o_row, pos, L, y);
+    }
+}
+
+// ---- four wavefronts per row -------------------------------------------------------------
+// Workgroup = one row.  Per 2048-position chunk wave w takes positions [w*512, w*512+512).
+// LDS: agg[2][N][4] pass totals (double-buffered by chunk parity), state[2][N] chunk-start
+// state (running a-product, h).  One barrier per (chunk, state).
+template <typename in_t, typename out_t, bool kVec>
+__global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
+    extern __shared__ __align__(16) float smem[];
+    const int N = p.N;
+    float2 *agg = reinterpret_cast<float2 *>(smem);                  // [2][N][4]
+    float2 *state = agg + 2 * N * kWavesPerWg;                       // [2][N]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int row = (int)xcd_contiguous_id(blockIdx.x, gridDim.x);   // grid == rows exactly
+
+    const int b = row / p.dim, d = row - b * p.dim;
+    const int grp = d / p.dim_per_group, dg = d / p.dim_per_delta;
+    const in_t *u_row = reinterpret_cast<const in_t *>(p.u) + b * p.u_bs + d * p.u_ds;
+    const in_t *dl_row = reinterpret_cast<const in_t *>(p.delta) + b * p.dl_bs + dg * p.dl_ds;
+    const in_t *B_row = reinterpret_cast<const in_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
+    const in_t *C_row = reinterpret_cast<const in_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+    out_t *o_row = reinterpret_cast<out_t *>(p.out) + b * p.o_bs + d * p.o_ds;
+    const float *A_row = p.A + d * p.A_ds;
+    float *x_row = p.x ? p.x + (size_t)row * p.n_chunks * 2 * N : nullptr;
+    const float Dv = p.D ? p.D[d] : 0.0f;
+    const float bias = p.bias ? p.bias[dg] : 0.0f;
+    const bool softplus = p.softplus != 0;
+    const int L = p.L;
+
+    const int n_chunks = (L + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
+    for (int chunk = 0; chunk < n_chunks; ++chunk) {
+        const int par = chunk & 1;
+        const int pos = chunk * SS2D_SCAN_CHUNK + wave * kPass + lane * kItems;
+        float dl[kItems], du[kItems], y[kItems];
+        load_delta_u<in_t, kVec>(u_row, dl_row, pos, L, bias, Dv, softplus, dl, du, y);
+        for (int n = 0; n < N; ++n) {
+            float Bv[kItems], Cv[kItems];
+            load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+            load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+            const float A_log2e = A_row[n * p.A_ns] * kLog2e;
+            float ac[kItems], hh[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
+                const float bb = Bv[i] * du[i];
+                ac[i] = i == 0 ? a : ac[i - 1] * a;
+                hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
+            }
+            float a_ex, h_ex, a_tot, h_tot;
+            wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+            float2 *agg_n = agg + ((size_t)par * N + n) * kWavesPerWg;
+            if (lane == 0) agg_n[wave] = make_float2(a_tot, h_tot);
+            __syncthreads();
+            const float2 st = chunk == 0 ? make_float2(1.0f, 0.0f) : state[par * N + n];
+            float cin = st.y, aprod = st.x;
+#pragma unroll
+            for (int j = 0; j < kWavesPerWg; ++j) {
+                const float2 g = agg_n[j];
+                if (j < wave) cin = fmaf(g.x, cin, g.y);
+                aprod *= g.x;
+            }
+            const float s_in = fmaf(a_ex, cin, h_ex);
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
+            if (wave == kWavesPerWg - 1 && lane == 0) {
+                const float h_end = fmaf(a_tot, cin, h_tot);
+                state[(par ^ 1) * N + n] = make_float2(aprod, h_end);
+                if (x_row) {
+                    x_row[(size_t)chunk * 2 * N + 2 * n] = aprod;
+                    x_row[(size_t)chunk * 2 * N + 2 * n + 1] = h_end;
+                }
+            }
+        }
+        store_items<out_t, kVec>(o_row, pos, L, y);
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------
+static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+template <typename in_t, typename out_t, bool kVec>
+static int launch_scan(const ScanArgs &a, hipStream_t stream) {
+    // Few long rows: split every row over the 4 wavefronts of a workgroup.
+    const bool split_rows = a.L > SS2D_SCAN_CHUNK && a.rows < 16384;
+    if (split_rows) {
+        const size_t smem = (size_t)(2 * a.N * kWavesPerWg + 2 * a.N) * sizeof(float2);
+        hipLaunchKernelGGL((scan_row4_kernel<in_t, out_t, kVec>), dim3((uint32_t)a.rows), dim3(kBlock), smem, stream, a);
+        return launch_status();
+    }
+    const uint32_t n_wg = (uint32_t)((a.rows + kWavesPerWg - 1) / kWavesPerWg);
+    if (a.N == 1) {
+        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 1, kVec>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+    } else if (a.N == 16) {
+        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 16, kVec>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+    } else {
+        const size_t smem = (size_t)kWavesPerWg * 2 * a.N * sizeof(float);
+        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 0, kVec>), dim3(n_wg), dim3(kBlock), smem, stream, a);
+    }
+    return launch_status();
+}
+
+template <typename in_t, typename out_t>
+static int dispatch_vec(const ScanArgs &a, bool vec, hipStream_t stream) {
+    return vec ? launch_scan<in_t, out_t, true>(a, stream) : launch_scan<in_t, out_t, false>(a, stream);
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) {
+    using namespace ss2d;
+    if (!q) return SS2D_EINVAL;
+    if (q->batch < 0 || q->dim < 0 || q->seqlen < 0) return SS2D_EINVAL;
+    if (q->dstate <= 0 || q->dstate > 256 || q->n_groups <= 0 || q->delta_dim <= 0) return SS2D_EINVAL;
+    if (q->in_dtype != SS2D_F32 && q->in_dtype != SS2D_BF16 && q->in_dtype != SS2D_F16) return SS2D_EINVAL;
+    if (q->out_dtype != SS2D_F32 && q->out_dtype != q->in_dtype) return SS2D_EINVAL;
+    if (q->dim % q->n_groups != 0 || q->dim % q->delta_dim != 0) return SS2D_EINVAL;
+    if (q->batch == 0 || q->dim == 0 || q->seqlen == 0) return SS2D_OK;
+    if (!q->u || !q->delta || !q->A || !q->B || !q->C || !q->out) return SS2D_EINVAL;
+    if ((int64_t)q->batch * q->dim > 0x7fffffff - kWavesPerWg) return SS2D_ENOTSUP;
+
+    ScanArgs a;
+    a.u = q->u; a.delta = q->delta; a.B = q->B; a.C = q->C;
+    a.A = (const float *)q->A; a.D = (const float *)q->D; a.bias = (const float *)q->delta_bias;
+    a.out = q->out; a.x = (float *)q->x;
+    a.batch = q->batch; a.dim = q->dim; a.L = q->seqlen; a.N = q->dstate;
+    a.dim_per_group = q->dim / q->n_groups;
+    a.dim_per_delta = q->dim / q->delta_dim;
+    a.n_chunks = (q->seqlen + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
+    a.softplus = q->delta_softplus;
+    a.u_bs = q->u_batch_stride; a.u_ds = q->u_d_stride;
+    a.dl_bs = q->delta_batch_stride; a.dl_ds = q->delta_d_stride;
+    a.A_ds = q->A_d_stride; a.A_ns = q->A_dstate_stride;
+    a.B_bs = q->B_batch_stride; a.B_gs = q->B_group_stride; a.B_ns = q->B_dstate_stride;
+    a.C_bs = q->C_batch_stride; a.C_gs = q->C_group_stride; a.C_ns = q->C_dstate_stride;
+    a.o_bs = q->out_batch_stride; a.o_ds = q->out_d_stride;
+    a.rows = q->batch * q->dim;
+
+    // 16-byte vector I/O needs every row start and the row length on a 16-byte grid.
+    const int64_t in_vec = q->in_dtype == SS2D_F32 ? 4 : 8;
+    const int64_t out_vec = q->out_dtype == SS2D_F32 ? 4 : 8;
+    const int64_t in_strides[] = {a.u_bs, a.u_ds, a.dl_bs, a.dl_ds, a.B_bs, a.B_gs, a.B_ns, a.C_bs, a.C_gs, a.C_ns};
+    bool vec = aligned16(q->u) && aligned16(q->delta) && aligned16(q->B) && aligned16(q->C) && aligned16(q->out);
+    vec = vec && (q->seqlen % in_vec == 0) && (q->seqlen % out_vec == 0);
+    for (int64_t s : in_strides) vec = vec && (s % in_vec == 0);
+    vec = vec && (a.o_bs % out_vec == 0) && (a.o_ds % out_vec == 0);
+
+    hipStream_t s = (hipStream_t)stream;
+    if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, s);
+    if (q->in_dtype == SS2D_BF16) {
+        return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, s) : dispatch_vec<bf16_t, bf16_t>(a, vec, s);
+    }
+    return q->out_dtype == SS2D_F32 ? dispatch_vec<f16_t, float>(a, vec, s) : dispatch_vec<f16_t, f16_t>(a, vec, s);
+}
+
+extern "C" int ss2d_abi_version(void) { return SS2D_ABI_VERSION; }
+
+extern "C" const char *ss2d_strerror(int code) {
+    switch (code) {
+        case SS2D_OK: return "ok";
+        case SS2D_EINVAL: return "invalid argument (shape, stride, dtype, pointer or flag)";
+        case SS2D_ENOTSUP: return "request is valid but not supported by this build";
+        case SS2D_ELAUNCH: return "HIP runtime refused the kernel launch";
+        default: return "unknown ss2d status";
+    }
+}

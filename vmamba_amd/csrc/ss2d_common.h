@@ -1,0 +1,91 @@
+// Device-side helpers shared by the SS2D kernels (gfx950 / CDNA4, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ss2d_hip.h"
+
+namespace ss2d {
+
+constexpr int kWave = 64;       // CDNA wavefront
+constexpr int kBlock = 256;     // 4 waves per workgroup everywhere
+constexpr int kXcds = 8;        // MI355X: 8 XCDs, workgroups are dealt to them round-robin
+
+// ---- element types ----------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+template <typename T> struct ElemTraits;
+template <> struct ElemTraits<float> { static constexpr int dtype = SS2D_F32; };
+template <> struct ElemTraits<bf16_t> { static constexpr int dtype = SS2D_BF16; };
+template <> struct ElemTraits<f16_t> { static constexpr int dtype = SS2D_F16; };
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bits_to_f32(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float to_f32(f16_t v) { return (float)__builtin_bit_cast(_Float16, v.bits); }
+
+// round-to-nearest-even, NaN stays NaN (quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = f32_to_bits(f);
+    uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
+    r = ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
+    return (uint16_t)(r >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) { return bf16_t{f32_to_bf16_bits(f)}; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) {
+    return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
+}
+
+// ---- division by a runtime constant -------------------------------------------
+// q = n / d for n < 2^32 using one mulhi and one correction; m = floor(2^32 / d) (d >= 2) or
+// the divisor 1 flagged by m == 0.
+struct FastDiv {
+    uint32_t d, m;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d <= 1 ? 0u : (uint32_t)((1ull << 32) / d);
+    return f;
+}
+__device__ __forceinline__ void divmod(uint32_t n, const FastDiv f, uint32_t &q, uint32_t &r) {
+    if (f.m == 0u) { q = n; r = 0; return; }
+    q = __umulhi(n, f.m);
+    r = n - q * f.d;
+    if (r >= f.d) { q += 1; r -= f.d; }
+}
+
+// ---- XCD-aware workgroup order ---------------------------------------------------
+// Hardware deals workgroup ids round-robin over the 8 XCDs (each with its own L2).  This maps
+// a hardware id to a logical id so that every XCD works on one contiguous range of logical
+// workgroups: neighbours (which share B/C rows or cache lines) meet in the same L2.
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t hw_id, uint32_t n_wg) {
+    const uint32_t per = n_wg / kXcds, rem = n_wg % kXcds;
+    const uint32_t xcd = hw_id % kXcds, idx = hw_id / kXcds;
+    return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+// ---- DPP lane movement --------------------------------------------------------------
+// Lanes whose source is out of range (or whose row is masked off) receive `old`.
+template <int kCtrl, int kRowMask = 0xF>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+    return bits_to_f32((uint32_t)__builtin_amdgcn_update_dpp((int)f32_to_bits(old), (int)f32_to_bits(v), kCtrl,
+                                                             kRowMask, 0xF, false));
+}
+constexpr int kDppRowShr1 = 0x111, kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143, kDppWaveShr1 = 0x138;
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return bits_to_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_to_bits(v), lane));
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? SS2D_OK : SS2D_ELAUNCH; }
+
+}  // namespace ss2d
