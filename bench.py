@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the SS2D inference hot path on one MI355X.
+
+Step     = one forward of a random-init VMamba-T (vmamba_tiny_s1l8 shape) on a synthetic
+           (128, 3, 224, 224) bf16 batch already resident in HBM; the reference's throughput
+           protocol (classification/main.py:346-363) with explicit warm-up / step counts.
+value    = images per second of that forward.
+roofline = the selective-scan kernel at stage-1 shape (BASELINE config 1: B=128, D=96, 56x56,
+           K=4, N=1, bf16 in, fp32 out), timed with HIP events on the launch stream;
+           achieved = algorithmic bytes / average launch time, peak = 8 TB/s.
+cpu_baseline = the torch-on-CPU restatement of the reference path (oracle/) run through the same
+           model on a bounded sample, on this box's host cores.
+
+One JSON line is printed on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def scan_bytes(B, KD, L, N, K, s_in, s_out):
+    """Algorithmic bytes of one scan launch: u, delta in; out; B, C rows; A, D, bias."""
+    return B * KD * L * (2 * s_in + s_out) + 2 * B * K * N * L * s_in + 4 * KD * (N + 2)
+
+
+def time_op(fn, reps, warm=5):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps * 1e-3      # seconds per launch
+
+
+def kernel_lines(reps):
+    """Per-kernel timings of the SS2D core at the four VMamba-T stage shapes (bs128, bf16 in)."""
+    import torch
+    import vmamba_amd as va
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(0)
+    out = []
+    for name, (B, D, H, W, N) in dict(stage1=(128, 96, 56, 56, 1), stage2=(128, 192, 28, 28, 1),
+                                      stage3=(128, 384, 14, 14, 1), stage4=(128, 768, 7, 7, 1)).items():
+        K, L = 4, H * W
+        x = torch.randn(B, D, H, W, device=dev, generator=g).bfloat16()
+        delta = (torch.randn(B, K * D, L, device=dev, generator=g) * 0.5).bfloat16()
+        Bm = torch.randn(B, K, N, L, device=dev, generator=g).bfloat16()
+        Cm = torch.randn(B, K, N, L, device=dev, generator=g).bfloat16()
+        A = -torch.arange(1, N + 1, device=dev, dtype=torch.float32).repeat(K * D, 1)
+        Dv = torch.ones(K * D, device=dev)
+        bias = torch.full((K * D,), -3.0, device=dev)
+        xs = va.cross_scan_fn(x)
+        u = xs.view(B, K * D, L)
+        ys = va.selective_scan_fn(u, delta, A, Bm, Cm, Dv, bias, True)
+        ys5 = ys.view(B, K, D, H, W)
+        E = B * D * L
+        t_cs = time_op(lambda: va.cross_scan_fn(x), reps)
+        t_sc = time_op(lambda: va.selective_scan_fn(u, delta, A, Bm, Cm, Dv, bias, True), reps)
+        t_cm = time_op(lambda: va.cross_merge_fn(ys5), reps)
+        b_cs, b_sc, b_cm = 5 * E * 2, scan_bytes(B, K * D, L, N, K, 2, 4), 5 * E * 4
+        out.append(dict(shape=name, B=B, D=D, H=H, W=W, N=N,
+                        cross_scan_us=t_cs * 1e6, cross_scan_GBs=b_cs / t_cs / 1e9,
+                        scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9,
+                        cross_merge_us=t_cm * 1e6, cross_merge_GBs=b_cm / t_cm / 1e9,
+                        core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
+                        scan_bytes=b_sc))
+        log("kernels", out[-1])
+        del x, delta, Bm, Cm, xs, u, ys, ys5
+    return out
+
+
+def cpu_baseline(seconds_budget=30.0):
+    """Reference torch CPU path through the same model, fp32, on a bounded sample."""
+    import torch
+    from oracle.ss2d_core_ref import RefSS2D
+    from vmamba_amd.vssm import vmamba_tiny_s1l8
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    model = vmamba_tiny_s1l8(ss2d_cls=RefSS2D).eval()
+    batch = 16
+    x = torch.randn(batch, 3, 224, 224)
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        model(x)
+        first = time.perf_counter() - t0
+        reps, spent = 0, 0.0
+        while reps < 3 and spent + first < seconds_budget:
+            t0 = time.perf_counter()
+            model(x)
+            spent += time.perf_counter() - t0
+            reps += 1
+    per = spent / reps if reps else first
+    return dict(value=batch / per, unit="img/s", cores=cores, kind="port",
+                sample=f"VMamba-T forward, batch {batch} @224^2 fp32, torch CPU restatement of selective_scan_ref + "
+                       f"torch CrossScan/CrossMerge, {max(reps, 1)} timed forward(s) after 1 warm-up, {per:.2f} s each")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--kernel-reps", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build is the single-GPU SS2D hot path; it runs on exactly one GPU (--gpus 1).")
+        sys.exit(2)
+
+    import torch
+    import vmamba_amd  # noqa: F401  (fails loudly if libss2d_hip.so is missing)
+    from vmamba_amd.vssm import vmamba_tiny_s1l8
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    dev = "cuda:0"
+    torch.backends.cudnn.benchmark = True
+    torch.manual_seed(0)
+    model = vmamba_tiny_s1l8().to(dev).bfloat16().eval()
+    x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
+
+    with torch.no_grad():
+        for i in range(args.warmup):
+            model(x)
+            if i == 0:
+                torch.cuda.synchronize()
+                log("first forward done")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model(x)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    log(f"VMamba-T bs{args.batch}: {ms:.2f} ms/step, {value:.0f} img/s")
+
+    kernels, roofline = None, None
+    if not args.no_kernels:
+        with torch.no_grad():
+            kernels = kernel_lines(args.kernel_reps)
+        k1 = kernels[0]
+        roofline = dict(bound="hbm", kernel="scan_row_kernel<bf16,f32,N=1> @ stage1 (B=128, KD=384, L=3136)",
+                        achieved=k1["scan_GBs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=k1["scan_GBs"] / HBM_PEAK_GBS,
+                        traffic=None, bytes_per_launch=k1["scan_bytes"], us_per_launch=k1["scan_us"])
+    cpu = None if args.no_cpu_baseline else cpu_baseline()
+
+    print(json.dumps({
+        "metric": "VMamba-T img/s @224^2 bs128 on 1xMI355X; SS2D scan HBM GB/s vs peak",
+        "value": value, "unit": "img/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
+                               "bf16 activations/weights, fp32 scan state; SS2D core on HIP kernels"},
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
+    }))
+
+
+if __name__ == "__main__":
+    main()

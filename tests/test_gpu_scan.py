@@ -54,11 +54,11 @@ def run_gpu(u, delta, A, B, C, D, bias, softplus, out_float=True):
     return out.cpu(), x.cpu()
 
 
-def check(u, delta, A, B, C, D, bias, softplus, out_float=True):
+def check(u, delta, A, B, C, D, bias, softplus, out_float=True, tol32=None):
     want, xw = orc.selective_scan(u, delta, A, B, C, D, bias, softplus, out_float=out_float, return_x=True)
     got, xg = run_gpu(u, delta, A, B, C, D, bias, softplus, out_float)
     assert got.dtype == want.dtype and got.shape == want.shape
-    tol = TOL32 if out_float or u.dtype == torch.float32 else TOL16
+    tol = (tol32 or TOL32) if out_float or u.dtype == torch.float32 else TOL16
     err = (got.float() - want.float()).abs().max().item()
     assert torch.allclose(got.float(), want.float(), **tol), f"max abs err {err}"
     assert torch.allclose(xg[..., 1::2], xw[..., 1::2], **TOL32), "chunk-end states"
@@ -133,7 +133,10 @@ def test_scan_delta_group_broadcast(L):
 def test_scan_many_rows_long_sequence_uses_one_wave_per_row():
     # >= 16384 rows with L > 2048: the unsplit kernel carries state across 2048-chunks in registers
     _announce("scan-manyrows")
-    check(*make_inputs(26, 4, 4096, 4, 1, 2560, torch.bfloat16), True)
+    # 42 M outputs of the reference's test distribution (A down to 0: state memory as long as the row, |y| up to
+    # ~230): the fp32 oracle itself is 3e-4 away from float64 here, so the absolute part of the tolerance is the
+    # reference's own fp32 atol, test_selective_scan.py:401
+    check(*make_inputs(26, 4, 4096, 4, 1, 2560, torch.bfloat16), True, tol32=dict(rtol=1e-3, atol=2e-3))
 
 
 def test_scan_strided_views_of_the_projection():

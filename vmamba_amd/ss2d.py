@@ -1,0 +1,117 @@
+"""SS2D block and its hot core, mirroring SS2Dv2 of classification/models/vmamba.py:380-664.
+
+``SS2D.forward_core`` keeps the reference's calling convention, ``(B, D, H, W) -> (B, D, H, W)``
+channel-first (vmamba.py:493-646, the non-cascade ``cross2d`` branch with ``no_einsum=True``,
+``force_fp32=False``, i.e. forward types ``v05`` / ``v05_noz``):
+
+    CrossScan -> x_proj -> split (dt, B, C) -> dt_proj -> selective scan -> CrossMerge -> out_norm
+
+CrossScan, the selective scan and CrossMerge run on this package's HIP kernels; the two tiny
+projections stay PyTorch-ROCm GEMMs.  B and C are handed to the scan as strided views of the
+projection output: the kernel honours batch/group/state strides, so the reference's
+``.contiguous()`` copies (vmamba.py:621-622) are not needed.
+
+Parameter names, shapes and initialisation follow vmamba.py:165-232 and :463-479, so a
+reference state_dict of this block loads as is.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .csm import cross_merge_fn, cross_scan_fn
+from .csms6s import selective_scan_fn
+
+
+class Linear2d(nn.Linear):
+    """1x1 convolution stored as a Linear weight (vmamba.py:42-49)."""
+
+    def forward(self, x):
+        return F.conv2d(x, self.weight[:, :, None, None], self.bias)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        key = prefix + "weight"
+        if key in state_dict:
+            state_dict[key] = state_dict[key].view(self.weight.shape)
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+
+class LayerNorm2d(nn.LayerNorm):
+    """LayerNorm over the channel axis of a (B, C, H, W) tensor (vmamba.py:52-57)."""
+
+    def forward(self, x):
+        y = F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight.to(x.dtype),
+                         self.bias.to(x.dtype), self.eps)
+        return y.permute(0, 3, 1, 2)
+
+
+def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.1, dt_init_floor=1e-4, k_group=4):
+    """S4D-real A, unit D, dt bias = softplus^-1(dt), dt log-uniform in [dt_min, dt_max] (vmamba.py:165-232)."""
+    std = dt_rank ** -0.5 * dt_scale
+    dt_w = torch.empty(k_group, d_inner, dt_rank).uniform_(-std, std)
+    dt = torch.exp(torch.rand(k_group, d_inner) * (math.log(dt_max) - math.log(dt_min)) + math.log(dt_min)).clamp(min=dt_init_floor)
+    dt_b = dt + torch.log(-torch.expm1(-dt))
+    A_logs = torch.log(torch.arange(1, d_state + 1, dtype=torch.float32)).repeat(k_group * d_inner, 1)
+    Ds = torch.ones(k_group * d_inner)
+    return nn.Parameter(A_logs), nn.Parameter(Ds), nn.Parameter(dt_w), nn.Parameter(dt_b)
+
+
+class SS2D(nn.Module):
+    """Channel-first SS2D block: in_proj -> dwconv3x3 -> SiLU -> forward_core -> (gate) -> out_proj."""
+
+    def __init__(self, d_model=96, d_state=1, ssm_ratio=1.0, dt_rank="auto", d_conv=3, conv_bias=False, bias=False,
+                 disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4):
+        super().__init__()
+        self.k_group = 4
+        self.d_model, self.d_state = int(d_model), int(d_state)
+        self.d_inner = int(ssm_ratio * d_model)
+        self.dt_rank = int(math.ceil(self.d_model / 16) if dt_rank == "auto" else dt_rank)
+        self.disable_z = disable_z
+        self.with_dconv = d_conv > 1
+        self.in_proj = Linear2d(self.d_model, self.d_inner if disable_z else 2 * self.d_inner, bias=bias)
+        self.act = nn.SiLU()
+        if self.with_dconv:
+            self.conv2d = nn.Conv2d(self.d_inner, self.d_inner, kernel_size=d_conv, padding=(d_conv - 1) // 2,
+                                    groups=self.d_inner, bias=conv_bias)
+        x_proj = [nn.Linear(self.d_inner, self.dt_rank + 2 * self.d_state, bias=False) for _ in range(self.k_group)]
+        self.x_proj_weight = nn.Parameter(torch.stack([t.weight for t in x_proj], dim=0))   # (K, R+2N, D)
+        self.out_norm = LayerNorm2d(self.d_inner)
+        self.out_proj = Linear2d(self.d_inner, self.d_model, bias=bias)
+        self.A_logs, self.Ds, self.dt_projs_weight, self.dt_projs_bias = init_dt_A_D(
+            self.d_state, self.dt_rank, self.d_inner, dt_scale, dt_min, dt_max, dt_init_floor, self.k_group)
+
+    def project(self, xs):
+        """x_proj / dt_proj as grouped 1x1 conv1d (vmamba.py:605-608).  xs: (B, K, D, L)."""
+        B, K, D, L = xs.shape
+        R, N = self.dt_rank, self.d_state
+        x_dbl = F.conv1d(xs.view(B, K * D, L), self.x_proj_weight.view(-1, D, 1), groups=K)
+        dts, Bs, Cs = torch.split(x_dbl.view(B, K, -1, L), [R, N, N], dim=2)
+        dts = F.conv1d(dts.contiguous().view(B, K * R, L), self.dt_projs_weight.view(K * D, R, 1), groups=K)
+        return dts, Bs, Cs
+
+    def forward_core(self, x):
+        B, D, H, W = x.shape
+        K, L = self.k_group, H * W
+        xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
+        dts, Bs, Cs = self.project(xs)
+        As = -self.A_logs.float().exp()
+        ys = selective_scan_fn(xs.view(B, K * D, L), dts, As, Bs, Cs, self.Ds.float(),
+                               self.dt_projs_bias.view(-1).float(), True, True)                # fp32 (oflex)
+        y = cross_merge_fn(ys.view(B, K, D, H, W), in_channel_first=True, out_channel_first=True, scans=0)
+        y = self.out_norm(y.view(B, D, H, W))
+        return y.to(x.dtype)
+
+    def forward(self, x):
+        x = self.in_proj(x)
+        z = None
+        if not self.disable_z:
+            x, z = x.chunk(2, dim=1)
+            z = self.act(z)
+        if self.with_dconv:
+            x = self.conv2d(x)
+        x = self.act(x)
+        y = self.forward_core(x)
+        if z is not None:
+            y = y * z
+        return self.out_proj(y)
