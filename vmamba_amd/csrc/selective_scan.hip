@@ -235,6 +235,122 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     }
 }
 
+// ---- many short rows per wavefront ------------------------------------------------------------
+// Rows shorter than a pass would leave most lanes idle in the row kernel.  Here a wavefront
+// walks a contiguous run of `rows_per_wave` rows as ONE stream of positions (u, delta and out
+// are dense, so consecutive rows are adjacent in memory and the 16-byte lane vectors stay
+// aligned because rows_per_wave is a multiple of 8).  The recurrence restarts at every row
+// simply by forcing a = 0 at a row's first position: the pair (0, b) discards whatever state
+// arrives from the previous row.  Per-row constants (A, D, bias, the B/C row) are held for the
+// at most two rows a lane's 8 items can touch (L >= 8) and selected per item; B and C are
+// gathered element-wise (their rows are shared by dim/n_groups channels and stay in L1/L2).
+template <typename in_t, typename out_t, int kN>
+__global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int rows_per_wave, FastDiv divL,
+                                                           FastDiv divDim, FastDiv divDpg) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int64_t r0 = ((int64_t)wg * kWavesPerWg + wave) * rows_per_wave;
+    if (r0 >= p.rows) return;
+    const int L = p.L;
+    const int n_rows = (int)min((int64_t)rows_per_wave, (int64_t)p.rows - r0);
+    const int n_el = n_rows * L;
+    const in_t *u_base = reinterpret_cast<const in_t *>(p.u) + r0 * L;
+    const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + r0 * L;
+    const in_t *B_base = reinterpret_cast<const in_t *>(p.B);
+    const in_t *C_base = reinterpret_cast<const in_t *>(p.C);
+    out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
+    const bool softplus = p.softplus != 0;
+
+    float h_reg[kN];
+#pragma unroll
+    for (int n = 0; n < kN; ++n) h_reg[n] = 0.0f;
+
+    const int n_pass = (n_el + kPass - 1) / kPass;
+    for (int pass = 0; pass < n_pass; ++pass) {
+        const int e0 = pass * kPass + lane * kItems;
+        const bool full = e0 + kItems <= n_el;
+        float uv[kItems], dl[kItems];
+        if (full) {
+            load_items<in_t, true>(u_base, e0, n_el, uv);
+            load_items<in_t, true>(dl_base, e0, n_el, dl);
+        } else {
+            load_items<in_t, false>(u_base, e0, n_el, uv);
+            load_items<in_t, false>(dl_base, e0, n_el, dl);
+        }
+
+        // the (at most) two rows this lane touches
+        uint32_t rl, l0;
+        divmod((uint32_t)min(e0, n_el - 1), divL, rl, l0);
+        const int k = min(kItems, L - (int)l0);              // items [0,k) in row a, [k,8) in row b
+        float A_a[kN], A_b[kN], D_a, D_b, bias_a, bias_b;
+        int64_t Boff_a, Boff_b, Coff_a, Coff_b;
+        {
+            const uint32_t row_a = (uint32_t)r0 + rl;
+            const uint32_t row_b = min(row_a + 1u, (uint32_t)p.rows - 1u);
+            uint32_t b, d, grp, rem;
+            divmod(row_a, divDim, b, d);
+            divmod(d, divDpg, grp, rem);
+#pragma unroll
+            for (int n = 0; n < kN; ++n) A_a[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
+            D_a = p.D ? p.D[d] : 0.0f;
+            bias_a = p.bias ? p.bias[d] : 0.0f;
+            Boff_a = b * p.B_bs + grp * p.B_gs;
+            Coff_a = b * p.C_bs + grp * p.C_gs;
+            divmod(row_b, divDim, b, d);
+            divmod(d, divDpg, grp, rem);
+#pragma unroll
+            for (int n = 0; n < kN; ++n) A_b[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
+            D_b = p.D ? p.D[d] : 0.0f;
+            bias_b = p.bias ? p.bias[d] : 0.0f;
+            Boff_b = b * p.B_bs + grp * p.B_gs;
+            Coff_b = b * p.C_bs + grp * p.C_gs;
+        }
+
+        float du[kItems], y[kItems];
+        int64_t boff[kItems], coff[kItems];
+        bool first[kItems], valid[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const bool in_a = i < k;
+            const int li = in_a ? (int)l0 + i : i - k;
+            valid[i] = e0 + i < n_el;
+            first[i] = li == 0;
+            float d = dl[i] + (in_a ? bias_a : bias_b);
+            if (softplus) d = softplus_f32(d);
+            d = valid[i] ? d : 0.0f;
+            dl[i] = d;
+            du[i] = d * uv[i];
+            y[i] = (in_a ? D_a : D_b) * uv[i];
+            boff[i] = (in_a ? Boff_a : Boff_b) + li;
+            coff[i] = (in_a ? Coff_a : Coff_b) + li;
+        }
+
+#pragma unroll
+        for (int n = 0; n < kN; ++n) {
+            float ac[kItems], hh[kItems], Cv[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const float Bv = valid[i] ? to_f32(B_base[boff[i] + n * p.B_ns]) : 0.0f;
+                Cv[i] = valid[i] ? to_f32(C_base[coff[i] + n * p.C_ns]) : 0.0f;
+                float a = __builtin_amdgcn_exp2f(dl[i] * (i < k ? A_a[n] : A_b[n]));
+                a = first[i] ? 0.0f : a;
+                const float bb = Bv * du[i];
+                ac[i] = i == 0 ? a : ac[i - 1] * a;
+                hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
+            }
+            float a_ex, h_ex, a_tot, h_tot;
+            wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+            const float s_in = fmaf(a_ex, h_reg[n], h_ex);
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
+            h_reg[n] = fmaf(a_tot, h_reg[n], h_tot);
+        }
+        if (full) store_items<out_t, true>(o_base, e0, n_el, y);
+        else store_items<out_t, false>(o_base, e0, n_el, y);
+    }
+}
+
 // ---- four wavefronts per row -------------------------------------------------------------
 // Workgroup = one row.  Per 2048-position chunk wave w takes positions [w*512, w*512+512).
 // LDS: agg[2][N][4] pass totals (double-buffered by chunk parity), state[2][N] chunk-start
@@ -314,6 +430,35 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
 // ---- host side -----------------------------------------------------------------------------
 static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+constexpr int kFlatMaxL = 1024;          // rows shorter than this go to the flat kernel
+constexpr int kFlatTargetElems = 4096;   // positions a wavefront of the flat kernel walks
+
+// The flat kernel needs dense u / delta / out (rows adjacent in memory, base 16-byte aligned), one delta row
+// per channel, no chunk-state output, rows of at least one lane vector, and dstate 1 or 16.
+static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
+    const int64_t L = a.L, KD = a.dim;
+    return a.x == nullptr && L >= kItems && L < kFlatMaxL && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
+           a.u_ds == L && a.dl_ds == L && a.o_ds == L && a.u_bs == KD * L && a.dl_bs == KD * L && a.o_bs == KD * L &&
+           aligned16(q->u) && aligned16(q->delta) && aligned16(q->out);
+}
+
+template <typename in_t, typename out_t>
+static int launch_flat(const ScanArgs &a, hipStream_t stream) {
+    int rows_per_wave = 8 * (int)((kFlatTargetElems + 8 * (int64_t)a.L - 1) / (8 * (int64_t)a.L));
+    const int64_t n_waves = ((int64_t)a.rows + rows_per_wave - 1) / rows_per_wave;
+    const uint32_t n_wg = (uint32_t)((n_waves + kWavesPerWg - 1) / kWavesPerWg);
+    const FastDiv dL = make_fastdiv((uint32_t)a.L), dDim = make_fastdiv((uint32_t)a.dim),
+                  dDpg = make_fastdiv((uint32_t)a.dim_per_group);
+    if (a.N == 1) {
+        hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, 1>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL,
+                           dDim, dDpg);
+    } else {
+        hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, 16>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL,
+                           dDim, dDpg);
+    }
+    return launch_status();
+}
+
 template <typename in_t, typename out_t, bool kVec>
 static int launch_scan(const ScanArgs &a, hipStream_t stream) {
     // Few long rows: split every row over the 4 wavefronts of a workgroup.
@@ -336,7 +481,8 @@ static int launch_scan(const ScanArgs &a, hipStream_t stream) {
 }
 
 template <typename in_t, typename out_t>
-static int dispatch_vec(const ScanArgs &a, bool vec, hipStream_t stream) {
+static int dispatch_vec(const ScanArgs &a, bool vec, bool flat, hipStream_t stream) {
+    if (flat) return launch_flat<in_t, out_t>(a, stream);
     return vec ? launch_scan<in_t, out_t, true>(a, stream) : launch_scan<in_t, out_t, false>(a, stream);
 }
 
@@ -380,12 +526,14 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     for (int64_t s : in_strides) vec = vec && (s % in_vec == 0);
     vec = vec && (a.o_bs % out_vec == 0) && (a.o_ds % out_vec == 0);
 
+    const bool flat = flat_eligible(a, q);
     hipStream_t s = (hipStream_t)stream;
-    if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, s);
+    if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, flat, s);
     if (q->in_dtype == SS2D_BF16) {
-        return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, s) : dispatch_vec<bf16_t, bf16_t>(a, vec, s);
+        return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, flat, s)
+                                        : dispatch_vec<bf16_t, bf16_t>(a, vec, flat, s);
     }
-    return q->out_dtype == SS2D_F32 ? dispatch_vec<f16_t, float>(a, vec, s) : dispatch_vec<f16_t, f16_t>(a, vec, s);
+    return q->out_dtype == SS2D_F32 ? dispatch_vec<f16_t, float>(a, vec, flat, s) : dispatch_vec<f16_t, f16_t>(a, vec, flat, s);
 }
 
 extern "C" int ss2d_abi_version(void) { return SS2D_ABI_VERSION; }
