@@ -37,6 +37,7 @@ struct ScanArgs {
     int32_t batch, dim, L, N, dim_per_group, dim_per_delta, n_chunks, softplus;
     int64_t u_bs, u_ds, dl_bs, dl_ds, A_ds, A_ns, B_bs, B_gs, B_ns, C_bs, C_gs, C_ns, o_bs, o_ds;
     int32_t rows;
+    uint32_t B_span_bytes, C_span_bytes;   // flat kernel: extent of B / C reachable through the strides
 };
 
 // ---- 8-wide loads / stores ------------------------------------------------------------
@@ -86,6 +87,17 @@ __device__ __forceinline__ void store_items(T *__restrict__ row, int pos, int L,
 #pragma unroll
         for (int i = 0; i < kItems; ++i)
             if (pos + i < L) row[pos + i] = from_f32<T>(v[i]);
+    }
+}
+
+constexpr int kBufferRsrcWord3 = 0x00020000;   // raw buffer, 32-bit data format (gfx9 family)
+
+template <typename T>
+__device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset) {
+    if constexpr (sizeof(T) == 2) {
+        return to_f32(T{(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)(elem_offset * 2u), 0, 0)});
+    } else {
+        return bits_to_f32((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(elem_offset * 4u), 0, 0));
     }
 }
 
@@ -257,8 +269,10 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     const int n_el = n_rows * L;
     const in_t *u_base = reinterpret_cast<const in_t *>(p.u) + r0 * L;
     const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + r0 * L;
-    const in_t *B_base = reinterpret_cast<const in_t *>(p.B);
-    const in_t *C_base = reinterpret_cast<const in_t *>(p.C);
+    // B and C are gathered through buffer descriptors: a 32-bit byte offset per lane, no 64-bit address math,
+    // and hardware range checking (an offset past the extent reads 0).
+    const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.B), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
+    const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
     const bool softplus = p.softplus != 0;
 
@@ -284,7 +298,7 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
         divmod((uint32_t)min(e0, n_el - 1), divL, rl, l0);
         const int k = min(kItems, L - (int)l0);              // items [0,k) in row a, [k,8) in row b
         float A_a[kN], A_b[kN], D_a, D_b, bias_a, bias_b;
-        int64_t Boff_a, Boff_b, Coff_a, Coff_b;
+        uint32_t Boff_a, Boff_b, Coff_a, Coff_b;      // element offsets; the host checked they fit 32 bits
         {
             const uint32_t row_a = (uint32_t)r0 + rl;
             const uint32_t row_b = min(row_a + 1u, (uint32_t)p.rows - 1u);
@@ -295,32 +309,34 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
             for (int n = 0; n < kN; ++n) A_a[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
             D_a = p.D ? p.D[d] : 0.0f;
             bias_a = p.bias ? p.bias[d] : 0.0f;
-            Boff_a = b * p.B_bs + grp * p.B_gs;
-            Coff_a = b * p.C_bs + grp * p.C_gs;
+            Boff_a = b * (uint32_t)p.B_bs + grp * (uint32_t)p.B_gs;
+            Coff_a = b * (uint32_t)p.C_bs + grp * (uint32_t)p.C_gs;
             divmod(row_b, divDim, b, d);
             divmod(d, divDpg, grp, rem);
 #pragma unroll
             for (int n = 0; n < kN; ++n) A_b[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
             D_b = p.D ? p.D[d] : 0.0f;
             bias_b = p.bias ? p.bias[d] : 0.0f;
-            Boff_b = b * p.B_bs + grp * p.B_gs;
-            Coff_b = b * p.C_bs + grp * p.C_gs;
+            Boff_b = b * (uint32_t)p.B_bs + grp * (uint32_t)p.B_gs;
+            Coff_b = b * (uint32_t)p.C_bs + grp * (uint32_t)p.C_gs;
         }
 
+        // Every item's (row, position) is a real element of B / C even for items past the end of this
+        // wavefront's run (row_b is clamped, positions stay below L), so the gathers need no guard.
         float du[kItems], y[kItems];
-        int64_t boff[kItems], coff[kItems];
-        bool first[kItems], valid[kItems];
+        uint32_t boff[kItems], coff[kItems];
+        bool first[kItems];
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
             const bool in_a = i < k;
-            const int li = in_a ? (int)l0 + i : i - k;
-            valid[i] = e0 + i < n_el;
+            const uint32_t li = in_a ? l0 + i : (uint32_t)(i - k);
+            const bool valid = e0 + i < n_el;
             first[i] = li == 0;
             float d = dl[i] + (in_a ? bias_a : bias_b);
             if (softplus) d = softplus_f32(d);
-            d = valid[i] ? d : 0.0f;
+            d = valid ? d : 0.0f;
             dl[i] = d;
-            du[i] = d * uv[i];
+            du[i] = valid ? d * uv[i] : 0.0f;
             y[i] = (in_a ? D_a : D_b) * uv[i];
             boff[i] = (in_a ? Boff_a : Boff_b) + li;
             coff[i] = (in_a ? Coff_a : Coff_b) + li;
@@ -328,14 +344,19 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
 
 #pragma unroll
         for (int n = 0; n < kN; ++n) {
-            float ac[kItems], hh[kItems], Cv[kItems];
+            float Bv[kItems], Cv[kItems];
 #pragma unroll
             for (int i = 0; i < kItems; ++i) {
-                const float Bv = valid[i] ? to_f32(B_base[boff[i] + n * p.B_ns]) : 0.0f;
-                Cv[i] = valid[i] ? to_f32(C_base[coff[i] + n * p.C_ns]) : 0.0f;
+                Bv[i] = gather_elem<in_t>(B_rsrc, boff[i] + (uint32_t)n * (uint32_t)p.B_ns);
+                Cv[i] = gather_elem<in_t>(C_rsrc, coff[i] + (uint32_t)n * (uint32_t)p.C_ns);
+            }
+            float ac[kItems], hh[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
                 float a = __builtin_amdgcn_exp2f(dl[i] * (i < k ? A_a[n] : A_b[n]));
                 a = first[i] ? 0.0f : a;
-                const float bb = Bv * du[i];
+                // past the end of the run the gathered B belongs to some other row: keep it out
+                const float bb = (e0 + i < n_el) ? Bv[i] * du[i] : 0.0f;
                 ac[i] = i == 0 ? a : ac[i - 1] * a;
                 hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
             }
@@ -433,17 +454,32 @@ static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr
 constexpr int kFlatMaxL = 1024;          // rows shorter than this go to the flat kernel
 constexpr int kFlatTargetElems = 4096;   // positions a wavefront of the flat kernel walks
 
+// Largest element offset the flat kernel forms into B or C (it indexes them with 32-bit offsets).
+static int64_t span_elems(const ScanArgs &a, int64_t bs, int64_t gs, int64_t ns) {
+    const int64_t groups = a.dim / a.dim_per_group;
+    return (int64_t)(a.batch - 1) * bs + (groups - 1) * gs + (int64_t)(a.N - 1) * ns + a.L;
+}
+static bool span_fits_u32(const ScanArgs &a, int64_t elem_bytes) {
+    const int64_t lim = 0x7fffffffll;   // byte extents are handed to the buffer descriptor as a positive int
+    return a.B_bs >= 0 && a.B_gs >= 0 && a.B_ns >= 0 && a.C_bs >= 0 && a.C_gs >= 0 && a.C_ns >= 0 &&
+           span_elems(a, a.B_bs, a.B_gs, a.B_ns) * elem_bytes < lim && span_elems(a, a.C_bs, a.C_gs, a.C_ns) * elem_bytes < lim;
+}
+
 // The flat kernel needs dense u / delta / out (rows adjacent in memory, base 16-byte aligned), one delta row
 // per channel, no chunk-state output, rows of at least one lane vector, and dstate 1 or 16.
 static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
     const int64_t L = a.L, KD = a.dim;
     return a.x == nullptr && L >= kItems && L < kFlatMaxL && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
            a.u_ds == L && a.dl_ds == L && a.o_ds == L && a.u_bs == KD * L && a.dl_bs == KD * L && a.o_bs == KD * L &&
-           aligned16(q->u) && aligned16(q->delta) && aligned16(q->out);
+           aligned16(q->u) && aligned16(q->delta) && aligned16(q->out) &&
+           span_fits_u32(a, q->in_dtype == SS2D_F32 ? 4 : 2);
 }
 
 template <typename in_t, typename out_t>
-static int launch_flat(const ScanArgs &a, hipStream_t stream) {
+static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
+    ScanArgs a = a_in;
+    a.B_span_bytes = (uint32_t)(span_elems(a, a.B_bs, a.B_gs, a.B_ns) * (int64_t)sizeof(in_t));
+    a.C_span_bytes = (uint32_t)(span_elems(a, a.C_bs, a.C_gs, a.C_ns) * (int64_t)sizeof(in_t));
     int rows_per_wave = 8 * (int)((kFlatTargetElems + 8 * (int64_t)a.L - 1) / (8 * (int64_t)a.L));
     const int64_t n_waves = ((int64_t)a.rows + rows_per_wave - 1) / rows_per_wave;
     const uint32_t n_wg = (uint32_t)((n_waves + kWavesPerWg - 1) / kWavesPerWg);
@@ -516,6 +552,7 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     a.C_bs = q->C_batch_stride; a.C_gs = q->C_group_stride; a.C_ns = q->C_dstate_stride;
     a.o_bs = q->out_batch_stride; a.o_ds = q->out_d_stride;
     a.rows = q->batch * q->dim;
+    a.B_span_bytes = a.C_span_bytes = 0;
 
     // 16-byte vector I/O needs every row start and the row length on a 16-byte grid.
     const int64_t in_vec = q->in_dtype == SS2D_F32 ? 4 : 8;
