@@ -122,6 +122,8 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--layout", choices=["channel_first", "channel_last"], default="channel_last",
+                    help="activation layout of the harness outside the SS2D core (same weights, same math)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build is the single-GPU SS2D hot path; it runs on exactly one GPU (--gpus 1).")
@@ -135,7 +137,7 @@ def main():
     dev = "cuda:0"
     torch.backends.cudnn.benchmark = True
     torch.manual_seed(0)
-    model = vmamba_tiny_s1l8().to(dev).bfloat16().eval()
+    model = vmamba_tiny_s1l8(channel_first=(args.layout == "channel_first")).to(dev).bfloat16().eval()
     x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
 
     with torch.no_grad():
@@ -170,7 +172,7 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
-                               "bf16 activations/weights, fp32 scan state; SS2D core on HIP kernels"},
+                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks; SS2D core on HIP kernels"},
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
     }))
 

@@ -20,4 +20,4 @@ class RefSS2D(SS2D):
         ys = torch_ref.selective_scan(xs.reshape(B, K * D, L), dts, -self.A_logs.float().exp(), Bs.contiguous(),
                                       Cs.contiguous(), self.Ds.float(), self.dt_projs_bias.view(-1).float(), True)
         y = torch_ref.cross_merge(ys.view(B, K, D, H, W))
-        return self.out_norm(y.view(B, D, H, W)).to(x.dtype)
+        return self.finish_core(y, B, D, H, W, x.dtype)

@@ -55,12 +55,13 @@ def test_block_with_gate_matches():
         assert torch.allclose(hip(x.to(DEV)).cpu(), ref(x), rtol=1e-3, atol=1e-3)
 
 
-def test_vmamba_tiny_logits_match_reference_core():
-    print("CASE vssm", flush=True)
+@pytest.mark.parametrize("channel_first", [True, False])
+def test_vmamba_tiny_logits_match_reference_core(channel_first):
+    print("CASE vssm", channel_first, flush=True)
     torch.manual_seed(4)
-    ref = vmamba_tiny_s1l8(ss2d_cls=RefSS2D).eval()
+    ref = vmamba_tiny_s1l8(ss2d_cls=RefSS2D).eval()                  # reference core, channel-first layout
     assert sum(p.numel() for p in ref.parameters()) == 30249064      # analyze/tp.py:162
-    hip = vmamba_tiny_s1l8().eval()
+    hip = vmamba_tiny_s1l8(channel_first=channel_first).eval()
     hip.load_state_dict(ref.state_dict())
     hip = hip.to(DEV)
     x = torch.randn(2, 3, 96, 96, generator=torch.Generator().manual_seed(5))

@@ -451,7 +451,6 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
 // ---- host side -----------------------------------------------------------------------------
 static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
-constexpr int kFlatMaxL = 1024;          // rows shorter than this go to the flat kernel
 constexpr int kFlatTargetElems = 4096;   // positions a wavefront of the flat kernel walks
 
 // Largest element offset the flat kernel forms into B or C (it indexes them with 32-bit offsets).
@@ -469,7 +468,7 @@ static bool span_fits_u32(const ScanArgs &a, int64_t elem_bytes) {
 // per channel, no chunk-state output, rows of at least one lane vector, and dstate 1 or 16.
 static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
     const int64_t L = a.L, KD = a.dim;
-    return a.x == nullptr && L >= kItems && L < kFlatMaxL && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
+    return a.x == nullptr && L >= kItems && L < 4 * kPass && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
            a.u_ds == L && a.dl_ds == L && a.o_ds == L && a.u_bs == KD * L && a.dl_bs == KD * L && a.o_bs == KD * L &&
            aligned16(q->u) && aligned16(q->delta) && aligned16(q->out) &&
            span_fits_u32(a, q->in_dtype == SS2D_F32 ? 4 : 2);
@@ -563,7 +562,10 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     for (int64_t s : in_strides) vec = vec && (s % in_vec == 0);
     vec = vec && (a.o_bs % out_vec == 0) && (a.o_ds % out_vec == 0);
 
-    const bool flat = flat_eligible(a, q);
+    // A pass of the flat kernel costs about 1.4x a pass of the row kernel (measured), so the flat kernel wins
+    // when the row kernel would leave more than ~30 % of its lanes idle, or cannot use vector I/O at all.
+    const int64_t row_slots = ((int64_t)q->seqlen + kPass - 1) / kPass * kPass;
+    const bool flat = flat_eligible(a, q) && (!vec || 10 * (int64_t)q->seqlen < 7 * row_slots);
     hipStream_t s = (hipStream_t)stream;
     if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, flat, s);
     if (q->in_dtype == SS2D_BF16) {

@@ -58,26 +58,34 @@ def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.
 
 
 class SS2D(nn.Module):
-    """Channel-first SS2D block: in_proj -> dwconv3x3 -> SiLU -> forward_core -> (gate) -> out_proj."""
+    """SS2D block: in_proj -> dwconv3x3 -> SiLU -> forward_core -> (gate) -> out_proj.
+
+    ``channel_first=True`` takes and returns (B, C, H, W) with 1x1-conv projections and LayerNorm2d
+    (the reference's "ln2d" models); ``channel_first=False`` takes and returns (B, H, W, C) with nn.Linear
+    and nn.LayerNorm (its "ln" models, vmamba.py:415-417, 642-643, 654-655).  The core itself always works
+    channel-first.
+    """
 
     def __init__(self, d_model=96, d_state=1, ssm_ratio=1.0, dt_rank="auto", d_conv=3, conv_bias=False, bias=False,
-                 disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4):
+                 disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4, channel_first=True):
         super().__init__()
+        self.channel_first = channel_first
+        Linear = Linear2d if channel_first else nn.Linear
         self.k_group = 4
         self.d_model, self.d_state = int(d_model), int(d_state)
         self.d_inner = int(ssm_ratio * d_model)
         self.dt_rank = int(math.ceil(self.d_model / 16) if dt_rank == "auto" else dt_rank)
         self.disable_z = disable_z
         self.with_dconv = d_conv > 1
-        self.in_proj = Linear2d(self.d_model, self.d_inner if disable_z else 2 * self.d_inner, bias=bias)
+        self.in_proj = Linear(self.d_model, self.d_inner if disable_z else 2 * self.d_inner, bias=bias)
         self.act = nn.SiLU()
         if self.with_dconv:
             self.conv2d = nn.Conv2d(self.d_inner, self.d_inner, kernel_size=d_conv, padding=(d_conv - 1) // 2,
                                     groups=self.d_inner, bias=conv_bias)
         x_proj = [nn.Linear(self.d_inner, self.dt_rank + 2 * self.d_state, bias=False) for _ in range(self.k_group)]
         self.x_proj_weight = nn.Parameter(torch.stack([t.weight for t in x_proj], dim=0))   # (K, R+2N, D)
-        self.out_norm = LayerNorm2d(self.d_inner)
-        self.out_proj = Linear2d(self.d_inner, self.d_model, bias=bias)
+        self.out_norm = LayerNorm2d(self.d_inner) if channel_first else nn.LayerNorm(self.d_inner)
+        self.out_proj = Linear(self.d_inner, self.d_model, bias=bias)
         self.A_logs, self.Ds, self.dt_projs_weight, self.dt_projs_bias = init_dt_A_D(
             self.d_state, self.dt_rank, self.d_inner, dt_scale, dt_min, dt_max, dt_init_floor, self.k_group)
 
@@ -99,15 +107,24 @@ class SS2D(nn.Module):
         ys = selective_scan_fn(xs.view(B, K * D, L), dts, As, Bs, Cs, self.Ds.float(),
                                self.dt_projs_bias.view(-1).float(), True, True)                # fp32 (oflex)
         y = cross_merge_fn(ys.view(B, K, D, H, W), in_channel_first=True, out_channel_first=True, scans=0)
-        y = self.out_norm(y.view(B, D, H, W))
-        return y.to(x.dtype)
+        return self.finish_core(y, B, D, H, W, x.dtype)
+
+    def finish_core(self, y, B, D, H, W, dtype):
+        """out_norm on the merged (B, D, L) map, in the block's layout (vmamba.py:641-646)."""
+        if self.channel_first:
+            return self.out_norm(y.view(B, D, H, W)).to(dtype)
+        y = y.view(B, D, H * W).transpose(1, 2).contiguous().view(B, H, W, D)
+        return F.layer_norm(y, (D,), self.out_norm.weight.to(y.dtype), self.out_norm.bias.to(y.dtype),
+                            self.out_norm.eps).to(dtype)
 
     def forward(self, x):
         x = self.in_proj(x)
         z = None
         if not self.disable_z:
-            x, z = x.chunk(2, dim=1)
+            x, z = x.chunk(2, dim=(1 if self.channel_first else -1))
             z = self.act(z)
+        if not self.channel_first:
+            x = x.permute(0, 3, 1, 2).contiguous()
         if self.with_dconv:
             x = self.conv2d(x)
         x = self.act(x)

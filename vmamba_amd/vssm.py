@@ -1,9 +1,11 @@
 """VMamba-T-shaped backbone used as the throughput harness (random init, inference).
 
 Layer order and shapes follow VSSM / VSSBlock of classification/models/vmamba.py:1153-1505 for
-the ``vmamba_tiny_s1l8`` recipe (:1717-1728): channel-first ("ln2d"), patch-embed v2, downsample
-v3, depths 2/2/8/2, dims 96/192/384/768, d_state 1, ssm_ratio 1, forward type v05_noz, MLP ratio 4.
-Everything outside the SS2D core is stock torch; drop-path is the identity at inference.
+the ``vmamba_tiny_s1l8`` recipe (:1717-1728): patch-embed v2, downsample v3, depths 2/2/8/2, dims
+96/192/384/768, d_state 1, ssm_ratio 1, forward type v05_noz, MLP ratio 4.  As in the reference the
+same weights run in two activation layouts: ``channel_first=True`` ("ln2d": (B,C,H,W), 1x1 convs,
+LayerNorm2d) and ``channel_first=False`` ("ln": (B,H,W,C), nn.Linear, nn.LayerNorm).  Everything
+outside the SS2D core is stock torch; drop-path is the identity at inference.
 """
 import torch
 import torch.nn as nn
@@ -11,24 +13,43 @@ import torch.nn as nn
 from .ss2d import SS2D, LayerNorm2d, Linear2d
 
 
-class Mlp(nn.Module):
-    def __init__(self, dim, hidden):
+class Permute(nn.Module):
+    def __init__(self, *dims):
         super().__init__()
-        self.fc1 = Linear2d(dim, hidden)
+        self.dims = dims
+
+    def forward(self, x):
+        return x.permute(*self.dims)
+
+
+def _to_cl(channel_first):      # (B,C,H,W) -> block layout
+    return nn.Identity() if channel_first else Permute(0, 2, 3, 1)
+
+
+def _to_cf(channel_first):      # block layout -> (B,C,H,W)
+    return nn.Identity() if channel_first else Permute(0, 3, 1, 2)
+
+
+class Mlp(nn.Module):
+    def __init__(self, dim, hidden, channel_first=True):
+        super().__init__()
+        Linear = Linear2d if channel_first else nn.Linear
+        self.fc1 = Linear(dim, hidden)
         self.act = nn.GELU()
-        self.fc2 = Linear2d(hidden, dim)
+        self.fc2 = Linear(hidden, dim)
 
     def forward(self, x):
         return self.fc2(self.act(self.fc1(x)))
 
 
 class VSSBlock(nn.Module):
-    def __init__(self, dim, d_state=1, ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, **ss2d_kwargs):
+    def __init__(self, dim, d_state=1, ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, **ss2d_kwargs):
         super().__init__()
-        self.norm = LayerNorm2d(dim)
-        self.op = ss2d_cls(d_model=dim, d_state=d_state, ssm_ratio=ssm_ratio, **ss2d_kwargs)
-        self.norm2 = LayerNorm2d(dim)
-        self.mlp = Mlp(dim, int(dim * mlp_ratio))
+        Norm = LayerNorm2d if channel_first else nn.LayerNorm
+        self.norm = Norm(dim)
+        self.op = ss2d_cls(d_model=dim, d_state=d_state, ssm_ratio=ssm_ratio, channel_first=channel_first, **ss2d_kwargs)
+        self.norm2 = Norm(dim)
+        self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
     def forward(self, x):
         x = x + self.op(self.norm(x))
@@ -37,20 +58,24 @@ class VSSBlock(nn.Module):
 
 class VSSM(nn.Module):
     def __init__(self, in_chans=3, num_classes=1000, depths=(2, 2, 8, 2), dims=(96, 192, 384, 768), d_state=1,
-                 ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, **ss2d_kwargs):
+                 ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, **ss2d_kwargs):
         super().__init__()
+        cf = channel_first
+        Norm = LayerNorm2d if cf else nn.LayerNorm
         d0 = dims[0]
         self.patch_embed = nn.Sequential(
-            nn.Conv2d(in_chans, d0 // 2, kernel_size=3, stride=2, padding=1), LayerNorm2d(d0 // 2), nn.GELU(),
-            nn.Conv2d(d0 // 2, d0, kernel_size=3, stride=2, padding=1), LayerNorm2d(d0))
+            nn.Conv2d(in_chans, d0 // 2, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0 // 2), _to_cf(cf),
+            nn.GELU(),
+            nn.Conv2d(d0 // 2, d0, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0))
         layers = []
         for i, (depth, dim) in enumerate(zip(depths, dims)):
-            blocks = [VSSBlock(dim, d_state, ssm_ratio, mlp_ratio, ss2d_cls, **ss2d_kwargs) for _ in range(depth)]
-            down = (nn.Sequential(nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), LayerNorm2d(dims[i + 1]))
+            blocks = [VSSBlock(dim, d_state, ssm_ratio, mlp_ratio, ss2d_cls, cf, **ss2d_kwargs) for _ in range(depth)]
+            down = (nn.Sequential(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
+                                  Norm(dims[i + 1]))
                     if i + 1 < len(dims) else nn.Identity())
             layers.append(nn.Sequential(*blocks, down))
         self.layers = nn.ModuleList(layers)
-        self.classifier = nn.Sequential(LayerNorm2d(dims[-1]), nn.AdaptiveAvgPool2d(1), nn.Flatten(1),
+        self.classifier = nn.Sequential(Norm(dims[-1]), _to_cf(cf), nn.AdaptiveAvgPool2d(1), nn.Flatten(1),
                                         nn.Linear(dims[-1], num_classes))
         self.apply(self._init_weights)
 
@@ -71,5 +96,6 @@ class VSSM(nn.Module):
         return self.classifier(x)
 
 
-def vmamba_tiny_s1l8(**kwargs):
-    return VSSM(depths=(2, 2, 8, 2), dims=(96, 192, 384, 768), d_state=1, ssm_ratio=1.0, mlp_ratio=4.0, **kwargs)
+def vmamba_tiny_s1l8(channel_first=True, **kwargs):
+    return VSSM(depths=(2, 2, 8, 2), dims=(96, 192, 384, 768), d_state=1, ssm_ratio=1.0, mlp_ratio=4.0,
+                channel_first=channel_first, **kwargs)
