@@ -122,6 +122,9 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="skip the model: time the SS2D-core kernels at the four stage shapes plus a 1 GiB "
+                         "device copy (the known-size kernel profiler counters are scaled against)")
     ap.add_argument("--layout", choices=["channel_first", "channel_last"], default="channel_last",
                     help="activation layout of the harness outside the SS2D core (same weights, same math)")
     args = ap.parse_args()
@@ -135,6 +138,15 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = "cuda:0"
+    if args.kernels_only:
+        with torch.no_grad():
+            src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+            dst = torch.empty_like(src)
+            t = time_op(lambda: dst.copy_(src), args.kernel_reps)
+            log(f"calibration copy: 1 GiB read + 1 GiB write in {t * 1e6:.1f} us = {2 * (1 << 30) / t / 1e9:.0f} GB/s")
+            del src, dst
+            print(json.dumps({"kernels": kernel_lines(args.kernel_reps)}))
+        return
     torch.backends.cudnn.benchmark = True
     torch.manual_seed(0)
     model = vmamba_tiny_s1l8(channel_first=(args.layout == "channel_first")).to(dev).bfloat16().eval()
