@@ -41,13 +41,16 @@ struct ScanArgs {
 };
 
 // ---- 8-wide loads / stores ------------------------------------------------------------
+// Items at positions >= L come back as `fill`.
 template <typename T, bool kVec>
-__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems]) {
+__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems],
+                                           float fill = 0.0f) {
     if constexpr (kVec) {
         // the host guarantees 16-byte alignment and L % (16/sizeof(T)) == 0, so a vector is either
         // entirely inside the row or entirely outside
         if constexpr (sizeof(T) == 2) {
-            uint4 raw = make_uint4(0, 0, 0, 0);
+            const uint32_t fill2 = (uint32_t)from_f32<T>(fill).bits * 0x10001u;
+            uint4 raw = make_uint4(fill2, fill2, fill2, fill2);
             if (pos < L) raw = *reinterpret_cast<const uint4 *>(row + pos);
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -56,7 +59,7 @@ __device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, i
                 v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
             }
         } else {
-            float4 lo = make_float4(0, 0, 0, 0), hi = make_float4(0, 0, 0, 0);
+            float4 lo = make_float4(fill, fill, fill, fill), hi = lo;
             if (pos < L) lo = *reinterpret_cast<const float4 *>(row + pos);
             if (pos + 4 < L) hi = *reinterpret_cast<const float4 *>(row + pos + 4);
             v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
@@ -64,7 +67,7 @@ __device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, i
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) v[i] = (pos + i < L) ? to_f32(row[pos + i]) : 0.0f;
+        for (int i = 0; i < kItems; ++i) v[i] = (pos + i < L) ? to_f32(row[pos + i]) : fill;
     }
 }
 
@@ -101,14 +104,41 @@ __device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32
     }
 }
 
-// softplus(x) = log1p(exp(x)) with two hardware transcendentals; for small exp(x) the series
-// t - t^2/2 + t^3/3 replaces log(1+t), whose rounding of 1+t would otherwise dominate.
-__device__ __forceinline__ float softplus_f32(float x) {
-    const float t = __builtin_amdgcn_exp2f(fminf(x, 20.0f) * kLog2e);
-    const float series = t * (1.0f - t * (0.5f - t * 0.33333334f));
-    const float full = kLn2 * __builtin_amdgcn_logf(1.0f + t);
-    const float sp = t < 0.015625f ? series : full;
-    return x > 20.0f ? x : sp;
+// delta -> dl for the 8 items of a lane.
+//   kSoftplus: dl = softplus(raw + bias) = ln2 * log2(1 + 2^((raw + bias) * log2e)) with the two hardware
+//   transcendentals.  w = 1 + t loses the low bits of a small t; c = t - (w - 1) is exactly that loss (t < 1), and
+//   log(1 + t) = log(w) + c/w with c/w ~ c.  Arguments above 20 return the argument itself (the reference's
+//   threshold); that select sits behind a wave-uniform vote because it is almost never taken.
+//   A raw value of -inf (the fill for positions past the end of a row) gives t = 0, dl = 0: the identity pair.
+//   !kSoftplus: dl = raw + bias; the caller zeroes positions past the end.
+constexpr float kSoftplusThreshold = 20.0f;
+
+template <bool kSoftplus>
+__device__ __forceinline__ void delta_transform(const float (&raw)[kItems], const float (&bias)[kItems],
+                                                float (&dl)[kItems]) {
+    if constexpr (kSoftplus) {
+        float zmax = -__builtin_inff();
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const float z = fmaf(raw[i], kLog2e, bias[i] * kLog2e);
+            zmax = __builtin_fmaxf(zmax, z);
+            const float t = __builtin_amdgcn_exp2f(z);
+            const float w = 1.0f + t;
+            float c = t - (w - 1.0f);
+            c = t < 1.0f ? c : 0.0f;
+            dl[i] = fmaf(kLn2, __builtin_amdgcn_logf(w), c);
+        }
+        if (__builtin_amdgcn_ballot_w64(zmax > kSoftplusThreshold * kLog2e) != 0) {
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const float x = raw[i] + bias[i];
+                dl[i] = x > kSoftplusThreshold ? x : dl[i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) dl[i] = raw[i] + bias[i];
+    }
 }
 
 // Inclusive scan of (a,h) over the 64 lanes; returns this lane's EXCLUSIVE prefix in
@@ -156,20 +186,19 @@ __device__ __forceinline__ void scan_state_pass(const float (&dl)[kItems], const
     for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
 }
 
-template <typename in_t, bool kVec>
+template <typename in_t, bool kVec, bool kSoftplus>
 __device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_row, int pos, int L, float bias,
-                                             float Dv, bool softplus, float (&dl)[kItems], float (&du)[kItems],
-                                             float (&y)[kItems]) {
-    float uv[kItems];
+                                             float Dv, float (&dl)[kItems], float (&du)[kItems], float (&y)[kItems]) {
+    float uv[kItems], raw[kItems], bias_items[kItems];
     load_items<in_t, kVec>(u_row, pos, L, uv);
-    load_items<in_t, kVec>(dl_row, pos, L, dl);
+    load_items<in_t, kVec>(dl_row, pos, L, raw, kSoftplus ? -__builtin_inff() : 0.0f);
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
+    delta_transform<kSoftplus>(raw, bias_items, dl);
 #pragma unroll
     for (int i = 0; i < kItems; ++i) {
-        float d = dl[i] + bias;
-        if (softplus) d = softplus_f32(d);
-        d = (pos + i < L) ? d : 0.0f;     // identity pair past the end of the row (u is 0 there)
-        dl[i] = d;
-        du[i] = d * uv[i];
+        if constexpr (!kSoftplus) dl[i] = (pos + i < L) ? dl[i] : 0.0f;   // identity pair past the end of the row
+        du[i] = dl[i] * uv[i];                                            // u is 0 past the end
         y[i] = Dv * uv[i];
     }
 }
@@ -177,7 +206,7 @@ __device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_r
 // ---- one wavefront per row ------------------------------------------------------------
 // kN > 0: dstate known at compile time, states live in registers.
 // kN == 0: any dstate; the per-wave states live in LDS (2*dstate floats per wave).
-template <typename in_t, typename out_t, int kN, bool kVec>
+template <typename in_t, typename out_t, int kN, bool kVec, bool kSoftplus>
 __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
     const int lane = threadIdx.x & (kWave - 1);
@@ -198,7 +227,6 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     float *x_row = p.x ? p.x + (size_t)row * p.n_chunks * 2 * N : nullptr;
     const float Dv = p.D ? p.D[d] : 0.0f;
     const float bias = p.bias ? p.bias[dg] : 0.0f;
-    const bool softplus = p.softplus != 0;
     const int L = p.L;
 
     float h_reg[kN > 0 ? kN : 1], ap_reg[kN > 0 ? kN : 1], A_reg[kN > 0 ? kN : 1];
@@ -214,7 +242,7 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     for (int pass = 0; pass < n_pass; ++pass) {
         const int pos = pass * kPass + lane * kItems;
         float dl[kItems], du[kItems], y[kItems];
-        load_delta_u<in_t, kVec>(u_row, dl_row, pos, L, bias, Dv, softplus, dl, du, y);
+        load_delta_u<in_t, kVec, kSoftplus>(u_row, dl_row, pos, L, bias, Dv, dl, du, y);
         const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || pass == n_pass - 1);
         float *x_out = chunk_end ? x_row + (size_t)(pass / kPassesPerChunk) * 2 * N : nullptr;
 
@@ -256,7 +284,7 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 // arrives from the previous row.  Per-row constants (A, D, bias, the B/C row) are held for the
 // at most two rows a lane's 8 items can touch (L >= 8) and selected per item; B and C are
 // gathered element-wise (their rows are shared by dim/n_groups channels and stay in L1/L2).
-template <typename in_t, typename out_t, int kN>
+template <typename in_t, typename out_t, int kN, bool kSoftplus>
 __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int rows_per_wave, FastDiv divL,
                                                            FastDiv divDim, FastDiv divDpg) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -274,7 +302,6 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.B), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
-    const bool softplus = p.softplus != 0;
 
     float h_reg[kN];
 #pragma unroll
@@ -284,13 +311,14 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     for (int pass = 0; pass < n_pass; ++pass) {
         const int e0 = pass * kPass + lane * kItems;
         const bool full = e0 + kItems <= n_el;
-        float uv[kItems], dl[kItems];
+        constexpr float kFill = kSoftplus ? -__builtin_inff() : 0.0f;   // see delta_transform
+        float uv[kItems], raw[kItems], dl[kItems];
         if (full) {
             load_items<in_t, true>(u_base, e0, n_el, uv);
-            load_items<in_t, true>(dl_base, e0, n_el, dl);
+            load_items<in_t, true>(dl_base, e0, n_el, raw, kFill);
         } else {
             load_items<in_t, false>(u_base, e0, n_el, uv);
-            load_items<in_t, false>(dl_base, e0, n_el, dl);
+            load_items<in_t, false>(dl_base, e0, n_el, raw, kFill);
         }
 
         // the (at most) two rows this lane touches
@@ -323,20 +351,19 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
 
         // Every item's (row, position) is a real element of B / C even for items past the end of this
         // wavefront's run (row_b is clamped, positions stay below L), so the gathers need no guard.
-        float du[kItems], y[kItems];
+        float du[kItems], y[kItems], bias_items[kItems];
         uint32_t boff[kItems], coff[kItems];
         bool first[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) bias_items[i] = i < k ? bias_a : bias_b;
+        delta_transform<kSoftplus>(raw, bias_items, dl);
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
             const bool in_a = i < k;
             const uint32_t li = in_a ? l0 + i : (uint32_t)(i - k);
-            const bool valid = e0 + i < n_el;
             first[i] = li == 0;
-            float d = dl[i] + (in_a ? bias_a : bias_b);
-            if (softplus) d = softplus_f32(d);
-            d = valid ? d : 0.0f;
-            dl[i] = d;
-            du[i] = valid ? d * uv[i] : 0.0f;
+            if constexpr (!kSoftplus) dl[i] = (e0 + i < n_el) ? dl[i] : 0.0f;
+            du[i] = dl[i] * uv[i];                       // u is 0 past the end of the run
             y[i] = (in_a ? D_a : D_b) * uv[i];
             boff[i] = (in_a ? Boff_a : Boff_b) + li;
             coff[i] = (in_a ? Coff_a : Coff_b) + li;
@@ -376,7 +403,7 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
 // Workgroup = one row.  Per 2048-position chunk wave w takes positions [w*512, w*512+512).
 // LDS: agg[2][N][4] pass totals (double-buffered by chunk parity), state[2][N] chunk-start
 // state (running a-product, h).  One barrier per (chunk, state).
-template <typename in_t, typename out_t, bool kVec>
+template <typename in_t, typename out_t, bool kVec, bool kSoftplus>
 __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
     extern __shared__ __align__(16) float smem[];
     const int N = p.N;
@@ -397,7 +424,6 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
     float *x_row = p.x ? p.x + (size_t)row * p.n_chunks * 2 * N : nullptr;
     const float Dv = p.D ? p.D[d] : 0.0f;
     const float bias = p.bias ? p.bias[dg] : 0.0f;
-    const bool softplus = p.softplus != 0;
     const int L = p.L;
 
     const int n_chunks = (L + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
@@ -405,7 +431,7 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
         const int par = chunk & 1;
         const int pos = chunk * SS2D_SCAN_CHUNK + wave * kPass + lane * kItems;
         float dl[kItems], du[kItems], y[kItems];
-        load_delta_u<in_t, kVec>(u_row, dl_row, pos, L, bias, Dv, softplus, dl, du, y);
+        load_delta_u<in_t, kVec, kSoftplus>(u_row, dl_row, pos, L, bias, Dv, dl, du, y);
         for (int n = 0; n < N; ++n) {
             float Bv[kItems], Cv[kItems];
             load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
@@ -484,13 +510,14 @@ static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
     const uint32_t n_wg = (uint32_t)((n_waves + kWavesPerWg - 1) / kWavesPerWg);
     const FastDiv dL = make_fastdiv((uint32_t)a.L), dDim = make_fastdiv((uint32_t)a.dim),
                   dDpg = make_fastdiv((uint32_t)a.dim_per_group);
+#define SS2D_LAUNCH_FLAT(N, SP) \
+    hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, N, SP>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL, dDim, dDpg)
     if (a.N == 1) {
-        hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, 1>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL,
-                           dDim, dDpg);
+        if (a.softplus) SS2D_LAUNCH_FLAT(1, true); else SS2D_LAUNCH_FLAT(1, false);
     } else {
-        hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, 16>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL,
-                           dDim, dDpg);
+        if (a.softplus) SS2D_LAUNCH_FLAT(16, true); else SS2D_LAUNCH_FLAT(16, false);
     }
+#undef SS2D_LAUNCH_FLAT
     return launch_status();
 }
 
@@ -500,18 +527,25 @@ static int launch_scan(const ScanArgs &a, hipStream_t stream) {
     const bool split_rows = a.L > SS2D_SCAN_CHUNK && a.rows < 16384;
     if (split_rows) {
         const size_t smem = (size_t)(2 * a.N * kWavesPerWg + 2 * a.N) * sizeof(float2);
-        hipLaunchKernelGGL((scan_row4_kernel<in_t, out_t, kVec>), dim3((uint32_t)a.rows), dim3(kBlock), smem, stream, a);
+        if (a.softplus) {
+            hipLaunchKernelGGL((scan_row4_kernel<in_t, out_t, kVec, true>), dim3((uint32_t)a.rows), dim3(kBlock), smem, stream, a);
+        } else {
+            hipLaunchKernelGGL((scan_row4_kernel<in_t, out_t, kVec, false>), dim3((uint32_t)a.rows), dim3(kBlock), smem, stream, a);
+        }
         return launch_status();
     }
     const uint32_t n_wg = (uint32_t)((a.rows + kWavesPerWg - 1) / kWavesPerWg);
+#define SS2D_LAUNCH_ROW(N, SP, SMEM) \
+    hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, N, kVec, SP>), dim3(n_wg), dim3(kBlock), SMEM, stream, a)
     if (a.N == 1) {
-        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 1, kVec>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+        if (a.softplus) SS2D_LAUNCH_ROW(1, true, 0); else SS2D_LAUNCH_ROW(1, false, 0);
     } else if (a.N == 16) {
-        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 16, kVec>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+        if (a.softplus) SS2D_LAUNCH_ROW(16, true, 0); else SS2D_LAUNCH_ROW(16, false, 0);
     } else {
         const size_t smem = (size_t)kWavesPerWg * 2 * a.N * sizeof(float);
-        hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 0, kVec>), dim3(n_wg), dim3(kBlock), smem, stream, a);
+        if (a.softplus) SS2D_LAUNCH_ROW(0, true, smem); else SS2D_LAUNCH_ROW(0, false, smem);
     }
+#undef SS2D_LAUNCH_ROW
     return launch_status();
 }
 
