@@ -21,19 +21,44 @@ constexpr int kMergeTargetElems = 4096;
 
 template <typename T> __device__ __forceinline__ T add_rn(T a, T b) { return from_f32<T>(to_f32(a) + to_f32(b)); }
 
-template <typename T, int kOrder>
+// 16-bit elements travel two to a lane (one 4-byte access) when L is even; kUnroll independent units are
+// loaded before any is combined, so each thread keeps several requests in flight.
+template <typename T, int kVec> struct MergePack { using type = T; };
+template <> struct MergePack<bf16_t, 2> { using type = uint32_t; };
+template <> struct MergePack<f16_t, 2> { using type = uint32_t; };
+
+template <typename T, int kVec>
+__device__ __forceinline__ T unit_get(typename MergePack<T, kVec>::type p, int i) {
+    if constexpr (kVec == 1) return p;
+    else return T{(uint16_t)(p >> (16 * i))};
+}
+template <typename T, int kVec>
+__device__ __forceinline__ typename MergePack<T, kVec>::type unit_make(T a, T b) {
+    if constexpr (kVec == 1) return a;
+    else return (uint32_t)a.bits | ((uint32_t)b.bits << 16);
+}
+// element i of the unit that sits REVERSED in memory
+template <typename T, int kVec>
+__device__ __forceinline__ T unit_get_reversed(typename MergePack<T, kVec>::type p, int i) {
+    return unit_get<T, kVec>(p, kVec - 1 - i);
+}
+
+constexpr int kMergeUnroll = 4;
+
+template <typename T, int kOrder, int kVec>
 __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__restrict__ ys, T *__restrict__ out, int C,
                                                                   int H, int W, int G, int groups_per_image,
                                                                   FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
+    using unit_t = typename MergePack<T, kVec>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *lds = reinterpret_cast<T *>(smem_raw);
 
-    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const uint32_t wg = blockIdx.x;
     const uint32_t b = wg / (uint32_t)groups_per_image;
     const uint32_t c0 = (wg - b * groups_per_image) * (uint32_t)G;
     const uint32_t g = min((uint32_t)G, (uint32_t)C - c0);
     const uint32_t L = divL.d;
-    const uint32_t n = g * L;
+    const uint32_t units = g * L / kVec;           // the host guarantees L % kVec == 0
     const uint32_t Lp = (uint32_t)H * (uint32_t)Wp;
     const uint32_t lds_dir = (uint32_t)G * Lp;     // second LDS plane (left-to-right order only)
 
@@ -44,31 +69,72 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
     const T *y3 = y2 + CL;
     T *o = out + ((size_t)b * C + c0) * L;
 
-    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
-        uint32_t m, t, h, w;
-        divmod(e, divL, m, t);
-        divmod(t, divH, w, h);
-        const T a = y1[e];
-        const T c = y3[m * L + (L - 1 - t)];
-        if (kOrder == SS2D_MERGE_PAIRWISE) {
-            lds[m * Lp + h * Wp + w] = add_rn(a, c);
-        } else {
-            lds[m * Lp + h * Wp + w] = a;
-            lds[lds_dir + m * Lp + h * Wp + w] = c;
+    // column-major operands -> LDS, transposed
+    for (uint32_t base = threadIdx.x; base < units; base += kBlock * kMergeUnroll) {
+        unit_t a[kMergeUnroll], c[kMergeUnroll];
+        uint32_t mm[kMergeUnroll], tt[kMergeUnroll];
+#pragma unroll
+        for (int k = 0; k < kMergeUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q < units) {
+                divmod(q * kVec, divL, mm[k], tt[k]);
+                a[k] = reinterpret_cast<const unit_t *>(y1)[q];
+                c[k] = *reinterpret_cast<const unit_t *>(y3 + mm[k] * L + (L - kVec - tt[k]));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kMergeUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q >= units) continue;
+            uint32_t w, h;
+            divmod(tt[k], divH, w, h);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                const T ai = unit_get<T, kVec>(a[k], i), ci = unit_get_reversed<T, kVec>(c[k], i);
+                const uint32_t li = mm[k] * Lp + h * Wp + w;
+                if (kOrder == SS2D_MERGE_PAIRWISE) {
+                    lds[li] = add_rn(ai, ci);
+                } else {
+                    lds[li] = ai;
+                    lds[lds_dir + li] = ci;
+                }
+                if (++h == (uint32_t)H) { h = 0; ++w; }
+            }
         }
     }
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
-        uint32_t m, r, h, w;
-        divmod(e, divL, m, r);
-        divmod(r, divW, h, w);
-        const T a = y0[e];
-        const T c = y2[m * L + (L - 1 - r)];
-        const uint32_t li = m * Lp + h * Wp + w;
-        if (kOrder == SS2D_MERGE_PAIRWISE) {
-            o[e] = add_rn(add_rn(a, c), lds[li]);
-        } else {
-            o[e] = add_rn(add_rn(add_rn(a, lds[li]), c), lds[lds_dir + li]);
+    // row-major operands + LDS -> out
+    for (uint32_t base = threadIdx.x; base < units; base += kBlock * kMergeUnroll) {
+        unit_t a[kMergeUnroll], c[kMergeUnroll];
+        uint32_t mm[kMergeUnroll], rr[kMergeUnroll];
+#pragma unroll
+        for (int k = 0; k < kMergeUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q < units) {
+                divmod(q * kVec, divL, mm[k], rr[k]);
+                a[k] = reinterpret_cast<const unit_t *>(y0)[q];
+                c[k] = *reinterpret_cast<const unit_t *>(y2 + mm[k] * L + (L - kVec - rr[k]));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kMergeUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q >= units) continue;
+            uint32_t h, w;
+            divmod(rr[k], divW, h, w);
+            T res[kVec];
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                const T ai = unit_get<T, kVec>(a[k], i), ci = unit_get_reversed<T, kVec>(c[k], i);
+                const uint32_t li = mm[k] * Lp + h * Wp + w;
+                if (kOrder == SS2D_MERGE_PAIRWISE) {
+                    res[i] = add_rn(add_rn(ai, ci), lds[li]);
+                } else {
+                    res[i] = add_rn(add_rn(add_rn(ai, lds[li]), ci), lds[lds_dir + li]);
+                }
+                if (++w == (uint32_t)W) { w = 0; ++h; }
+            }
+            reinterpret_cast<unit_t *>(o)[q] = unit_make<T, kVec>(res[0], res[kVec - 1]);
         }
     }
 }
@@ -138,9 +204,21 @@ static int launch_cross_merge(const void *ys, void *out, int B, int C, int H, in
         const int groups = (C + G - 1) / G;
         const int64_t n_wg = (int64_t)B * groups;
         if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-        hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder>), dim3((uint32_t)n_wg), dim3(kBlock),
-                           (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
-                           make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+        bool pairs = false;
+        if constexpr (sizeof(T) == 2) {
+            pairs = (L % 2 == 0) && ((reinterpret_cast<uintptr_t>(ys) | reinterpret_cast<uintptr_t>(out)) % 4 == 0);
+        }
+        if (pairs) {
+            if constexpr (sizeof(T) == 2) {
+                hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 2>), dim3((uint32_t)n_wg), dim3(kBlock),
+                                   (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
+                                   make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+            }
+        } else {
+            hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 1>), dim3((uint32_t)n_wg), dim3(kBlock),
+                               (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
+                               make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+        }
     } else {
         const int tiles_h = (H + kMTile - 1) / kMTile, tiles_w = (W + kMTile - 1) / kMTile;
         const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;

@@ -18,19 +18,39 @@ constexpr int kTilePitch = kTile + 1;
 constexpr int kMapsLdsBytes = 32 * 1024;   // per-workgroup LDS budget of the maps kernel
 constexpr int kMapsTargetElems = 4096;     // elements a maps-workgroup aims to move per direction
 
-template <typename T>
+// kVec elements travel per lane and memory instruction: 2 for 16-bit elements when L is even (a 4-byte lane
+// access moves ~1.3x the bytes per second of a 2-byte one on this GPU), else 1.  kUnroll independent
+// units are loaded before any is stored, so each thread keeps several requests in flight.
+template <typename T, int kVec> struct PackOf { using type = T; };
+template <> struct PackOf<uint16_t, 2> { using type = uint32_t; };
+
+template <typename T, int kVec>
+__device__ __forceinline__ T pack_get(typename PackOf<T, kVec>::type p, int i) {
+    if constexpr (kVec == 1) return p;
+    else return (T)(p >> (16 * i));
+}
+template <typename T, int kVec>
+__device__ __forceinline__ typename PackOf<T, kVec>::type pack_reversed(typename PackOf<T, kVec>::type p) {
+    if constexpr (kVec == 1) return p;
+    else return (p >> 16) | (p << 16);
+}
+
+constexpr int kUnroll = 4;
+
+template <typename T, int kVec>
 __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__restrict__ x, T *__restrict__ y, int C,
                                                                  int H, int W, int G, int groups_per_image,
                                                                  FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
+    using pack_t = typename PackOf<T, kVec>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *lds = reinterpret_cast<T *>(smem_raw);
 
-    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const uint32_t wg = blockIdx.x;
     const uint32_t b = wg / (uint32_t)groups_per_image;
     const uint32_t c0 = (wg - b * groups_per_image) * (uint32_t)G;
     const uint32_t g = min((uint32_t)G, (uint32_t)C - c0);
     const uint32_t L = divL.d;
-    const uint32_t n = g * L;
+    const uint32_t units = g * L / kVec;             // the host guarantees L % kVec == 0
     const uint32_t Lp = (uint32_t)H * (uint32_t)Wp;
 
     const size_t CL = (size_t)C * L;
@@ -39,24 +59,54 @@ __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__rest
     T *y1 = y0 + CL;
     T *y2 = y1 + CL;
     T *y3 = y2 + CL;
+    const pack_t *xin_p = reinterpret_cast<const pack_t *>(xin);
+    pack_t *y0_p = reinterpret_cast<pack_t *>(y0);
+    pack_t *y1_p = reinterpret_cast<pack_t *>(y1);
 
-    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
-        uint32_t m, j, h, w;
-        divmod(e, divL, m, j);
-        divmod(j, divW, h, w);
-        const T v = xin[e];
-        lds[m * Lp + h * Wp + w] = v;
-        y0[e] = v;
-        y2[m * L + (L - 1 - j)] = v;
+    for (uint32_t base = threadIdx.x; base < units; base += kBlock * kUnroll) {
+        pack_t v[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q < units) v[k] = xin_p[q];
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q >= units) continue;
+            uint32_t m, j, h, w;
+            divmod(q * kVec, divL, m, j);
+            divmod(j, divW, h, w);
+            y0_p[q] = v[k];
+            *reinterpret_cast<pack_t *>(y2 + m * L + (L - kVec - j)) = pack_reversed<T, kVec>(v[k]);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                lds[m * Lp + h * Wp + w] = pack_get<T, kVec>(v[k], i);
+                if (++w == (uint32_t)W) { w = 0; ++h; }
+            }
+        }
     }
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e < n; e += kBlock) {
-        uint32_t m, t, h, w;
-        divmod(e, divL, m, t);
-        divmod(t, divH, w, h);          // t = w*H + h
-        const T v = lds[m * Lp + h * Wp + w];
-        y1[e] = v;
-        y3[m * L + (L - 1 - t)] = v;
+    for (uint32_t base = threadIdx.x; base < units; base += kBlock * kUnroll) {
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q >= units) continue;
+            uint32_t m, t, h, w;
+            divmod(q * kVec, divL, m, t);
+            divmod(t, divH, w, h);          // t = w*H + h
+            pack_t v;
+            if constexpr (kVec == 1) {
+                v = lds[m * Lp + h * Wp + w];
+            } else {
+                const uint32_t lo = lds[m * Lp + h * Wp + w];
+                if (++h == (uint32_t)H) { h = 0; ++w; }
+                const uint32_t hi = lds[m * Lp + h * Wp + w];
+                v = lo | (hi << 16);
+            }
+            y1_p[q] = v;
+            *reinterpret_cast<pack_t *>(y3 + m * L + (L - kVec - t)) = pack_reversed<T, kVec>(v);
+        }
     }
 }
 
@@ -114,9 +164,22 @@ static int launch_cross_scan(const void *x, void *y, int B, int C, int H, int W,
         const int groups = (C + G - 1) / G;
         const int64_t n_wg = (int64_t)B * groups;
         if (n_wg > 0x7fffffff || (int64_t)G * L > 0x7fffffff) return SS2D_ENOTSUP;
-        hipLaunchKernelGGL(cross_scan_maps_kernel<T>, dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds), stream,
-                           (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
-                           make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+        // 16-bit elements go two to a lane when every map starts on a 4-byte boundary
+        bool pairs = false;
+        if constexpr (sizeof(T) == 2) {
+            pairs = (L % 2 == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 4 == 0);
+        }
+        if (pairs) {
+            if constexpr (sizeof(T) == 2) {
+                hipLaunchKernelGGL((cross_scan_maps_kernel<T, 2>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds),
+                                   stream, (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
+                                   make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+            }
+        } else {
+            hipLaunchKernelGGL((cross_scan_maps_kernel<T, 1>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds),
+                               stream, (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
+                               make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+        }
     } else {
         const int tiles_h = (H + kTile - 1) / kTile, tiles_w = (W + kTile - 1) / kTile;
         const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;

@@ -41,34 +41,66 @@ struct ScanArgs {
 };
 
 // ---- 8-wide loads / stores ------------------------------------------------------------
+// Eight consecutive elements of a row as they sit in registers before widening: 4 dwords for 16-bit
+// types, 8 for fp32.  Keeping loads in this form lets a pass issue the NEXT pass's loads before it
+// starts computing (software prefetch), which is what keeps enough bytes in flight per wavefront.
+template <typename T> struct Raw8 { uint32_t w[sizeof(T) * 2]; };
+
 // Items at positions >= L come back as `fill`.
 template <typename T, bool kVec>
-__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems],
-                                           float fill = 0.0f) {
+__device__ __forceinline__ Raw8<T> load_raw(const T *__restrict__ row, int pos, int L, float fill = 0.0f) {
+    Raw8<T> r;
     if constexpr (kVec) {
         // the host guarantees 16-byte alignment and L % (16/sizeof(T)) == 0, so a vector is either
         // entirely inside the row or entirely outside
         if constexpr (sizeof(T) == 2) {
             const uint32_t fill2 = (uint32_t)from_f32<T>(fill).bits * 0x10001u;
-            uint4 raw = make_uint4(fill2, fill2, fill2, fill2);
-            if (pos < L) raw = *reinterpret_cast<const uint4 *>(row + pos);
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+            uint4 v = make_uint4(fill2, fill2, fill2, fill2);
+            if (pos < L) v = *reinterpret_cast<const uint4 *>(row + pos);
+            r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z; r.w[3] = v.w;
+        } else {
+            const uint32_t f = f32_to_bits(fill);
+            uint4 lo = make_uint4(f, f, f, f), hi = lo;
+            if (pos < L) lo = *reinterpret_cast<const uint4 *>(row + pos);
+            if (pos + 4 < L) hi = *reinterpret_cast<const uint4 *>(row + pos + 4);
+            r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w;
+            r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
+        }
+    } else {
+        if constexpr (sizeof(T) == 2) {
+            const uint32_t fb = from_f32<T>(fill).bits;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                v[2 * i] = to_f32(T{(uint16_t)(w[i] & 0xffffu)});
-                v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
+                const uint32_t lo = (pos + 2 * i < L) ? row[pos + 2 * i].bits : fb;
+                const uint32_t hi = (pos + 2 * i + 1 < L) ? row[pos + 2 * i + 1].bits : fb;
+                r.w[i] = lo | (hi << 16);
             }
         } else {
-            float4 lo = make_float4(fill, fill, fill, fill), hi = lo;
-            if (pos < L) lo = *reinterpret_cast<const float4 *>(row + pos);
-            if (pos + 4 < L) hi = *reinterpret_cast<const float4 *>(row + pos + 4);
-            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
-            v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) r.w[i] = f32_to_bits((pos + i < L) ? row[pos + i] : fill);
+        }
+    }
+    return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void unpack_raw(const Raw8<T> &r, float (&v)[kItems]) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = to_f32(T{(uint16_t)(r.w[i] & 0xffffu)});
+            v[2 * i + 1] = to_f32(T{(uint16_t)(r.w[i] >> 16)});
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) v[i] = (pos + i < L) ? to_f32(row[pos + i]) : fill;
+        for (int i = 0; i < kItems; ++i) v[i] = bits_to_f32(r.w[i]);
     }
+}
+
+template <typename T, bool kVec>
+__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems],
+                                           float fill = 0.0f) {
+    unpack_raw<T>(load_raw<T, kVec>(row, pos, L, fill), v);
 }
 
 template <typename T, bool kVec>
@@ -186,21 +218,37 @@ __device__ __forceinline__ void scan_state_pass(const float (&dl)[kItems], const
     for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
 }
 
-template <typename in_t, bool kVec, bool kSoftplus>
-__device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_row, int pos, int L, float bias,
-                                             float Dv, float (&dl)[kItems], float (&du)[kItems], float (&y)[kItems]) {
+// The fill the delta loads use past the end of a row (see delta_transform).
+template <bool kSoftplus> __device__ __forceinline__ constexpr float delta_fill() {
+    return kSoftplus ? -__builtin_inff() : 0.0f;
+}
+
+// Widen u and delta, apply bias/softplus, and start the output with the D*u skip term.  `n_valid` is how many
+// of the 8 items lie inside the row.
+template <typename in_t, bool kSoftplus>
+__device__ __forceinline__ void prepare_delta_u(const Raw8<in_t> &u_raw, const Raw8<in_t> &dl_raw, int n_valid,
+                                                float bias, float Dv, float (&dl)[kItems], float (&du)[kItems],
+                                                float (&y)[kItems]) {
     float uv[kItems], raw[kItems], bias_items[kItems];
-    load_items<in_t, kVec>(u_row, pos, L, uv);
-    load_items<in_t, kVec>(dl_row, pos, L, raw, kSoftplus ? -__builtin_inff() : 0.0f);
+    unpack_raw<in_t>(u_raw, uv);
+    unpack_raw<in_t>(dl_raw, raw);
 #pragma unroll
     for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
     delta_transform<kSoftplus>(raw, bias_items, dl);
 #pragma unroll
     for (int i = 0; i < kItems; ++i) {
-        if constexpr (!kSoftplus) dl[i] = (pos + i < L) ? dl[i] : 0.0f;   // identity pair past the end of the row
+        if constexpr (!kSoftplus) dl[i] = (i < n_valid) ? dl[i] : 0.0f;   // identity pair past the end of the row
         du[i] = dl[i] * uv[i];                                            // u is 0 past the end
         y[i] = Dv * uv[i];
     }
+}
+
+template <typename in_t, bool kVec, bool kSoftplus>
+__device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_row, int pos, int L, float bias,
+                                             float Dv, float (&dl)[kItems], float (&du)[kItems], float (&y)[kItems]) {
+    const Raw8<in_t> u_raw = load_raw<in_t, kVec>(u_row, pos, L);
+    const Raw8<in_t> dl_raw = load_raw<in_t, kVec>(dl_row, pos, L, delta_fill<kSoftplus>());
+    prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
 }
 
 // ---- one wavefront per row ------------------------------------------------------------
@@ -211,7 +259,10 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // With several states the B/C rows (shared by dim/n_groups channels) are worth keeping in one XCD's L2, so
+    // each XCD gets a contiguous range of rows.  With one state they are 1 % of the traffic and the hardware's
+    // round-robin order, which keeps all active rows in one moving window of memory, measured faster.
+    const uint32_t wg = kN == 1 ? blockIdx.x : xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int row = (int)(wg * kWavesPerWg) + wave;
     if (row >= p.rows) return;           // whole wavefront leaves; this kernel has no barrier
 
@@ -238,11 +289,32 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
         for (int n = lane; n < N; n += kWave) { st[2 * n] = 1.0f; st[2 * n + 1] = 0.0f; }
     }
 
+    // Software prefetch: the loads of pass p+1 (u, delta, and B/C when there is a single state) are issued
+    // before pass p computes, so every wavefront keeps two passes of input in flight.
+    constexpr bool kPrefetchBC = kN == 1;
     const int n_pass = (L + kPass - 1) / kPass;
+    Raw8<in_t> u_next = load_raw<in_t, kVec>(u_row, lane * kItems, L);
+    Raw8<in_t> dl_next = load_raw<in_t, kVec>(dl_row, lane * kItems, L, delta_fill<kSoftplus>());
+    Raw8<in_t> B_next, C_next;
+    if constexpr (kPrefetchBC) {
+        B_next = load_raw<in_t, kVec>(B_row, lane * kItems, L);
+        C_next = load_raw<in_t, kVec>(C_row, lane * kItems, L);
+    }
     for (int pass = 0; pass < n_pass; ++pass) {
         const int pos = pass * kPass + lane * kItems;
+        const Raw8<in_t> u_raw = u_next, dl_raw = dl_next;
+        Raw8<in_t> B_raw, C_raw;
+        if constexpr (kPrefetchBC) { B_raw = B_next; C_raw = C_next; }
+        if (pass + 1 < n_pass) {
+            u_next = load_raw<in_t, kVec>(u_row, pos + kPass, L);
+            dl_next = load_raw<in_t, kVec>(dl_row, pos + kPass, L, delta_fill<kSoftplus>());
+            if constexpr (kPrefetchBC) {
+                B_next = load_raw<in_t, kVec>(B_row, pos + kPass, L);
+                C_next = load_raw<in_t, kVec>(C_row, pos + kPass, L);
+            }
+        }
         float dl[kItems], du[kItems], y[kItems];
-        load_delta_u<in_t, kVec, kSoftplus>(u_row, dl_row, pos, L, bias, Dv, dl, du, y);
+        prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
         const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || pass == n_pass - 1);
         float *x_out = chunk_end ? x_row + (size_t)(pass / kPassesPerChunk) * 2 * N : nullptr;
 
@@ -250,8 +322,13 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 #pragma unroll
             for (int n = 0; n < kN; ++n) {
                 float Bv[kItems], Cv[kItems], a_tot, h_tot;
-                load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
-                load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                if constexpr (kPrefetchBC) {
+                    unpack_raw<in_t>(B_raw, Bv);
+                    unpack_raw<in_t>(C_raw, Cv);
+                } else {
+                    load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+                    load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                }
                 scan_state_pass(dl, du, Bv, Cv, A_reg[n], h_reg[n], y, a_tot, h_tot);
                 h_reg[n] = fmaf(a_tot, h_reg[n], h_tot);
                 ap_reg[n] *= a_tot;
