@@ -88,13 +88,12 @@ def kernel_lines(reps):
 def cpu_baseline(seconds_budget=30.0):
     """Reference torch CPU path through the same model, fp32, on a bounded sample."""
     import torch
-    from oracle.ss2d_core_ref import RefSS2D
-    from vmamba_amd.vssm import vmamba_tiny_s1l8
+    from oracle.ss2d_core_ref import reference_vmamba_tiny
     cores = os.cpu_count() or 1
     cores = min(cores, 16)
     torch.set_num_threads(cores)
     torch.manual_seed(0)
-    model = vmamba_tiny_s1l8(ss2d_cls=RefSS2D).eval()
+    model = reference_vmamba_tiny().eval()
     batch = 16
     x = torch.randn(batch, 3, 224, 224)
     with torch.no_grad():

@@ -118,6 +118,24 @@ typedef struct ss2d_scan_params {
 
 int ss2d_selective_scan_fwd(const ss2d_scan_params *params, void *stream);
 
+/*
+ * LayerNorm over the channel axis, the step after CrossMerge (out_norm) and the block norms of the model.
+ * Replaces the torch calls of LayerNorm2d.forward (classification/models/vmamba.py:52-57: permute,
+ * F.layer_norm, permute) and of nn.LayerNorm on (B,H,W,C) activations, including the transposition
+ * forward_core does before out_norm in channel-last models (vmamba.py:642-644).
+ *   y = (x - mean) * rsqrt(var + eps) * weight + bias, mean / biased var over the C channels, fp32 statistics
+ *   and arithmetic for every I/O type; weight / bias (C) may be NULL.
+ * Supported (in, weight, out) dtype triples: (f32,f32,f32) (f32,f32,bf16) (f32,bf16,bf16) (f32,bf16,f32)
+ * (bf16,bf16,bf16) (bf16,f32,bf16) (f32,f16,f16) (f16,f16,f16) (f16,f32,f16); others return SS2D_ENOTSUP.
+ *
+ * ss2d_layer_norm:    x, y (rows, C) contiguous.
+ * ss2d_layer_norm_cf: x (B,C,L) contiguous, channel-first; y (B,L,C) if out_channel_last else (B,C,L).
+ */
+int ss2d_layer_norm(const void *x, const void *weight, const void *bias, void *y, int64_t rows, int C, float eps,
+                    int in_dtype, int w_dtype, int out_dtype, void *stream);
+int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void *y, int B, int C, int L, float eps,
+                       int in_dtype, int w_dtype, int out_dtype, int out_channel_last, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,23 @@ def cross_merge_left_to_right(ys):
     return ((y[:, 0] + t(y[:, 1])) + y[:, 2].flip(-1)) + t(y[:, 3].flip(-1))
 
 
+def layer_norm_rows(x, weight, bias, eps=1e-5, out_dtype=None):
+    """nn.LayerNorm over the last axis, statistics in fp32 (what torch does for 16-bit inputs as well)."""
+    y = F.layer_norm(x.float(), (x.shape[-1],), None if weight is None else weight.float(),
+                     None if bias is None else bias.float(), eps)
+    return y.to(out_dtype or x.dtype)
+
+
+def layer_norm_cf(x, weight, bias, eps=1e-5, out_channel_last=False, out_dtype=None):
+    """LayerNorm2d (classification/models/vmamba.py:52-57): permute to channel-last, layer_norm, permute back;
+    with ``out_channel_last`` the result stays channel-last, which is forward_core's out_norm step in
+    channel-last models (vmamba.py:642-644)."""
+    nd = x.dim()
+    to_cl = (0, *range(2, nd), 1)
+    y = layer_norm_rows(x.permute(*to_cl), weight, bias, eps, out_dtype)
+    return y.contiguous() if out_channel_last else y.permute(0, nd - 1, *range(1, nd - 1)).contiguous()
+
+
 def selective_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
                    return_last_state=False):
     dtype_in = u.dtype

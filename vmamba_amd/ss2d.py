@@ -22,6 +22,7 @@ import torch.nn.functional as F
 
 from .csm import cross_merge_fn, cross_scan_fn
 from .csms6s import selective_scan_fn
+from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip
 
 
 class Linear2d(nn.Linear):
@@ -37,13 +38,16 @@ class Linear2d(nn.Linear):
         return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
 
-class LayerNorm2d(nn.LayerNorm):
-    """LayerNorm over the channel axis of a (B, C, H, W) tensor (vmamba.py:52-57)."""
+class HipLayers:
+    """The layer classes the blocks are built from: LayerNorm on the HIP kernels of this package."""
+    LayerNorm = LayerNorm
+    LayerNorm2d = LayerNorm2d
 
-    def forward(self, x):
-        y = F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight.to(x.dtype),
-                         self.bias.to(x.dtype), self.eps)
-        return y.permute(0, 3, 1, 2)
+    @staticmethod
+    def out_norm(norm, y, channel_first, dtype):
+        """out_norm of forward_core on the merged channel-first map y (B, D, H, W), returned in the block's
+        layout and dtype: one kernel reads (B, D, L) and writes the normalised (B, D, L) or (B, L, D)."""
+        return layer_norm_cf_hip(y, norm.weight, norm.bias, norm.eps, out_channel_last=not channel_first, out_dtype=dtype)
 
 
 def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.1, dt_init_floor=1e-4, k_group=4):
@@ -67,9 +71,11 @@ class SS2D(nn.Module):
     """
 
     def __init__(self, d_model=96, d_state=1, ssm_ratio=1.0, dt_rank="auto", d_conv=3, conv_bias=False, bias=False,
-                 disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4, channel_first=True):
+                 disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4, channel_first=True,
+                 layers=HipLayers):
         super().__init__()
         self.channel_first = channel_first
+        self.layers = layers
         Linear = Linear2d if channel_first else nn.Linear
         self.k_group = 4
         self.d_model, self.d_state = int(d_model), int(d_state)
@@ -84,18 +90,23 @@ class SS2D(nn.Module):
                                     groups=self.d_inner, bias=conv_bias)
         x_proj = [nn.Linear(self.d_inner, self.dt_rank + 2 * self.d_state, bias=False) for _ in range(self.k_group)]
         self.x_proj_weight = nn.Parameter(torch.stack([t.weight for t in x_proj], dim=0))   # (K, R+2N, D)
-        self.out_norm = LayerNorm2d(self.d_inner) if channel_first else nn.LayerNorm(self.d_inner)
+        self.out_norm = layers.LayerNorm2d(self.d_inner) if channel_first else layers.LayerNorm(self.d_inner)
         self.out_proj = Linear(self.d_inner, self.d_model, bias=bias)
         self.A_logs, self.Ds, self.dt_projs_weight, self.dt_projs_bias = init_dt_A_D(
             self.d_state, self.dt_rank, self.d_inner, dt_scale, dt_min, dt_max, dt_init_floor, self.k_group)
 
     def project(self, xs):
-        """x_proj / dt_proj as grouped 1x1 conv1d (vmamba.py:605-608).  xs: (B, K, D, L)."""
+        """x_proj and dt_proj (vmamba.py:605-615) as two batched PyTorch-ROCm GEMMs.  xs: (B, K, D, L).
+
+        The reference offers a grouped-conv1d and an einsum spelling of the same contraction; on this stack
+        a broadcast ``matmul`` (one strided-batched GEMM over B*K) is several times faster than either.
+        Returns dts (B, K*D, L) and B, C as strided views (B, K, N, L) of the projection output.
+        """
         B, K, D, L = xs.shape
         R, N = self.dt_rank, self.d_state
-        x_dbl = F.conv1d(xs.view(B, K * D, L), self.x_proj_weight.view(-1, D, 1), groups=K)
-        dts, Bs, Cs = torch.split(x_dbl.view(B, K, -1, L), [R, N, N], dim=2)
-        dts = F.conv1d(dts.contiguous().view(B, K * R, L), self.dt_projs_weight.view(K * D, R, 1), groups=K)
+        x_dbl = torch.matmul(self.x_proj_weight.unsqueeze(0), xs)                    # (B, K, R+2N, L)
+        dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
+        dts = torch.matmul(self.dt_projs_weight.unsqueeze(0), dts).view(B, K * D, L)  # (B, K, D, L)
         return dts, Bs, Cs
 
     def forward_core(self, x):
@@ -111,11 +122,7 @@ class SS2D(nn.Module):
 
     def finish_core(self, y, B, D, H, W, dtype):
         """out_norm on the merged (B, D, L) map, in the block's layout (vmamba.py:641-646)."""
-        if self.channel_first:
-            return self.out_norm(y.view(B, D, H, W)).to(dtype)
-        y = y.view(B, D, H * W).transpose(1, 2).contiguous().view(B, H, W, D)
-        return F.layer_norm(y, (D,), self.out_norm.weight.to(y.dtype), self.out_norm.bias.to(y.dtype),
-                            self.out_norm.eps).to(dtype)
+        return self.layers.out_norm(self.out_norm, y.view(B, D, H, W), self.channel_first, dtype)
 
     def forward(self, x):
         x = self.in_proj(x)

@@ -4,13 +4,14 @@ Layer order and shapes follow VSSM / VSSBlock of classification/models/vmamba.py
 the ``vmamba_tiny_s1l8`` recipe (:1717-1728): patch-embed v2, downsample v3, depths 2/2/8/2, dims
 96/192/384/768, d_state 1, ssm_ratio 1, forward type v05_noz, MLP ratio 4.  As in the reference the
 same weights run in two activation layouts: ``channel_first=True`` ("ln2d": (B,C,H,W), 1x1 convs,
-LayerNorm2d) and ``channel_first=False`` ("ln": (B,H,W,C), nn.Linear, nn.LayerNorm).  Everything
-outside the SS2D core is stock torch; drop-path is the identity at inference.
+LayerNorm2d) and ``channel_first=False`` ("ln": (B,H,W,C), nn.Linear, nn.LayerNorm).  The norm
+layers come from ``layers`` (default: this package's HIP LayerNorm kernels); convolutions, the projection and
+MLP GEMMs and activations are stock torch; drop-path is the identity at inference.
 """
 import torch
 import torch.nn as nn
 
-from .ss2d import SS2D, LayerNorm2d, Linear2d
+from .ss2d import SS2D, HipLayers, Linear2d
 
 
 class Permute(nn.Module):
@@ -43,11 +44,13 @@ class Mlp(nn.Module):
 
 
 class VSSBlock(nn.Module):
-    def __init__(self, dim, d_state=1, ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, **ss2d_kwargs):
+    def __init__(self, dim, d_state=1, ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, layers=HipLayers,
+                 **ss2d_kwargs):
         super().__init__()
-        Norm = LayerNorm2d if channel_first else nn.LayerNorm
+        Norm = layers.LayerNorm2d if channel_first else layers.LayerNorm
         self.norm = Norm(dim)
-        self.op = ss2d_cls(d_model=dim, d_state=d_state, ssm_ratio=ssm_ratio, channel_first=channel_first, **ss2d_kwargs)
+        self.op = ss2d_cls(d_model=dim, d_state=d_state, ssm_ratio=ssm_ratio, channel_first=channel_first, layers=layers,
+                           **ss2d_kwargs)
         self.norm2 = Norm(dim)
         self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
@@ -58,23 +61,23 @@ class VSSBlock(nn.Module):
 
 class VSSM(nn.Module):
     def __init__(self, in_chans=3, num_classes=1000, depths=(2, 2, 8, 2), dims=(96, 192, 384, 768), d_state=1,
-                 ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, **ss2d_kwargs):
+                 ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, layers=HipLayers, **ss2d_kwargs):
         super().__init__()
         cf = channel_first
-        Norm = LayerNorm2d if cf else nn.LayerNorm
+        Norm = layers.LayerNorm2d if cf else layers.LayerNorm
         d0 = dims[0]
         self.patch_embed = nn.Sequential(
             nn.Conv2d(in_chans, d0 // 2, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0 // 2), _to_cf(cf),
             nn.GELU(),
             nn.Conv2d(d0 // 2, d0, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0))
-        layers = []
+        stages = []
         for i, (depth, dim) in enumerate(zip(depths, dims)):
-            blocks = [VSSBlock(dim, d_state, ssm_ratio, mlp_ratio, ss2d_cls, cf, **ss2d_kwargs) for _ in range(depth)]
+            blocks = [VSSBlock(dim, d_state, ssm_ratio, mlp_ratio, ss2d_cls, cf, layers, **ss2d_kwargs) for _ in range(depth)]
             down = (nn.Sequential(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
                                   Norm(dims[i + 1]))
                     if i + 1 < len(dims) else nn.Identity())
-            layers.append(nn.Sequential(*blocks, down))
-        self.layers = nn.ModuleList(layers)
+            stages.append(nn.Sequential(*blocks, down))
+        self.layers = nn.ModuleList(stages)
         self.classifier = nn.Sequential(Norm(dims[-1]), _to_cf(cf), nn.AdaptiveAvgPool2d(1), nn.Flatten(1),
                                         nn.Linear(dims[-1], num_classes))
         self.apply(self._init_weights)
