@@ -136,6 +136,16 @@ int ss2d_layer_norm(const void *x, const void *weight, const void *bias, void *y
 int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void *y, int B, int C, int L, float eps,
                        int in_dtype, int w_dtype, int out_dtype, int out_channel_last, void *stream);
 
+/*
+ * Depthwise 3x3 convolution (stride 1, zero padding 1) + optional bias + optional SiLU: the two ops in front of
+ * forward_core in SS2Dv2.forwardv2 (classification/models/vmamba.py:654-658: permute to channel-first,
+ * self.conv2d (groups = d_inner), self.act), fused with the layout change.
+ *   x (B,H,W,D) if in_channel_last else (B,D,H,W); weight (D,1,3,3); bias (D) or NULL; all of `dtype`
+ *   y (B,D,H,W), channel-first.  fp32 accumulation; the convolution result is rounded to `dtype` before SiLU.
+ */
+int ss2d_dwconv3x3_silu(const void *x, const void *weight, const void *bias, void *y, int B, int D, int H, int W,
+                        int dtype, int in_channel_last, int apply_silu, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

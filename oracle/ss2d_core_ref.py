@@ -34,6 +34,14 @@ class TorchLayers:
         return F.layer_norm(y, (D,), norm.weight.to(y.dtype), norm.bias.to(y.dtype), norm.eps).to(dtype)
 
 
+    @staticmethod
+    def conv_act(conv2d, x, channel_first):
+        # vmamba.py:654-658
+        if not channel_first:
+            x = x.permute(0, 3, 1, 2).contiguous()
+        return F.silu(conv2d(x) if conv2d is not None else x)
+
+
 class RefSS2D(SS2D):
     def __init__(self, *args, **kwargs):
         kwargs.setdefault("layers", TorchLayers)

@@ -58,6 +58,14 @@ def layer_norm_cf(x, weight, bias, eps=1e-5, out_channel_last=False, out_dtype=N
     return y.contiguous() if out_channel_last else y.permute(0, nd - 1, *range(1, nd - 1)).contiguous()
 
 
+def dwconv3x3_silu(x, weight, bias=None, in_channel_last=False, apply_silu=True):
+    """vmamba.py:654-658: to channel-first, depthwise conv2d (k=3, pad=1), SiLU -- as separate torch ops in x.dtype."""
+    if in_channel_last:
+        x = x.permute(0, 3, 1, 2)
+    y = F.conv2d(x, weight.to(x.dtype), None if bias is None else bias.to(x.dtype), padding=1, groups=x.shape[1])
+    return F.silu(y) if apply_silu else y
+
+
 def selective_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
                    return_last_state=False):
     dtype_in = u.dtype

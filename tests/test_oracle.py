@@ -276,3 +276,29 @@ def test_layer_norm_cf_is_permute_norm_permute():
     for h in range(3):
         for wi in range(5):
             assert torch.allclose(cl[1, h, wi], torch_ref.layer_norm_rows(x[1, :, h, wi][None], w, b)[0], atol=1e-6)
+
+
+# ------------------------------------------------------------- depthwise conv
+def test_dwconv_against_brute_force():
+    g = torch.Generator().manual_seed(33)
+    B, D, H, W = 2, 3, 4, 5
+    x, w, b = torch.randn(B, D, H, W, generator=g), torch.randn(D, 1, 3, 3, generator=g), torch.randn(D, generator=g)
+    want = torch.zeros(B, D, H, W, dtype=torch.float64)
+    for bi in range(B):
+        for d in range(D):
+            for h in range(H):
+                for wi in range(W):
+                    acc = float(b[d])
+                    for kh in range(3):
+                        for kw in range(3):
+                            hh, ww = h + kh - 1, wi + kw - 1
+                            if 0 <= hh < H and 0 <= ww < W:
+                                acc += float(w[d, 0, kh, kw]) * float(x[bi, d, hh, ww])
+                    want[bi, d, h, wi] = acc / (1.0 + math.exp(-acc))
+    got = torch_ref.dwconv3x3_silu(x, w, b)
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-6)
+    got_cl = torch_ref.dwconv3x3_silu(x.permute(0, 2, 3, 1).contiguous(), w, b, in_channel_last=True)
+    assert torch.allclose(got_cl, got, rtol=1e-6, atol=1e-6)
+    # identity kernel (centre tap 1) without SiLU returns the input
+    ident = torch.zeros(D, 1, 3, 3); ident[:, 0, 1, 1] = 1.0
+    assert torch.equal(torch_ref.dwconv3x3_silu(x, ident, None, apply_silu=False), x)

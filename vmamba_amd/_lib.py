@@ -15,7 +15,7 @@ SCAN_CHUNK = 2048
 ABI_VERSION = 1
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
-           "ss2d_layer_norm", "ss2d_layer_norm_cf")
+           "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu")
 
 
 class ScanParams(ctypes.Structure):
@@ -64,6 +64,8 @@ def lib():
         L.ss2d_layer_norm_cf.restype = ctypes.c_int
         L.ss2d_layer_norm_cf.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 + [ctypes.c_float]
                                          + [ctypes.c_int] * 4 + [ctypes.c_void_p])
+        L.ss2d_dwconv3x3_silu.restype = ctypes.c_int
+        L.ss2d_dwconv3x3_silu.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_void_p]
         if L.ss2d_abi_version() != ABI_VERSION:
             raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L

@@ -1,0 +1,196 @@
+// Depthwise 3x3 convolution (+ bias) + SiLU: the step in front of the SS2D core
+// (classification/models/vmamba.py:654-658: permute to channel-first, conv2d(groups=d_inner, k=3, pad=1), act).
+//
+//   x  (B,H,W,D) channel-last (the layout in_proj = nn.Linear produces) or (B,D,H,W) channel-first
+//   w  (D,1,3,3), bias (D) or NULL
+//   y  (B,D,H,W) channel-first, always: what CrossScan reads
+//   y = silu(round(conv(x) + bias)), products and sums in fp32; the conv result is rounded to the tensor dtype
+//   before SiLU because the reference runs conv2d and SiLU as two ops.
+//
+// HBM-bound (one read, one write).  The channel-last variant fuses the layout change: a workgroup owns 64
+// consecutive positions x 32 channels; each lane convolves 8 channels at one position from nine 16-byte
+// channel-vector loads (neighbouring positions re-use the same lines out of L1/L2), parks its results in LDS and
+// the tile is written back transposed, 16 bytes per lane along the position axis.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+constexpr int kDwPos = 64;           // positions per workgroup tile
+constexpr int kDwCh = 32;            // channels per workgroup tile
+constexpr int kDwPitch = kDwPos + 8; // LDS row pitch in elements: keeps 16-byte alignment, spreads banks
+
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+
+template <typename T> __device__ __forceinline__ void unpack8(const uint4 raw, float (&v)[8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = to_f32(T{(uint16_t)(w[i] & 0xffffu)});
+        v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
+    }
+}
+
+// 16-bit element types, D % 8 == 0, 16-byte aligned tensors (host-checked).
+template <typename T, bool kSilu>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_kernel(const T *__restrict__ x, const T *__restrict__ weight,
+                                                                 const T *__restrict__ bias, T *__restrict__ y, int D,
+                                                                 int H, int W, int pos_tiles, int ch_tiles, FastDiv divW) {
+    __shared__ __align__(16) uint16_t tile[kDwCh * kDwPitch];
+    uint32_t wg = blockIdx.x;
+    const uint32_t ct = wg % ch_tiles; wg /= ch_tiles;
+    const uint32_t pt = wg % pos_tiles;
+    const uint32_t b = wg / pos_tiles;
+    const int L = H * W;
+    const int r0 = (int)pt * kDwPos;
+    const int p = threadIdx.x / 4, cv = threadIdx.x % 4;
+    const int c0 = (int)ct * kDwCh + cv * 8;            // this lane's 8 channels
+    const int r = r0 + p;
+
+    if (r < L && c0 < D) {
+        uint32_t h, w;
+        divmod((uint32_t)r, divW, h, w);
+        // 72 weights of the 8 channels: 9 consecutive 16-byte vectors
+        float wt[8][9];
+        {
+            const uint4 *wp = reinterpret_cast<const uint4 *>(weight + (size_t)c0 * 9);
+            float flat[72];
+#pragma unroll
+            for (int k = 0; k < 9; ++k) {
+                float t8[8];
+                unpack8<T>(wp[k], t8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) flat[k * 8 + i] = t8[i];
+            }
+#pragma unroll
+            for (int ci = 0; ci < 8; ++ci)
+#pragma unroll
+                for (int t = 0; t < 9; ++t) wt[ci][t] = flat[ci * 9 + t];
+        }
+        float acc[8];
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci) acc[ci] = 0.0f;
+        const T *xb = x + (size_t)b * L * D;
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int hh = (int)h + kh - 1, ww = (int)w + kw - 1;
+                if (hh >= 0 && hh < H && ww >= 0 && ww < W) {
+                    float xv[8];
+                    unpack8<T>(*reinterpret_cast<const uint4 *>(xb + ((size_t)hh * W + ww) * D + c0), xv);
+#pragma unroll
+                    for (int ci = 0; ci < 8; ++ci) acc[ci] = fmaf(wt[ci][kh * 3 + kw], xv[ci], acc[ci]);
+                }
+            }
+        }
+        float bv[8];
+        if (bias) unpack8<T>(*reinterpret_cast<const uint4 *>(bias + c0), bv);
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci) {
+            float v = acc[ci] + (bias ? bv[ci] : 0.0f);
+            T o = from_f32<T>(v);
+            if (kSilu) o = from_f32<T>(silu_f32(to_f32(o)));
+            tile[(cv * 8 + ci) * kDwPitch + p] = o.bits;
+        }
+    }
+    __syncthreads();
+    // write back: lane -> (channel = tid / 8, eight consecutive positions)
+    const int c = threadIdx.x / 8, chunk = threadIdx.x % 8;
+    const int cg = (int)ct * kDwCh + c;
+    const int rr = r0 + chunk * 8;
+    if (cg < D && rr < L) {
+        T *yo = y + ((size_t)b * D + cg) * L + rr;
+        const uint16_t *src = tile + c * kDwPitch + chunk * 8;
+        if (rr + 8 <= L && (L % 8) == 0) {
+            *reinterpret_cast<uint4 *>(yo) = *reinterpret_cast<const uint4 *>(src);
+        } else {
+            for (int i = 0; i < 8 && rr + i < L; ++i) yo[i] = T{src[i]};
+        }
+    }
+}
+
+// Generic variant: any element type, either input layout, one output element per lane (lanes along W).
+template <typename T, bool kInChannelLast, bool kSilu>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_generic_kernel(const T *__restrict__ x, const T *__restrict__ weight,
+                                                                   const T *__restrict__ bias, T *__restrict__ y, int D, int H,
+                                                                   int W, int64_t total, FastDiv divW, FastDiv divH,
+                                                                   FastDiv divD) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;     // over (b, d, h, w)
+    if (idx >= total) return;
+    const int64_t L = (int64_t)H * W;
+    const uint32_t map = (uint32_t)(idx / L);
+    const uint32_t r = (uint32_t)(idx - (int64_t)map * L);
+    uint32_t b, d, h, w;
+    divmod(map, divD, b, d);
+    divmod(r, divW, h, w);
+    (void)divH;
+    float acc = 0.0f;
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+            const int hh = (int)h + kh - 1, ww = (int)w + kw - 1;
+            if (hh >= 0 && hh < H && ww >= 0 && ww < W) {
+                const size_t off = kInChannelLast ? (((size_t)b * H + hh) * W + ww) * D + d
+                                                  : (((size_t)b * D + d) * H + hh) * W + ww;
+                acc = fmaf(to_f32(weight[(size_t)d * 9 + kh * 3 + kw]), to_f32(x[off]), acc);
+            }
+        }
+    if (bias) acc += to_f32(bias[d]);
+    T o = from_f32<T>(acc);
+    if (kSilu) o = from_f32<T>(silu_f32(to_f32(o)));
+    y[idx] = o;
+}
+
+template <typename T>
+static int launch_dwconv(const void *x, const void *w, const void *bias, void *y, int B, int D, int H, int W,
+                         int in_channel_last, int apply_silu, hipStream_t stream) {
+    const int64_t L = (int64_t)H * W;
+    auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if constexpr (sizeof(T) == 2) {
+        if (in_channel_last && D % 8 == 0 && al16(x) && al16(w) && al16(y) && (!bias || al16(bias))) {
+            const int pos_tiles = (int)((L + kDwPos - 1) / kDwPos), ch_tiles = (D + kDwCh - 1) / kDwCh;
+            const int64_t n_wg = (int64_t)B * pos_tiles * ch_tiles;
+            if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+            if (apply_silu) {
+                hipLaunchKernelGGL((dwconv3x3_cl2cf_kernel<T, true>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                                   (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, pos_tiles, ch_tiles,
+                                   make_fastdiv((uint32_t)W));
+            } else {
+                hipLaunchKernelGGL((dwconv3x3_cl2cf_kernel<T, false>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                                   (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, pos_tiles, ch_tiles,
+                                   make_fastdiv((uint32_t)W));
+            }
+            return launch_status();
+        }
+    }
+    const int64_t total = (int64_t)B * D * L;
+    const int64_t n_wg = (total + kBlock - 1) / kBlock;
+    if (n_wg > 0x7fffffff || (int64_t)B * D > 0x7fffffff) return SS2D_ENOTSUP;
+#define SS2D_DW_GENERIC(CL, SILU)                                                                                       \
+    hipLaunchKernelGGL((dwconv3x3_generic_kernel<T, CL, SILU>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,         \
+                       (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, total, make_fastdiv((uint32_t)W), \
+                       make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)D))
+    if (in_channel_last) { if (apply_silu) SS2D_DW_GENERIC(true, true); else SS2D_DW_GENERIC(true, false); }
+    else { if (apply_silu) SS2D_DW_GENERIC(false, true); else SS2D_DW_GENERIC(false, false); }
+#undef SS2D_DW_GENERIC
+    return launch_status();
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_dwconv3x3_silu(const void *x, const void *weight, const void *bias, void *y, int B, int D, int H, int W,
+                                   int dtype, int in_channel_last, int apply_silu, void *stream) {
+    using namespace ss2d;
+    if (B < 0 || D < 0 || H < 0 || W < 0) return SS2D_EINVAL;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (B == 0 || D == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!x || !weight || !y) return SS2D_EINVAL;
+    if ((int64_t)H * W > 0x3fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case SS2D_F32: return launch_dwconv<float>(x, weight, bias, y, B, D, H, W, in_channel_last, apply_silu, s);
+        case SS2D_BF16: return launch_dwconv<bf16_t>(x, weight, bias, y, B, D, H, W, in_channel_last, apply_silu, s);
+        default: return launch_dwconv<f16_t>(x, weight, bias, y, B, D, H, W, in_channel_last, apply_silu, s);
+    }
+}

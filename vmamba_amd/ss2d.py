@@ -22,6 +22,7 @@ import torch.nn.functional as F
 
 from .csm import cross_merge_fn, cross_scan_fn
 from .csms6s import selective_scan_fn
+from .conv import dwconv3x3_silu_hip
 from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip
 
 
@@ -48,6 +49,16 @@ class HipLayers:
         """out_norm of forward_core on the merged channel-first map y (B, D, H, W), returned in the block's
         layout and dtype: one kernel reads (B, D, L) and writes the normalised (B, D, L) or (B, L, D)."""
         return layer_norm_cf_hip(y, norm.weight, norm.bias, norm.eps, out_channel_last=not channel_first, out_dtype=dtype)
+
+    @staticmethod
+    def conv_act(conv2d, x, channel_first):
+        """Depthwise conv + SiLU on the in_proj output x ((B,D,H,W) if channel_first else (B,H,W,D)); returns the
+        channel-first (B,D,H,W) input of forward_core (vmamba.py:654-658).  ``conv2d`` None means no conv."""
+        if conv2d is not None and conv2d.kernel_size == (3, 3) and conv2d.padding == (1, 1) and conv2d.stride == (1, 1):
+            return dwconv3x3_silu_hip(x, conv2d.weight, conv2d.bias, in_channel_last=not channel_first, apply_silu=True)
+        if not channel_first:
+            x = x.permute(0, 3, 1, 2).contiguous()
+        return F.silu(conv2d(x) if conv2d is not None else x)
 
 
 def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.1, dt_init_floor=1e-4, k_group=4):
@@ -130,11 +141,7 @@ class SS2D(nn.Module):
         if not self.disable_z:
             x, z = x.chunk(2, dim=(1 if self.channel_first else -1))
             z = self.act(z)
-        if not self.channel_first:
-            x = x.permute(0, 3, 1, 2).contiguous()
-        if self.with_dconv:
-            x = self.conv2d(x)
-        x = self.act(x)
+        x = self.layers.conv_act(self.conv2d if self.with_dconv else None, x, self.channel_first)   # (B, D, H, W)
         y = self.forward_core(x)
         if z is not None:
             y = y * z
