@@ -91,3 +91,13 @@ def test_host_api_rejects_cpu_tensors_and_unsupported_modes():
         va.selective_scan_fn(u, u, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8))
     with pytest.raises(NotImplementedError):
         va.selective_scan_fn(u, u, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8), backend="torch")
+
+
+def test_torch_extension_shim_loads_and_validates_on_cpu():
+    import torch
+    from vmamba_amd import oflex_ext
+    ext = oflex_ext.load()
+    assert hasattr(ext, "fwd") and hasattr(ext, "bwd")
+    z = torch.zeros(1, 4, 8)
+    with pytest.raises(RuntimeError):       # CPU tensors are refused before anything touches a GPU
+        ext.fwd(z, z, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8), None, None, True, 1, True)

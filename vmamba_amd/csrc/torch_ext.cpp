@@ -1,0 +1,108 @@
+// selective_scan_cuda_oflex -- the PyTorch extension module the reference probes for
+// (classification/models/csms6s.py:9-14) and calls as
+//     out, x, *rest = selective_scan_cuda_oflex.fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, 1, oflex)
+// (csms6s.py:81).  This is a thin shim: the argument checks and output allocation of the reference's
+// selective_scan_fwd (kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:143-231),
+// then one call into the C ABI of libss2d_hip.so on PyTorch's current HIP stream.  No kernel lives here.
+// `bwd` exists so that attribute lookups succeed, and raises: this build is the inference forward.
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPGuard.h>
+#include <torch/extension.h>
+
+#include <vector>
+
+#include "../../include/ss2d_hip.h"
+
+#define CHECK_SHAPE(x, ...) \
+    TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
+
+static int dtype_code(at::ScalarType t) {
+    switch (t) {
+        case at::ScalarType::Float: return SS2D_F32;
+        case at::ScalarType::BFloat16: return SS2D_BF16;
+        case at::ScalarType::Half: return SS2D_F16;
+        default: return -1;
+    }
+}
+
+static std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
+                                                  const at::Tensor &B, const at::Tensor &C,
+                                                  const c10::optional<at::Tensor> &D_,
+                                                  const c10::optional<at::Tensor> &delta_bias_, bool delta_softplus,
+                                                  int nrows, bool out_float) {
+    (void)nrows;  // accepted and ignored, as in the reference (selective_scan_oflex.cpp:224-226)
+    const auto input_type = u.scalar_type();
+    TORCH_CHECK(dtype_code(input_type) >= 0, "selective_scan_fwd not implemented for input type '", toString(input_type), "'");
+    TORCH_CHECK(A.scalar_type() == at::ScalarType::Float, "A must be float32");
+    TORCH_CHECK(delta.scalar_type() == input_type && B.scalar_type() == input_type && C.scalar_type() == input_type,
+                "delta, B, C must have the dtype of u");
+    TORCH_CHECK(u.is_cuda() && delta.is_cuda() && A.is_cuda() && B.is_cuda() && C.is_cuda(), "inputs must be GPU tensors");
+    TORCH_CHECK(u.dim() == 3 && delta.dim() == 3 && A.dim() == 2 && B.dim() == 4 && C.dim() == 4, "bad tensor ranks");
+    TORCH_CHECK(u.stride(-1) == 1 || u.size(-1) == 1);
+    TORCH_CHECK(delta.stride(-1) == 1 || delta.size(-1) == 1);
+
+    const int batch_size = u.size(0), dim = u.size(1), seqlen = u.size(2);
+    const int dstate = A.size(1), n_groups = B.size(1), delta_dim = delta.size(1);
+    TORCH_CHECK(dim % n_groups == 0, "dims should be dividable by n_groups");
+    TORCH_CHECK(dim % delta_dim == 0, "dims should be dividable by delta_dim");
+    TORCH_CHECK(dstate <= 256, "selective_scan only supports state dimension <= 256");
+    CHECK_SHAPE(u, batch_size, dim, seqlen);
+    CHECK_SHAPE(delta, batch_size, delta_dim, seqlen);
+    CHECK_SHAPE(A, dim, dstate);
+    CHECK_SHAPE(B, batch_size, n_groups, dstate, seqlen);
+    TORCH_CHECK(B.stride(-1) == 1 || B.size(-1) == 1);
+    CHECK_SHAPE(C, batch_size, n_groups, dstate, seqlen);
+    TORCH_CHECK(C.stride(-1) == 1 || C.size(-1) == 1);
+
+    at::Tensor D, delta_bias;
+    if (D_.has_value()) {
+        D = D_.value();
+        TORCH_CHECK(D.scalar_type() == at::ScalarType::Float && D.is_cuda());
+        TORCH_CHECK(D.stride(-1) == 1 || D.size(-1) == 1);
+        CHECK_SHAPE(D, dim);
+    }
+    if (delta_bias_.has_value()) {
+        delta_bias = delta_bias_.value();
+        TORCH_CHECK(delta_bias.scalar_type() == at::ScalarType::Float && delta_bias.is_cuda());
+        TORCH_CHECK(delta_bias.stride(-1) == 1 || delta_bias.size(-1) == 1);
+        CHECK_SHAPE(delta_bias, delta_dim);
+    }
+
+    const int n_chunks = (seqlen + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
+    at::Tensor out = torch::empty({batch_size, dim, seqlen}, u.options().dtype(out_float ? at::ScalarType::Float : input_type));
+    at::Tensor x = torch::empty({batch_size, dim, n_chunks, dstate * 2}, u.options().dtype(at::ScalarType::Float));
+
+    ss2d_scan_params p = {};
+    p.batch = batch_size; p.dim = dim; p.seqlen = seqlen; p.dstate = dstate; p.n_groups = n_groups; p.delta_dim = delta_dim;
+    p.in_dtype = dtype_code(input_type);
+    p.out_dtype = dtype_code(out.scalar_type());
+    p.delta_softplus = delta_softplus ? 1 : 0;
+    p.u = u.data_ptr(); p.delta = delta.data_ptr(); p.A = A.data_ptr(); p.B = B.data_ptr(); p.C = C.data_ptr();
+    p.D = D.defined() ? D.data_ptr() : nullptr;
+    p.delta_bias = delta_bias.defined() ? delta_bias.data_ptr() : nullptr;
+    p.out = out.data_ptr(); p.x = x.data_ptr();
+    p.u_batch_stride = u.stride(0); p.u_d_stride = u.stride(1);
+    p.delta_batch_stride = delta.stride(0); p.delta_d_stride = delta.stride(1);
+    p.A_d_stride = A.stride(0); p.A_dstate_stride = A.stride(1);
+    p.B_batch_stride = B.stride(0); p.B_group_stride = B.stride(1); p.B_dstate_stride = B.stride(2);
+    p.C_batch_stride = C.stride(0); p.C_group_stride = C.stride(1); p.C_dstate_stride = C.stride(2);
+    p.out_batch_stride = out.stride(0); p.out_d_stride = out.stride(1);
+
+    // Otherwise the kernel would be launched on device 0
+    const c10::hip::HIPGuard device_guard(u.device());
+    hipStream_t stream = at::hip::getCurrentHIPStream().stream();
+    const int rc = ss2d_selective_scan_fwd(&p, (void *)stream);
+    TORCH_CHECK(rc == SS2D_OK, "ss2d_selective_scan_fwd: ", ss2d_strerror(rc), " (status ", rc, ")");
+    return {out, x};
+}
+
+static std::vector<at::Tensor> selective_scan_bwd(py::args, py::kwargs) {
+    TORCH_CHECK(false, "selective_scan_cuda_oflex.bwd: this build implements the inference forward only");
+    return {};
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.doc() = "MI355X-native selective-scan forward behind the reference's extension interface";
+    m.def("fwd", &selective_scan_fwd, "Selective scan forward (HIP, gfx950)");
+    m.def("bwd", &selective_scan_bwd, "not built: inference-only");
+}
