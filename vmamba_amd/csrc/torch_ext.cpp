@@ -6,7 +6,8 @@
 // then one call into the C ABI of libss2d_hip.so on PyTorch's current HIP stream.  No kernel lives here.
 // `bwd` exists so that attribute lookups succeed, and raises: this build is the inference forward.
 #include <ATen/hip/HIPContext.h>
-#include <c10/hip/HIPGuard.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <vector>
@@ -88,9 +89,10 @@ static std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at:
     p.C_batch_stride = C.stride(0); p.C_group_stride = C.stride(1); p.C_dstate_stride = C.stride(2);
     p.out_batch_stride = out.stride(0); p.out_d_stride = out.stride(1);
 
-    // Otherwise the kernel would be launched on device 0
-    const c10::hip::HIPGuard device_guard(u.device());
-    hipStream_t stream = at::hip::getCurrentHIPStream().stream();
+    // Otherwise the kernel would be launched on device 0.  PyTorch-ROCm presents HIP devices under the "cuda"
+    // device type, so the guard and the stream getter are the ones that understand that naming.
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(u.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const int rc = ss2d_selective_scan_fwd(&p, (void *)stream);
     TORCH_CHECK(rc == SS2D_OK, "ss2d_selective_scan_fwd: ", ss2d_strerror(rc), " (status ", rc, ")");
     return {out, x};
