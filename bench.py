@@ -124,6 +124,9 @@ def main():
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the model: time the SS2D-core kernels at the four stage shapes plus a 1 GiB "
                          "device copy (the known-size kernel profiler counters are scaled against)")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the forward as one captured HIP graph (validated against eager) instead of eager "
+                         "launches; measured equal within noise at batch 128, so eager is the default")
     ap.add_argument("--layout", choices=["channel_first", "channel_last"], default="channel_last",
                     help="activation layout of the harness outside the SS2D core (same weights, same math)")
     args = ap.parse_args()
@@ -151,18 +154,55 @@ def main():
     model = vmamba_tiny_s1l8(channel_first=(args.layout == "channel_first")).to(dev).bfloat16().eval()
     x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
 
+    def capture_forward():
+        """Capture one forward into a HIP graph and check replays against the eager result (replays interleaved
+        with eager work and synchronisations); returns (graph, static_output) or None if anything differs."""
+        eager = model(x).float()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                model(x)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(x)
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            if not torch.equal(out.float(), eager):
+                return None
+            model(x)                       # eager work between replays
+            torch.cuda.synchronize()
+        return graph, out
+
     with torch.no_grad():
+        model(x)
+        torch.cuda.synchronize()
+        log("first forward done")
+        graph = None
+        if args.graph:
+            try:
+                captured = capture_forward()
+            except Exception as e:          # capture is an optimisation of the launch path, never a requirement
+                log(f"graph capture failed ({type(e).__name__}: {e}); timing eager launches")
+                captured = None
+            if captured is None:
+                log("graph replay did not reproduce the eager result; timing eager launches")
+            else:
+                graph = captured[0]
+        step = graph.replay if graph is not None else (lambda: model(x))
         for i in range(args.warmup):
-            model(x)
-            if i == 0:
-                torch.cuda.synchronize()
-                log("first forward done")
+            step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            model(x)
+            step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+    launch_mode = "one captured HIP graph per forward" if graph is not None else "eager launches"
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     log(f"VMamba-T bs{args.batch}: {ms:.2f} ms/step, {value:.0f} img/s")
@@ -183,7 +223,7 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
-                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks; SS2D core on HIP kernels"},
+                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}; SS2D core on HIP kernels"},
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels,
     }))
 
