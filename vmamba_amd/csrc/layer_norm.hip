@@ -136,7 +136,8 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_generic_kernel(const i
 }
 
 // ---- channel-first input ------------------------------------------------------------------------
-// x (B,C,L).  A workgroup takes kCfTile (32, 16 or 8: whatever keeps the tile under 48 KB) consecutive positions of one image and all C channels: the tile is read
+// LDS-tile variant (rows wider than the register variant below covers).
+// x (B,C,L).  A workgroup takes kCfTile consecutive positions of one image and all C channels: the tile is read
 // lane-contiguously along L (each channel row gives a kCfTile-element segment), parked in LDS as fp32
 // [C][kCfTile+1], reduced per position (a group of 256/kCfTile lanes walks the channels of one position; the odd
 // pitch keeps those column reads conflict-free), normalised in LDS, and written out lane-contiguously in the
@@ -195,6 +196,94 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_kernel(const in_t *__res
     }
 }
 
+// Register variant of the channel-first LayerNorm (C up to kG*kVPT channels).  Threads are laid out positions x
+// groups: lane -> position (so every channel row is read as one contiguous run of kTP elements), group g holds
+// channels g, g+kG, g+2kG, ... of its position in registers.  The two reductions cross the kG groups through a
+// few floats of LDS.  Channel-first output goes straight back from registers (contiguous along positions);
+// channel-last output is turned round through an LDS tile [position][channel] and copied out row by row.
+template <typename in_t, typename w_t, typename out_t, bool kOutChannelLast, int kTP, int kG, int kVPT>
+__global__ __launch_bounds__(kBlock) void layer_norm_cf_reg_kernel(const in_t *__restrict__ x, const w_t *__restrict__ weight,
+                                                                   const w_t *__restrict__ bias, out_t *__restrict__ y, int C,
+                                                                   int L, int tiles_per_image, int Cp, float eps) {
+    static_assert(kTP * kG == kBlock, "one thread per (position, group)");
+    extern __shared__ __align__(16) unsigned char ln_smem[];
+    __shared__ float red[2][kG][kTP];
+    const uint32_t b = blockIdx.x / tiles_per_image;
+    const int l0 = (int)(blockIdx.x - b * tiles_per_image) * kTP;
+    const int p = threadIdx.x % kTP, g = threadIdx.x / kTP;
+    const int l = l0 + p;
+    const bool valid = l < L;
+    const in_t *xb = x + (size_t)b * C * L + l;
+
+    float v[kVPT];
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+        const int c = g + i * kG;
+        v[i] = (valid && c < C) ? to_f32(xb[(size_t)c * L]) : 0.0f;
+        s += v[i];
+    }
+    red[0][g][p] = s;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kG; ++j) tot += red[0][j][p];
+    const float mean = tot / (float)C;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kVPT; ++i) {
+        const float d = v[i] - mean;
+        q = (g + i * kG < C) ? fmaf(d, d, q) : q;
+    }
+    red[1][g][p] = q;
+    __syncthreads();
+    float qt = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kG; ++j) qt += red[1][j][p];
+    const float rstd = rsqrtf(qt / (float)C + eps);
+
+    if constexpr (!kOutChannelLast) {
+        out_t *yb = y + (size_t)b * C * L + l;
+#pragma unroll
+        for (int i = 0; i < kVPT; ++i) {
+            const int c = g + i * kG;
+            if (valid && c < C) {
+                float t = (v[i] - mean) * rstd;
+                if (weight) t *= to_f32(weight[c]);
+                if (bias) t += to_f32(bias[c]);
+                yb[(size_t)c * L] = from_f32<out_t>(t);
+            }
+        }
+    } else {
+        out_t *ot = reinterpret_cast<out_t *>(ln_smem);          // [kTP][Cp]
+#pragma unroll
+        for (int i = 0; i < kVPT; ++i) {
+            const int c = g + i * kG;
+            if (c < C) {
+                float t = (v[i] - mean) * rstd;
+                if (weight) t *= to_f32(weight[c]);
+                if (bias) t += to_f32(bias[c]);
+                ot[p * Cp + c] = from_f32<out_t>(t);
+            }
+        }
+        __syncthreads();
+        const int nl = min(kTP, L - l0);
+        out_t *yb = y + ((size_t)b * L + l0) * C;
+        if (sizeof(out_t) == 2 && (C % 2) == 0) {
+            const int half = C / 2;                                // 4-byte units per row
+            for (int idx = threadIdx.x; idx < nl * half; idx += kBlock) {
+                const int pp = idx / half, cc = (idx - pp * half) * 2;
+                *reinterpret_cast<uint32_t *>(yb + (size_t)pp * C + cc) = *reinterpret_cast<const uint32_t *>(ot + pp * Cp + cc);
+            }
+        } else {
+            for (int idx = threadIdx.x; idx < nl * C; idx += kBlock) {
+                const int pp = idx / C, cc = idx - pp * C;
+                yb[(size_t)pp * C + cc] = ot[pp * Cp + cc];
+            }
+        }
+    }
+}
+
 // ---- host side ----------------------------------------------------------------------------------
 static bool ln_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -246,14 +335,35 @@ static int launch_ln_cf_tile(const void *x, const void *w, const void *b, void *
     return launch_status();
 }
 
+template <typename in_t, typename w_t, typename out_t, int kTP, int kG, int kVPT>
+static int launch_ln_cf_reg(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
+                            int out_channel_last, hipStream_t stream) {
+    const int tiles = (L + kTP - 1) / kTP;
+    const int64_t n_wg = (int64_t)B * tiles;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    // LDS pitch of the turn-round tile: lanes walk positions, so consecutive rows must land in different banks
+    int Cp = sizeof(out_t) == 2 ? ((C + 1) & ~1) : (C | 1);
+    if (sizeof(out_t) == 2 && (Cp / 2) % 2 == 0) Cp += 2;
+    if (out_channel_last) {
+        const size_t smem = (size_t)kTP * Cp * sizeof(out_t);
+        hipLaunchKernelGGL((layer_norm_cf_reg_kernel<in_t, w_t, out_t, true, kTP, kG, kVPT>), dim3((uint32_t)n_wg), dim3(kBlock),
+                           smem, stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+    } else {
+        hipLaunchKernelGGL((layer_norm_cf_reg_kernel<in_t, w_t, out_t, false, kTP, kG, kVPT>), dim3((uint32_t)n_wg), dim3(kBlock),
+                           0, stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+    }
+    return launch_status();
+}
+
 template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
                         int out_channel_last, hipStream_t stream) {
-    constexpr size_t kBudget = 48 * 1024;
-    if ((size_t)C * 33 * sizeof(float) <= kBudget)
-        return launch_ln_cf_tile<in_t, w_t, out_t, 32>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
-    if ((size_t)C * 17 * sizeof(float) <= kBudget)
-        return launch_ln_cf_tile<in_t, w_t, out_t, 16>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if (C <= 96) return launch_ln_cf_reg<in_t, w_t, out_t, 64, 4, 24>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if (C <= 192) return launch_ln_cf_reg<in_t, w_t, out_t, 64, 4, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if (C <= 384) return launch_ln_cf_reg<in_t, w_t, out_t, 32, 8, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if (C <= 768) return launch_ln_cf_reg<in_t, w_t, out_t, 16, 16, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if (C <= 1536) return launch_ln_cf_reg<in_t, w_t, out_t, 8, 32, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    constexpr size_t kBudget = 48 * 1024;      // very wide rows: the LDS-tile kernel
     if ((size_t)C * 9 * sizeof(float) <= kBudget)
         return launch_ln_cf_tile<in_t, w_t, out_t, 8>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     return SS2D_ENOTSUP;

@@ -106,28 +106,47 @@ class SS2D(nn.Module):
         self.A_logs, self.Ds, self.dt_projs_weight, self.dt_projs_bias = init_dt_A_D(
             self.d_state, self.dt_rank, self.d_inner, dt_scale, dt_min, dt_max, dt_init_floor, self.k_group)
 
-    def project(self, xs):
-        """x_proj and dt_proj (vmamba.py:605-615) as two batched PyTorch-ROCm GEMMs.  xs: (B, K, D, L).
+    def _inference_constants(self, batch):
+        """Tensors that depend only on the parameters (and the batch size): A = -exp(A_logs), fp32 D and dt bias
+        (vmamba.py:619-623) and the projection weights repeated over the batch so each projection is ONE
+        strided-batched GEMM over B*K problems.  Recomputed whenever autograd is on or a parameter changed."""
+        params = (self.A_logs, self.Ds, self.dt_projs_bias, self.x_proj_weight, self.dt_projs_weight)
+        key = (batch, torch.is_grad_enabled(), tuple((p._version, p.data_ptr(), p.dtype, p.device) for p in params))
+        cached = getattr(self, "_const_cache", None)
+        if cached is not None and cached[0] == key:
+            return cached[1]
+        K = self.k_group
+        consts = dict(
+            As=-self.A_logs.float().exp(), Ds=self.Ds.float(), dt_bias=self.dt_projs_bias.reshape(-1).float(),
+            Wx=self.x_proj_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, -1, self.d_inner).contiguous(),
+            Wdt=self.dt_projs_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, self.d_inner, -1).contiguous())
+        if not torch.is_grad_enabled():
+            self._const_cache = (key, consts)
+        return consts
+
+    def project(self, xs, consts=None):
+        """x_proj and dt_proj (vmamba.py:605-615) as two strided-batched PyTorch-ROCm GEMMs.  xs: (B, K, D, L).
 
         The reference offers a grouped-conv1d and an einsum spelling of the same contraction; on this stack
-        a broadcast ``matmul`` (one strided-batched GEMM over B*K) is several times faster than either.
+        a batched matmul over the B*K (image, direction) problems is several times faster than either.
         Returns dts (B, K*D, L) and B, C as strided views (B, K, N, L) of the projection output.
         """
         B, K, D, L = xs.shape
         R, N = self.dt_rank, self.d_state
-        x_dbl = torch.matmul(self.x_proj_weight.unsqueeze(0), xs)                    # (B, K, R+2N, L)
+        consts = consts or self._inference_constants(B)
+        x_dbl = torch.bmm(consts["Wx"], xs.view(B * K, D, L)).view(B, K, R + 2 * N, L)
         dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
-        dts = torch.matmul(self.dt_projs_weight.unsqueeze(0), dts).view(B, K * D, L)  # (B, K, D, L)
+        dts = torch.bmm(consts["Wdt"], dts.reshape(B * K, R, L)).view(B, K * D, L)
         return dts, Bs, Cs
 
     def forward_core(self, x):
         B, D, H, W = x.shape
         K, L = self.k_group, H * W
+        consts = self._inference_constants(B)
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
-        dts, Bs, Cs = self.project(xs)
-        As = -self.A_logs.float().exp()
-        ys = selective_scan_fn(xs.view(B, K * D, L), dts, As, Bs, Cs, self.Ds.float(),
-                               self.dt_projs_bias.view(-1).float(), True, True)                # fp32 (oflex)
+        dts, Bs, Cs = self.project(xs, consts)
+        ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
+                               True, True)                                                     # fp32 (oflex)
         y = cross_merge_fn(ys.view(B, K, D, H, W), in_channel_first=True, out_channel_first=True, scans=0)
         return self.finish_core(y, B, D, H, W, x.dtype)
 
