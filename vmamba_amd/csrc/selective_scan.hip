@@ -289,30 +289,33 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
         for (int n = lane; n < N; n += kWave) { st[2 * n] = 1.0f; st[2 * n + 1] = 0.0f; }
     }
 
-    // Software prefetch: the loads of pass p+1 (u, delta, and B/C when there is a single state) are issued
-    // before pass p computes, so every wavefront keeps two passes of input in flight.
-    constexpr bool kPrefetchBC = kN == 1;
+    // Burst loads: with a single state the inputs of kBurst consecutive passes (u, delta, B, C: 4 x 1 KB each per
+    // wavefront and pass) are requested together before any of them is processed.  A row is then fetched in two
+    // or three long runs instead of seven short visits, which the memory system serves measurably faster, and
+    // each wavefront keeps several KB in flight.
+    constexpr bool kBurstBC = kN == 1;
+    constexpr int kBurst = kN == 1 ? 4 : 1;
     const int n_pass = (L + kPass - 1) / kPass;
-    Raw8<in_t> u_next = load_raw<in_t, kVec>(u_row, lane * kItems, L);
-    Raw8<in_t> dl_next = load_raw<in_t, kVec>(dl_row, lane * kItems, L, delta_fill<kSoftplus>());
-    Raw8<in_t> B_next, C_next;
-    if constexpr (kPrefetchBC) {
-        B_next = load_raw<in_t, kVec>(B_row, lane * kItems, L);
-        C_next = load_raw<in_t, kVec>(C_row, lane * kItems, L);
-    }
-    for (int pass = 0; pass < n_pass; ++pass) {
-        const int pos = pass * kPass + lane * kItems;
-        const Raw8<in_t> u_raw = u_next, dl_raw = dl_next;
-        Raw8<in_t> B_raw, C_raw;
-        if constexpr (kPrefetchBC) { B_raw = B_next; C_raw = C_next; }
-        if (pass + 1 < n_pass) {
-            u_next = load_raw<in_t, kVec>(u_row, pos + kPass, L);
-            dl_next = load_raw<in_t, kVec>(dl_row, pos + kPass, L, delta_fill<kSoftplus>());
-            if constexpr (kPrefetchBC) {
-                B_next = load_raw<in_t, kVec>(B_row, pos + kPass, L);
-                C_next = load_raw<in_t, kVec>(C_row, pos + kPass, L);
+    for (int pass0 = 0; pass0 < n_pass; pass0 += kBurst) {
+        Raw8<in_t> u_burst[kBurst], dl_burst[kBurst], B_burst[kBurst], C_burst[kBurst];
+#pragma unroll
+        for (int s = 0; s < kBurst; ++s) {
+            const int pos_s = (pass0 + s) * kPass + lane * kItems;
+            u_burst[s] = load_raw<in_t, kVec>(u_row, pos_s, L);
+            dl_burst[s] = load_raw<in_t, kVec>(dl_row, pos_s, L, delta_fill<kSoftplus>());
+            if constexpr (kBurstBC) {
+                B_burst[s] = load_raw<in_t, kVec>(B_row, pos_s, L);
+                C_burst[s] = load_raw<in_t, kVec>(C_row, pos_s, L);
             }
         }
+#pragma unroll
+        for (int s = 0; s < kBurst; ++s) {
+        const int pass = pass0 + s;
+        if (pass >= n_pass) break;
+        const int pos = pass * kPass + lane * kItems;
+        const Raw8<in_t> u_raw = u_burst[s], dl_raw = dl_burst[s];
+        Raw8<in_t> B_raw, C_raw;
+        if constexpr (kBurstBC) { B_raw = B_burst[s]; C_raw = C_burst[s]; }
         float dl[kItems], du[kItems], y[kItems];
         prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
         const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || pass == n_pass - 1);
@@ -322,7 +325,7 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 #pragma unroll
             for (int n = 0; n < kN; ++n) {
                 float Bv[kItems], Cv[kItems], a_tot, h_tot;
-                if constexpr (kPrefetchBC) {
+                if constexpr (kBurstBC) {
                     unpack_raw<in_t>(B_raw, Bv);
                     unpack_raw<in_t>(C_raw, Cv);
                 } else {
@@ -349,6 +352,7 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
             }
         }
         store_items<out_t, kVec>(o_row, pos, L, y);
+        }
     }
 }
 
