@@ -362,12 +362,48 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 // are dense, so consecutive rows are adjacent in memory and the 16-byte lane vectors stay
 // aligned because rows_per_wave is a multiple of 8).  The recurrence restarts at every row
 // simply by forcing a = 0 at a row's first position: the pair (0, b) discards whatever state
-// arrives from the previous row.  Per-row constants (A, D, bias, the B/C row) are held for the
-// at most two rows a lane's 8 items can touch (L >= 8) and selected per item; B and C are
-// gathered element-wise (their rows are shared by dim/n_groups channels and stay in L1/L2).
-template <typename in_t, typename out_t, int kN, bool kSoftplus>
+// arrives from the previous row.
+//
+// kGran = gcd(L, 8) (further reduced by what the B/C strides and alignment allow) is the
+// granularity at which rows can change inside a lane's 8 items: the items form 8/kGran groups
+// that each lie in one row, so the per-row constants (A, D, bias, the B/C row) are selected per
+// group, not per item, and B/C are gathered kGran elements at a time through buffer
+// descriptors (their rows are shared by dim/n_groups channels and stay in L1/L2).  A lane
+// touches at most two rows (L >= 8); with kGran == 8 exactly one.
+template <typename T, int kGran>
+__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, float (&v)[kGran]) {
+    const int byte_off = (int)(elem_offset * (uint32_t)sizeof(T));
+    constexpr int kBytes = kGran * (int)sizeof(T);
+    uint32_t w[kBytes >= 4 ? kBytes / 4 : 1];
+    if constexpr (kBytes == 2) {
+        w[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_off, 0, 0);
+    } else if constexpr (kBytes == 4) {
+        w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_off, 0, 0);
+    } else if constexpr (kBytes == 8) {
+        const auto t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, byte_off, 0, 0);
+        w[0] = t[0]; w[1] = t[1];
+    } else if constexpr (kBytes == 16) {
+        const auto t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
+        w[0] = t[0]; w[1] = t[1]; w[2] = t[2]; w[3] = t[3];
+    } else {
+        static_assert(kBytes == 32, "8 fp32 elements");
+        const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
+        const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, 0, 0);
+        w[0] = t0[0]; w[1] = t0[1]; w[2] = t0[2]; w[3] = t0[3]; w[4] = t1[0]; w[5] = t1[1]; w[6] = t1[2]; w[7] = t1[3];
+    }
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < kGran; ++i) v[i] = to_f32(T{(uint16_t)(w[i / 2] >> (16 * (i % 2)))});
+    } else {
+#pragma unroll
+        for (int i = 0; i < kGran; ++i) v[i] = bits_to_f32(w[i]);
+    }
+}
+
+template <typename in_t, typename out_t, int kN, bool kSoftplus, int kGran>
 __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int rows_per_wave, FastDiv divL,
                                                            FastDiv divDim, FastDiv divDpg) {
+    constexpr int kGroups = kItems / kGran;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
@@ -378,8 +414,7 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     const int n_el = n_rows * L;
     const in_t *u_base = reinterpret_cast<const in_t *>(p.u) + r0 * L;
     const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + r0 * L;
-    // B and C are gathered through buffer descriptors: a 32-bit byte offset per lane, no 64-bit address math,
-    // and hardware range checking (an offset past the extent reads 0).
+    // 32-bit byte offsets per lane, no 64-bit address math, hardware range checking (past the extent reads 0)
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.B), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
@@ -392,7 +427,7 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     for (int pass = 0; pass < n_pass; ++pass) {
         const int e0 = pass * kPass + lane * kItems;
         const bool full = e0 + kItems <= n_el;
-        constexpr float kFill = kSoftplus ? -__builtin_inff() : 0.0f;   // see delta_transform
+        constexpr float kFill = delta_fill<kSoftplus>();
         float uv[kItems], raw[kItems], dl[kItems];
         if (full) {
             load_items<in_t, true>(u_base, e0, n_el, uv);
@@ -402,15 +437,14 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
             load_items<in_t, false>(dl_base, e0, n_el, raw, kFill);
         }
 
-        // the (at most) two rows this lane touches
+        // the (at most) two rows this lane touches: items [0,k) lie in row a, [k,8) in row b
         uint32_t rl, l0;
         divmod((uint32_t)min(e0, n_el - 1), divL, rl, l0);
-        const int k = min(kItems, L - (int)l0);              // items [0,k) in row a, [k,8) in row b
+        const int k = kGran == kItems ? kItems : min(kItems, L - (int)l0);
         float A_a[kN], A_b[kN], D_a, D_b, bias_a, bias_b;
         uint32_t Boff_a, Boff_b, Coff_a, Coff_b;      // element offsets; the host checked they fit 32 bits
         {
             const uint32_t row_a = (uint32_t)r0 + rl;
-            const uint32_t row_b = min(row_a + 1u, (uint32_t)p.rows - 1u);
             uint32_t b, d, grp, rem;
             divmod(row_a, divDim, b, d);
             divmod(d, divDpg, grp, rem);
@@ -420,49 +454,63 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
             bias_a = p.bias ? p.bias[d] : 0.0f;
             Boff_a = b * (uint32_t)p.B_bs + grp * (uint32_t)p.B_gs;
             Coff_a = b * (uint32_t)p.C_bs + grp * (uint32_t)p.C_gs;
-            divmod(row_b, divDim, b, d);
-            divmod(d, divDpg, grp, rem);
+            if constexpr (kGran != kItems) {
+                const uint32_t row_b = min(row_a + 1u, (uint32_t)p.rows - 1u);
+                divmod(row_b, divDim, b, d);
+                divmod(d, divDpg, grp, rem);
 #pragma unroll
-            for (int n = 0; n < kN; ++n) A_b[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
-            D_b = p.D ? p.D[d] : 0.0f;
-            bias_b = p.bias ? p.bias[d] : 0.0f;
-            Boff_b = b * (uint32_t)p.B_bs + grp * (uint32_t)p.B_gs;
-            Coff_b = b * (uint32_t)p.C_bs + grp * (uint32_t)p.C_gs;
+                for (int n = 0; n < kN; ++n) A_b[n] = p.A[d * p.A_ds + n * p.A_ns] * kLog2e;
+                D_b = p.D ? p.D[d] : 0.0f;
+                bias_b = p.bias ? p.bias[d] : 0.0f;
+                Boff_b = b * (uint32_t)p.B_bs + grp * (uint32_t)p.B_gs;
+                Coff_b = b * (uint32_t)p.C_bs + grp * (uint32_t)p.C_gs;
+            } else {
+#pragma unroll
+                for (int n = 0; n < kN; ++n) A_b[n] = A_a[n];
+                D_b = D_a; bias_b = bias_a; Boff_b = Boff_a; Coff_b = Coff_a;
+            }
         }
 
-        // Every item's (row, position) is a real element of B / C even for items past the end of this
-        // wavefront's run (row_b is clamped, positions stay below L), so the gathers need no guard.
+        // Every group's (row, position) is a real run of kGran elements of B / C even for items past the end of
+        // this wavefront's run (row b is clamped, positions stay below L), so the gathers need no guard.
         float du[kItems], y[kItems], bias_items[kItems];
-        uint32_t boff[kItems], coff[kItems];
-        bool first[kItems];
+        bool in_a[kGroups], first[kGroups];
+        uint32_t boff[kGroups], coff[kGroups];
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) bias_items[i] = i < k ? bias_a : bias_b;
+        for (int gi = 0; gi < kGroups; ++gi) {
+            in_a[gi] = kGran == kItems ? true : gi * kGran < k;
+            const uint32_t li = in_a[gi] ? l0 + gi * kGran : (uint32_t)(gi * kGran - k);
+            first[gi] = li == 0;
+            boff[gi] = (in_a[gi] ? Boff_a : Boff_b) + li;
+            coff[gi] = (in_a[gi] ? Coff_a : Coff_b) + li;
+#pragma unroll
+            for (int i = 0; i < kGran; ++i) bias_items[gi * kGran + i] = in_a[gi] ? bias_a : bias_b;
+        }
         delta_transform<kSoftplus>(raw, bias_items, dl);
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
-            const bool in_a = i < k;
-            const uint32_t li = in_a ? l0 + i : (uint32_t)(i - k);
-            first[i] = li == 0;
             if constexpr (!kSoftplus) dl[i] = (e0 + i < n_el) ? dl[i] : 0.0f;
             du[i] = dl[i] * uv[i];                       // u is 0 past the end of the run
-            y[i] = (in_a ? D_a : D_b) * uv[i];
-            boff[i] = (in_a ? Boff_a : Boff_b) + li;
-            coff[i] = (in_a ? Coff_a : Coff_b) + li;
+            y[i] = (in_a[i / kGran] ? D_a : D_b) * uv[i];
         }
 
 #pragma unroll
         for (int n = 0; n < kN; ++n) {
             float Bv[kItems], Cv[kItems];
 #pragma unroll
-            for (int i = 0; i < kItems; ++i) {
-                Bv[i] = gather_elem<in_t>(B_rsrc, boff[i] + (uint32_t)n * (uint32_t)p.B_ns);
-                Cv[i] = gather_elem<in_t>(C_rsrc, coff[i] + (uint32_t)n * (uint32_t)p.C_ns);
+            for (int gi = 0; gi < kGroups; ++gi) {
+                float bg[kGran], cg[kGran];
+                gather_group<in_t, kGran>(B_rsrc, boff[gi] + (uint32_t)n * (uint32_t)p.B_ns, bg);
+                gather_group<in_t, kGran>(C_rsrc, coff[gi] + (uint32_t)n * (uint32_t)p.C_ns, cg);
+#pragma unroll
+                for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
             }
             float ac[kItems], hh[kItems];
 #pragma unroll
             for (int i = 0; i < kItems; ++i) {
-                float a = __builtin_amdgcn_exp2f(dl[i] * (i < k ? A_a[n] : A_b[n]));
-                a = first[i] ? 0.0f : a;
+                const int gi = i / kGran;
+                float a = __builtin_amdgcn_exp2f(dl[i] * (in_a[gi] ? A_a[n] : A_b[n]));
+                if (i % kGran == 0) a = first[gi] ? 0.0f : a;
                 // past the end of the run the gathered B belongs to some other row: keep it out
                 const float bb = (e0 + i < n_el) ? Bv[i] * du[i] : 0.0f;
                 ac[i] = i == 0 ? a : ac[i - 1] * a;
@@ -581,6 +629,19 @@ static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
            span_fits_u32(a, q->in_dtype == SS2D_F32 ? 4 : 2);
 }
 
+static int gcd_i64(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
+
+// Largest granularity (1, 2, 4 or 8 elements) at which the flat kernel may treat rows and gather B / C: it must
+// divide L (rows change only at multiples of it) and every B / C stride, and the B / C bases must be aligned to it.
+static int flat_granularity(const ScanArgs &a, int64_t elem_bytes) {
+    int64_t g = gcd_i64(a.L, kItems);
+    const int64_t strides[] = {a.B_bs, a.B_gs, a.B_ns, a.C_bs, a.C_gs, a.C_ns};
+    for (int64_t s : strides) g = gcd_i64(g, s == 0 ? g : s);
+    const uintptr_t bases = reinterpret_cast<uintptr_t>(a.B) | reinterpret_cast<uintptr_t>(a.C);
+    while (g > 1 && (bases % (uintptr_t)(g * elem_bytes)) != 0) g /= 2;
+    return (int)g;
+}
+
 template <typename in_t, typename out_t>
 static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
     ScanArgs a = a_in;
@@ -591,13 +652,22 @@ static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
     const uint32_t n_wg = (uint32_t)((n_waves + kWavesPerWg - 1) / kWavesPerWg);
     const FastDiv dL = make_fastdiv((uint32_t)a.L), dDim = make_fastdiv((uint32_t)a.dim),
                   dDpg = make_fastdiv((uint32_t)a.dim_per_group);
-#define SS2D_LAUNCH_FLAT(N, SP) \
-    hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, N, SP>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL, dDim, dDpg)
-    if (a.N == 1) {
-        if (a.softplus) SS2D_LAUNCH_FLAT(1, true); else SS2D_LAUNCH_FLAT(1, false);
-    } else {
-        if (a.softplus) SS2D_LAUNCH_FLAT(16, true); else SS2D_LAUNCH_FLAT(16, false);
+    const int gran = flat_granularity(a, (int64_t)sizeof(in_t));
+#define SS2D_LAUNCH_FLAT(N, SP, G) \
+    hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, N, SP, G>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL, dDim, dDpg)
+#define SS2D_LAUNCH_FLAT_G(N, SP)                                   \
+    switch (gran) {                                                  \
+        case 8: SS2D_LAUNCH_FLAT(N, SP, 8); break;                   \
+        case 4: SS2D_LAUNCH_FLAT(N, SP, 4); break;                   \
+        case 2: SS2D_LAUNCH_FLAT(N, SP, 2); break;                   \
+        default: SS2D_LAUNCH_FLAT(N, SP, 1); break;                  \
     }
+    if (a.N == 1) {
+        if (a.softplus) { SS2D_LAUNCH_FLAT_G(1, true) } else { SS2D_LAUNCH_FLAT_G(1, false) }
+    } else {
+        if (a.softplus) { SS2D_LAUNCH_FLAT_G(16, true) } else { SS2D_LAUNCH_FLAT_G(16, false) }
+    }
+#undef SS2D_LAUNCH_FLAT_G
 #undef SS2D_LAUNCH_FLAT
     return launch_status();
 }
