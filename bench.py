@@ -49,14 +49,18 @@ def time_op(fn, reps, warm=5):
 
 
 def kernel_lines(reps):
-    """Per-kernel timings of the SS2D core at the four VMamba-T stage shapes (bs128, bf16 in)."""
+    """Per-kernel timings of the SS2D core at the four VMamba-T stage shapes (bs128, bf16 in) and at the
+    BASELINE config 3 / config 4 operator shapes."""
     import torch
     import vmamba_amd as va
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(0)
     out = []
-    for name, (B, D, H, W, N) in dict(stage1=(128, 96, 56, 56, 1), stage2=(128, 192, 28, 28, 1),
-                                      stage3=(128, 384, 14, 14, 1), stage4=(128, 768, 7, 7, 1)).items():
+    shapes = dict(stage1=(128, 96, 56, 56, 1), stage2=(128, 192, 28, 28, 1), stage3=(128, 384, 14, 14, 1),
+                  stage4=(128, 768, 7, 7, 1),
+                  # BASELINE config 3 (16 states, ssm_ratio 2) and the stage-1 shape of config 4 (1024^2 images, batch 4)
+                  n16=(64, 192, 56, 56, 16), hires=(4, 96, 256, 256, 1))
+    for name, (B, D, H, W, N) in shapes.items():
         K, L = 4, H * W
         x = torch.randn(B, D, H, W, device=dev, generator=g).bfloat16()
         delta = (torch.randn(B, K * D, L, device=dev, generator=g) * 0.5).bfloat16()

@@ -83,6 +83,19 @@ __device__ __forceinline__ Raw8<T> load_raw(const T *__restrict__ row, int pos, 
     return r;
 }
 
+// Eight in-range, 16-byte-aligned elements, no bounds check.
+template <typename T>
+__device__ __forceinline__ Raw8<T> load_raw_unchecked(const T *__restrict__ row, int pos) {
+    Raw8<T> r;
+    const uint4 lo = *reinterpret_cast<const uint4 *>(row + pos);
+    r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w;
+    if constexpr (sizeof(T) == 4) {
+        const uint4 hi = *reinterpret_cast<const uint4 *>(row + pos + 4);
+        r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
+    }
+    return r;
+}
+
 template <typename T>
 __device__ __forceinline__ void unpack_raw(const Raw8<T> &r, float (&v)[kItems]) {
     if constexpr (sizeof(T) == 2) {
@@ -252,8 +265,43 @@ __device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_r
 }
 
 // ---- one wavefront per row ------------------------------------------------------------
-// kN > 0: dstate known at compile time, states live in registers.
-// kN == 0: any dstate; the per-wave states live in LDS (2*dstate floats per wave).
+// kN == 1: the single state lives in registers and inputs are fetched in bursts.
+// kN == 0: any dstate; the per-wave states (running product, h) live in LDS, 2*dstate floats per wave: they
+//          are wave-uniform, and keeping 3*dstate of them in vector registers (tried for dstate 16) spills.
+// kGran consecutive elements through a buffer descriptor (32-bit offsets, hardware range check).
+template <typename T, int kGran>
+__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, uint32_t uniform_elem_offset,
+                                             float (&v)[kGran]) {
+    // elem_offset: per lane; uniform_elem_offset: the same for the whole wavefront (rides in a scalar register)
+    const int byte_off = (int)(elem_offset * (uint32_t)sizeof(T));
+    const int soff = (int)(uniform_elem_offset * (uint32_t)sizeof(T));
+    constexpr int kBytes = kGran * (int)sizeof(T);
+    uint32_t w[kBytes >= 4 ? kBytes / 4 : 1];
+    if constexpr (kBytes == 2) {
+        w[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_off, soff, 0);
+    } else if constexpr (kBytes == 4) {
+        w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_off, soff, 0);
+    } else if constexpr (kBytes == 8) {
+        const auto t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, byte_off, soff, 0);
+        w[0] = t[0]; w[1] = t[1];
+    } else if constexpr (kBytes == 16) {
+        const auto t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, soff, 0);
+        w[0] = t[0]; w[1] = t[1]; w[2] = t[2]; w[3] = t[3];
+    } else {
+        static_assert(kBytes == 32, "8 fp32 elements");
+        const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, soff, 0);
+        const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, soff, 0);
+        w[0] = t0[0]; w[1] = t0[1]; w[2] = t0[2]; w[3] = t0[3]; w[4] = t1[0]; w[5] = t1[1]; w[6] = t1[2]; w[7] = t1[3];
+    }
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < kGran; ++i) v[i] = to_f32(T{(uint16_t)(w[i / 2] >> (16 * (i % 2)))});
+    } else {
+#pragma unroll
+        for (int i = 0; i < kGran; ++i) v[i] = bits_to_f32(w[i]);
+    }
+}
+
 template <typename in_t, typename out_t, int kN, bool kVec, bool kSoftplus>
 __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
@@ -279,6 +327,11 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     const float Dv = p.D ? p.D[d] : 0.0f;
     const float bias = p.bias ? p.bias[dg] : 0.0f;
     const int L = p.L;
+    // multi-state vector path: B / C through buffer descriptors (the host checked the extents fit 31 bits)
+    const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.B), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
+    const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
+    const uint32_t B_soff = (uint32_t)(b * p.B_bs + grp * p.B_gs), C_soff = (uint32_t)(b * p.C_bs + grp * p.C_gs);
+    const bool use_buffers = kVec && p.B_span_bytes != 0;
 
     float h_reg[kN > 0 ? kN : 1], ap_reg[kN > 0 ? kN : 1], A_reg[kN > 0 ? kN : 1];
     float *st = dyn_state + (size_t)wave * 2 * N;
@@ -340,8 +393,25 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
         } else {
             for (int n = 0; n < N; ++n) {
                 float Bv[kItems], Cv[kItems], a_tot, h_tot;
-                load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
-                load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                if (use_buffers) {
+                    // the row / state part of the address is a wave-uniform scalar offset, the lane part (the position)
+                    // one 32-bit register shared by all 2N loads of the pass; unconditional (a lane past the end
+                    // re-reads the row's last vector; its du is 0, so the values are never used)
+                    // (each 16-byte half is clamped on its own: rows of fp32 may end on a multiple of 4)
+                    constexpr int kHalf = 16 / (int)sizeof(in_t) >= kItems ? kItems : 16 / (int)sizeof(in_t);
+#pragma unroll
+                    for (int hv = 0; hv < kItems / kHalf; ++hv) {
+                        const int pos_ld = min(pos + hv * kHalf, L - kHalf);
+                        float bh[kHalf], ch[kHalf];
+                        gather_group<in_t, kHalf>(B_rsrc, (uint32_t)pos_ld, B_soff + (uint32_t)n * (uint32_t)p.B_ns, bh);
+                        gather_group<in_t, kHalf>(C_rsrc, (uint32_t)pos_ld, C_soff + (uint32_t)n * (uint32_t)p.C_ns, ch);
+#pragma unroll
+                        for (int i = 0; i < kHalf; ++i) { Bv[hv * kHalf + i] = bh[i]; Cv[hv * kHalf + i] = ch[i]; }
+                    }
+                } else {
+                    load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+                    load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+                }
                 const float ap = st[2 * n], h0 = st[2 * n + 1];
                 scan_state_pass(dl, du, Bv, Cv, A_row[n * p.A_ns] * kLog2e, h0, y, a_tot, h_tot);
                 const float h1 = fmaf(a_tot, h0, h_tot), ap1 = ap * a_tot;
@@ -370,36 +440,6 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 // group, not per item, and B/C are gathered kGran elements at a time through buffer
 // descriptors (their rows are shared by dim/n_groups channels and stay in L1/L2).  A lane
 // touches at most two rows (L >= 8); with kGran == 8 exactly one.
-template <typename T, int kGran>
-__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, float (&v)[kGran]) {
-    const int byte_off = (int)(elem_offset * (uint32_t)sizeof(T));
-    constexpr int kBytes = kGran * (int)sizeof(T);
-    uint32_t w[kBytes >= 4 ? kBytes / 4 : 1];
-    if constexpr (kBytes == 2) {
-        w[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_off, 0, 0);
-    } else if constexpr (kBytes == 4) {
-        w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_off, 0, 0);
-    } else if constexpr (kBytes == 8) {
-        const auto t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, byte_off, 0, 0);
-        w[0] = t[0]; w[1] = t[1];
-    } else if constexpr (kBytes == 16) {
-        const auto t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
-        w[0] = t[0]; w[1] = t[1]; w[2] = t[2]; w[3] = t[3];
-    } else {
-        static_assert(kBytes == 32, "8 fp32 elements");
-        const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
-        const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, 0, 0);
-        w[0] = t0[0]; w[1] = t0[1]; w[2] = t0[2]; w[3] = t0[3]; w[4] = t1[0]; w[5] = t1[1]; w[6] = t1[2]; w[7] = t1[3];
-    }
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-        for (int i = 0; i < kGran; ++i) v[i] = to_f32(T{(uint16_t)(w[i / 2] >> (16 * (i % 2)))});
-    } else {
-#pragma unroll
-        for (int i = 0; i < kGran; ++i) v[i] = bits_to_f32(w[i]);
-    }
-}
-
 template <typename in_t, typename out_t, int kN, bool kSoftplus, int kGran>
 __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int rows_per_wave, FastDiv divL,
                                                            FastDiv divDim, FastDiv divDpg) {
@@ -500,8 +540,8 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
 #pragma unroll
             for (int gi = 0; gi < kGroups; ++gi) {
                 float bg[kGran], cg[kGran];
-                gather_group<in_t, kGran>(B_rsrc, boff[gi] + (uint32_t)n * (uint32_t)p.B_ns, bg);
-                gather_group<in_t, kGran>(C_rsrc, coff[gi] + (uint32_t)n * (uint32_t)p.C_ns, cg);
+                gather_group<in_t, kGran>(B_rsrc, boff[gi], (uint32_t)n * (uint32_t)p.B_ns, bg);
+                gather_group<in_t, kGran>(C_rsrc, coff[gi], (uint32_t)n * (uint32_t)p.C_ns, cg);
 #pragma unroll
                 for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
             }
@@ -690,8 +730,6 @@ static int launch_scan(const ScanArgs &a, hipStream_t stream) {
     hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, N, kVec, SP>), dim3(n_wg), dim3(kBlock), SMEM, stream, a)
     if (a.N == 1) {
         if (a.softplus) SS2D_LAUNCH_ROW(1, true, 0); else SS2D_LAUNCH_ROW(1, false, 0);
-    } else if (a.N == 16) {
-        if (a.softplus) SS2D_LAUNCH_ROW(16, true, 0); else SS2D_LAUNCH_ROW(16, false, 0);
     } else {
         const size_t smem = (size_t)kWavesPerWg * 2 * a.N * sizeof(float);
         if (a.softplus) SS2D_LAUNCH_ROW(0, true, smem); else SS2D_LAUNCH_ROW(0, false, smem);
@@ -737,6 +775,12 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     a.o_bs = q->out_batch_stride; a.o_ds = q->out_d_stride;
     a.rows = q->batch * q->dim;
     a.B_span_bytes = a.C_span_bytes = 0;
+    const int64_t in_bytes = q->in_dtype == SS2D_F32 ? 4 : 2;
+    const bool spans_fit = span_fits_u32(a, in_bytes);
+    if (spans_fit) {
+        a.B_span_bytes = (uint32_t)(span_elems(a, a.B_bs, a.B_gs, a.B_ns) * in_bytes);
+        a.C_span_bytes = (uint32_t)(span_elems(a, a.C_bs, a.C_gs, a.C_ns) * in_bytes);
+    }
 
     // 16-byte vector I/O needs every row start and the row length on a 16-byte grid.
     const int64_t in_vec = q->in_dtype == SS2D_F32 ? 4 : 8;
