@@ -23,6 +23,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the stage-1 scan kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --kernels-only`, each counter scaled by what it reads for the 1 GiB calibration copy (FETCH_SIZE x2.0,
+# WRITE_SIZE x1.0); the summary is profiles/ss2d_core_kernels_vmamba_t_bs128.txt.  Counters cannot be read from
+# inside the timed process, so this is the last profiled value, refreshed whenever the kernel changes.
+SCAN_STAGE1_MEASURED_TRAFFIC_BYTES = 668.4e6 + 617.1e6
 
 
 def log(*a):
@@ -218,7 +223,8 @@ def main():
         k1 = kernels[0]
         roofline = dict(bound="hbm", kernel="scan_row_kernel<bf16,f32,N=1> @ stage1 (B=128, KD=384, L=3136)",
                         achieved=k1["scan_GBs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=k1["scan_GBs"] / HBM_PEAK_GBS,
-                        traffic=None, bytes_per_launch=k1["scan_bytes"], us_per_launch=k1["scan_us"])
+                        traffic=SCAN_STAGE1_MEASURED_TRAFFIC_BYTES, bytes_per_launch=k1["scan_bytes"],
+                        us_per_launch=k1["scan_us"])
     cpu = None if args.no_cpu_baseline else cpu_baseline()
 
     print(json.dumps({
