@@ -146,6 +146,49 @@ int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void
 int ss2d_dwconv3x3_silu(const void *x, const void *weight, const void *bias, void *y, int B, int D, int H, int W,
                         int dtype, int in_channel_last, int apply_silu, void *stream);
 
+/*
+ * CrossScan, one-by-one, scans=0, channel-first: every direction slice of the input is put in ITS scan order.
+ * Replaces CrossScanTriton1b1.forward / cross_scan1b1_fwd (classification/models/csm_triton.py:88-131, 400-436).
+ *   x (B,4,C,H,W) contiguous -> y[b*y_batch_stride + k*y_dir_stride + c*y_chan_stride + j], j in [0, L):
+ *   y[b,0,c,h*W+w] = x[b,0,c,h,w];  y[b,1,c,w*H+h] = x[b,1,c,h,w];
+ *   y[b,2,c,L-1-(h*W+w)] = x[b,2,c,h,w];  y[b,3,c,L-1-(w*H+h)] = x[b,3,c,h,w]
+ * Strides in elements; (4*C*L, C*L, L) is the reference's contiguous (B,4,C,L).  Other strides let the caller
+ * produce e.g. the direction-major, batch-innermost (4,C,B,L) layout ss2d_core_fwd reads.  elem_bytes in {1,2,4,8}.
+ */
+int ss2d_cross_scan_1b1(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int64_t y_batch_stride,
+                        int64_t y_dir_stride, int64_t y_chan_stride, void *stream);
+
+/*
+ * Fused SS2D core for dstate = 1: CrossScan -> selective scan (softplus, fp32 state, fp32 "oflex" output) ->
+ * CrossMerge in one kernel.  Replaces the three calls of SS2Dv2.forward_corev2
+ * (classification/models/vmamba.py:604, 625-633, 638: cross_scan_fn, selective_scan, cross_merge_fn) for
+ * scans=0 / d_state=1; the projections between them (vmamba.py:605-615) stay the caller's GEMMs and are handed
+ * over already in scan order:
+ *   x      (batch, dim, height, width) contiguous, in_dtype: the conv+SiLU output; read once, never expanded
+ *   delta  [k*delta_dir_stride + d*delta_dim_stride + b*delta_batch_stride + j]  in_dtype, j = scan position
+ *          of direction k (dt_proj output before bias and softplus)
+ *   B, C   [k*dir_stride + b*batch_stride + j]  in_dtype (x_proj's B and C rows: one state, one group per direction)
+ *   A, D, delta_bias (4*dim) fp32, index k*dim + d; D and delta_bias may be NULL
+ *   y      (batch, dim, height*width) contiguous fp32:
+ *          y = (y_0 + flip(y_2)) + transpose(y_1 + flip(y_3)), y_k the scan output of direction k, each add
+ *          rounded to fp32 -- cross_merge_fwd's order (csm_triton.py:56-62) on the oflex fp32 scan outputs.
+ * Strides in elements.  The kernel walks several images per workgroup when delta_batch_stride == height*width
+ * (batch-innermost layout) and falls back to one image per workgroup otherwise.  Returns SS2D_ENOTSUP when the
+ * delta rows are not 16-byte aligned or the image does not fit the LDS planes (height*width above ~6000).
+ */
+typedef struct ss2d_core_params {
+    int32_t batch, dim, height, width;
+    int32_t in_dtype;
+    int32_t delta_softplus;
+    const void *x, *delta, *A, *B, *C, *D, *delta_bias;
+    void *y;
+    int64_t delta_dir_stride, delta_dim_stride, delta_batch_stride;
+    int64_t B_dir_stride, B_batch_stride;
+    int64_t C_dir_stride, C_batch_stride;
+} ss2d_core_params;
+
+int ss2d_core_fwd(const ss2d_core_params *params, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,6 +8,7 @@ CPU path" that the benchmark times on the host cores as ``cpu_baseline``.
 
 Follows, without importing them:
   cross_scan   classification/models/csm_triton.py:22-29 and :532-541
+  cross_scan_1b1  classification/models/csm_triton.py:88-99 (one-by-one, scans = 0)
   cross_merge  classification/models/csm_triton.py:56-62 and :543-551
   selective_scan  kernels/selective_scan/test_selective_scan.py:168-234
                   (selective_scan_ref; same arithmetic as csms6s.py:25-68 but
@@ -23,6 +24,14 @@ def cross_scan(x):
     row_major = x.reshape(B, C, H * W)
     col_major = x.transpose(2, 3).reshape(B, C, H * W)
     return torch.stack([row_major, col_major, row_major.flip(-1), col_major.flip(-1)], dim=1)
+
+
+def cross_scan_1b1(x):
+    """x (B,4,C,H,W): direction slice k laid out in the scan order of direction k."""
+    B, K, C, H, W = x.shape
+    col = lambda v: v.transpose(2, 3).reshape(B, C, H * W)
+    return torch.stack([x[:, 0].reshape(B, C, H * W), col(x[:, 1]),
+                        x[:, 2].reshape(B, C, H * W).flip(-1), col(x[:, 3]).flip(-1)], dim=1)
 
 
 def cross_merge(ys):

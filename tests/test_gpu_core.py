@@ -1,0 +1,182 @@
+"""GPU parity of the fused SS2D core (CrossScan -> selective scan -> CrossMerge in one kernel) and of the
+one-by-one CrossScan, through the C ABI, against the CPU oracle's composition of the three operators.
+
+Tolerance: the scan bound (fp32 output: rtol 1e-3) with an absolute floor of 4e-4 -- the merged value is a sum of
+four scan outputs, each good to atol 1e-4.
+"""
+import pytest
+import torch
+
+from oracle import ss2d_oracle as orc
+from oracle import torch_ref
+import vmamba_amd as va
+from vmamba_amd import _lib
+from vmamba_amd.core import ss2d_core_hip
+from vmamba_amd.csm import cross_scan_1b1_hip
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = dict(rtol=1e-3, atol=4e-4)
+
+
+def _announce(*what):
+    print("CASE", *what, flush=True)
+
+
+def make_core_inputs(seed, B, D, H, W, dtype):
+    g = torch.Generator().manual_seed(seed)
+    L = H * W
+    dt = torch.exp(torch.rand(4 * D, generator=g) * (torch.log(torch.tensor(0.1)) - torch.log(torch.tensor(1e-3)))
+                   + torch.log(torch.tensor(1e-3)))
+    bias = dt + torch.log(-torch.expm1(-dt))
+    A = -(0.5 + torch.rand(4 * D, generator=g))
+    Dv = torch.randn(4 * D, generator=g)
+    x = torch.randn(B, D, H, W, generator=g).to(dtype)
+    delta = torch.randn(4, D, B, L, generator=g).to(dtype)
+    Bs = torch.randn(4, B, L, generator=g).to(dtype)
+    Cs = torch.randn(4, B, L, generator=g).to(dtype)
+    return x, delta, Bs, Cs, A, Dv, bias
+
+
+def oracle_core(x, delta, Bs, Cs, A, Dv, bias, softplus=True):
+    """cross_scan -> selective_scan (fp32 out) -> cross_merge, each the CPU oracle's."""
+    B, D, H, W = x.shape
+    L = H * W
+    xs = orc.cross_scan(x)                                                    # (B, 4, D, L)
+    ys = orc.selective_scan(xs.reshape(B, 4 * D, L), delta.permute(2, 0, 1, 3).reshape(B, 4 * D, L).contiguous(),
+                            A.view(4 * D, 1), Bs.permute(1, 0, 2).unsqueeze(2).contiguous(),
+                            Cs.permute(1, 0, 2).unsqueeze(2).contiguous(), Dv, bias, softplus, out_float=True)
+    return orc.cross_merge(ys.view(B, 4, D, H, W))                            # (B, D, L) fp32, pairwise order
+
+
+def run_core(x, delta, Bs, Cs, A, Dv, bias, softplus=True):
+    dev = lambda t: None if t is None else t.to(DEV)
+    y = ss2d_core_hip(dev(x), dev(delta), dev(Bs), dev(Cs), dev(A), dev(Dv), dev(bias), softplus)
+    torch.cuda.synchronize()
+    return y.cpu()
+
+
+CORE_SHAPES = [
+    (2, 3, 56, 56),      # one image per workgroup, 8-wide B/C groups
+    (5, 4, 28, 28),      # four images per workgroup + a one-image tail
+    (18, 2, 14, 14),     # L % 8 == 4: 16 images per workgroup, tail of two
+    (70, 2, 7, 7),       # odd L: 64 images per workgroup, element-wise B/C gathers
+    (3, 2, 7, 9),        # H != W, odd L
+    (2, 2, 10, 12),      # H != W
+    (9, 1, 6, 5),        # L = 30: two-element granularity handled element-wise
+    (1, 1, 3, 3),        # smallest supported image
+    (1, 2, 64, 48),      # L = 3072
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", CORE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_core_matches_oracle_composition(shape, dtype):
+    _announce("core", shape, dtype)
+    args = make_core_inputs(sum(shape), *shape, dtype)
+    want = oracle_core(*args)
+    got = run_core(*args)
+    assert got.dtype == torch.float32 and got.shape == want.shape
+    err = (got - want).abs().max().item()
+    assert torch.allclose(got, want, **TOL), f"max abs err {err}"
+
+
+@pytest.mark.parametrize("softplus", [True, False])
+def test_core_optional_arguments(softplus):
+    _announce("core optional", softplus)
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(11, 6, 3, 14, 14, torch.bfloat16)
+    if not softplus:        # delta + bias is the step itself: keep it positive (the reference's own test ranges)
+        g = torch.Generator().manual_seed(3)
+        delta = (0.5 * torch.rand(delta.shape, generator=g)).to(delta.dtype)
+        bias = 0.5 * torch.rand(bias.shape, generator=g)
+    for dv, bi in ((None, bias), (Dv, None), (None, None)):
+        want = oracle_core(x, delta, Bs, Cs, A, dv, bi, softplus)
+        got = run_core(x, delta, Bs, Cs, A, dv, bi, softplus)
+        assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
+
+
+def test_core_reference_layout_strides():
+    """delta (B,4,D,L) and B/C (B,4,1,L) as the reference's projections lay them out, passed as permuted views:
+    one image per workgroup, same result."""
+    _announce("core strided")
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(21, 5, 3, 28, 28, torch.bfloat16)
+    want = oracle_core(x, delta, Bs, Cs, A, Dv, bias)
+    dev = lambda t: t.to(DEV)
+    delta_ref = dev(delta).permute(2, 0, 1, 3).contiguous()            # (B, 4, D, L)
+    B_ref = dev(Bs).permute(1, 0, 2).contiguous()                     # (B, 4, L)
+    C_ref = dev(Cs).permute(1, 0, 2).contiguous()
+    got = ss2d_core_hip(dev(x), delta_ref.permute(1, 2, 0, 3), B_ref.permute(1, 0, 2), C_ref.permute(1, 0, 2), dev(A), dev(Dv),
+                        dev(bias), True)
+    torch.cuda.synchronize()
+    assert torch.allclose(got.cpu(), want, **TOL)
+    same = run_core(x, delta, Bs, Cs, A, Dv, bias)
+    assert torch.allclose(got.cpu(), same, rtol=1e-5, atol=1e-6)      # both layouts: same arithmetic per image
+
+
+def test_core_equals_three_kernels_at_model_shape():
+    """Full stage shapes: the fused kernel against this package's own cross_scan / scan / merge kernels (which the
+    oracle pins at smaller sizes)."""
+    for (B, D, H, W) in ((16, 96, 56, 56), (16, 192, 28, 28), (32, 384, 14, 14), (128, 768, 7, 7)):
+        _announce("core vs kernels", B, D, H, W)
+        x, delta, Bs, Cs, A, Dv, bias = [None if t is None else t.to(DEV) for t in make_core_inputs(B + D, B, D, H, W, torch.bfloat16)]
+        L = H * W
+        xs = va.cross_scan_fn(x)
+        ys = va.selective_scan_fn(xs.view(B, 4 * D, L), delta.permute(2, 0, 1, 3).reshape(B, 4 * D, L), A.view(4 * D, 1),
+                                  Bs.permute(1, 0, 2).unsqueeze(2), Cs.permute(1, 0, 2).unsqueeze(2), Dv, bias, True, True)
+        want = va.cross_merge_fn(ys.view(B, 4, D, H, W))
+        got = ss2d_core_hip(x, delta, Bs, Cs, A, Dv, bias, True)
+        torch.cuda.synchronize()
+        err = (got - want).abs().max().item()
+        assert torch.allclose(got, want, **TOL), f"max abs err {err}"
+
+
+def test_core_rejections():
+    x, delta, Bs, Cs, A, Dv, bias = [t.to(DEV) for t in make_core_inputs(1, 2, 2, 4, 4, torch.bfloat16)]
+    with pytest.raises(RuntimeError):
+        ss2d_core_hip(x, delta[:, :, :1], Bs, Cs, A, Dv, bias)
+    with pytest.raises(RuntimeError):
+        ss2d_core_hip(x, delta.float(), Bs, Cs, A, Dv, bias)
+    with pytest.raises(RuntimeError):
+        ss2d_core_hip(x.cpu(), delta, Bs, Cs, A, Dv, bias)
+    # image too large for the LDS planes: a clean "not supported", never a launch
+    big = [t.to(DEV) for t in make_core_inputs(1, 1, 1, 96, 96, torch.bfloat16)]
+    with pytest.raises(_lib.Ss2dError) as e:
+        ss2d_core_hip(*big)
+    assert e.value.code == _lib.SS2D_ENOTSUP
+    # images shorter than one lane's 8 positions
+    tiny = [t.to(DEV) for t in make_core_inputs(1, 2, 2, 2, 2, torch.bfloat16)]
+    with pytest.raises(_lib.Ss2dError) as e:
+        ss2d_core_hip(*tiny)
+    assert e.value.code == _lib.SS2D_ENOTSUP
+    assert ss2d_core_hip(*[t.to(DEV) for t in make_core_inputs(1, 0, 2, 4, 4, torch.bfloat16)]).shape == (0, 2, 16)
+
+
+# ---- one-by-one CrossScan ----------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8, torch.float64], ids=str)
+@pytest.mark.parametrize("shape", [(2, 3, 56, 56), (3, 5, 7, 9), (1, 2, 1, 17), (2, 1, 13, 1), (1, 1, 130, 100)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_cross_scan_1b1_bit_exact(shape, dtype):
+    _announce("cross_scan_1b1", shape, dtype)
+    B, C, H, W = shape
+    g = torch.Generator().manual_seed(B * 100 + C)
+    x = (torch.randn(B, 4, C, H, W, generator=g) * 50).to(dtype)
+    want = torch_ref.cross_scan_1b1(x)
+    got = va.cross_scan_fn(x.to(DEV), one_by_one=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got.cpu(), want)
+    # direction-major, batch-innermost destination: same values through the strides
+    buf = torch.full((4, C, B, H * W), 7, dtype=dtype, device=DEV)
+    out = cross_scan_1b1_hip(x.to(DEV), out=buf.permute(2, 0, 1, 3))
+    torch.cuda.synchronize()
+    assert out.data_ptr() == buf.data_ptr()
+    assert torch.equal(buf.permute(2, 0, 1, 3).cpu(), want)
+
+
+def test_cross_scan_1b1_empty_and_bad_args():
+    assert va.cross_scan_fn(torch.zeros(0, 4, 3, 4, 4, device=DEV), one_by_one=True).shape == (0, 4, 3, 16)
+    with pytest.raises(ValueError):
+        va.cross_scan_fn(torch.zeros(2, 3, 3, 4, 4, device=DEV), one_by_one=True)
+    with pytest.raises(NotImplementedError):
+        va.cross_scan_fn(torch.zeros(2, 4, 3, 4, 4), one_by_one=True)

@@ -60,6 +60,24 @@ def test_cross_scan_brute_force_and_second_formulation(shape, dtype):
         assert torch.equal(y[:, k].float().sort(-1).values, x.reshape(B, C, L).float().sort(-1).values)
 
 
+def test_cross_scan_1b1_pins():
+    """One-by-one scan: with the same map in all four slices it IS cross_scan; and slice k only depends on
+    input slice k (checked by perturbing one slice at a time)."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 3, 4, 6, generator=g)
+    x4 = x.unsqueeze(1).expand(-1, 4, -1, -1, -1).contiguous()
+    assert torch.equal(torch_ref.cross_scan_1b1(x4), orc.cross_scan(x))
+    base = torch.randn(2, 4, 3, 4, 6, generator=g)
+    y = torch_ref.cross_scan_1b1(base)
+    for k in range(4):
+        z = base.clone()
+        z[:, k] += 1.0
+        yz = torch_ref.cross_scan_1b1(z)
+        for kk in range(4):
+            assert torch.equal(yz[:, kk], y[:, kk]) == (kk != k)
+        assert torch.equal(yz[:, k], orc.cross_scan(z[:, k])[:, k])
+
+
 def test_cross_scan_empty():
     assert orc.cross_scan(torch.zeros(0, 3, 4, 4)).shape == (0, 4, 3, 16)
     assert orc.cross_scan(torch.zeros(2, 0, 4, 4)).shape == (2, 4, 0, 16)

@@ -15,7 +15,7 @@ SCAN_CHUNK = 2048
 ABI_VERSION = 1
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
-           "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu")
+           "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd")
 
 
 class ScanParams(ctypes.Structure):
@@ -29,6 +29,16 @@ class ScanParams(ctypes.Structure):
                                          "B_batch_stride", "B_group_stride", "B_dstate_stride",
                                          "C_batch_stride", "C_group_stride", "C_dstate_stride",
                                          "out_batch_stride", "out_d_stride")]
+    )
+
+
+class CoreParams(ctypes.Structure):
+    """struct ss2d_core_params (include/ss2d_hip.h)."""
+    _fields_ = (
+        [(n, ctypes.c_int32) for n in ("batch", "dim", "height", "width", "in_dtype", "delta_softplus")]
+        + [(n, ctypes.c_void_p) for n in ("x", "delta", "A", "B", "C", "D", "delta_bias", "y")]
+        + [(n, ctypes.c_int64) for n in ("delta_dir_stride", "delta_dim_stride", "delta_batch_stride",
+                                         "B_dir_stride", "B_batch_stride", "C_dir_stride", "C_batch_stride")]
     )
 
 
@@ -66,6 +76,11 @@ def lib():
                                          + [ctypes.c_int] * 4 + [ctypes.c_void_p])
         L.ss2d_dwconv3x3_silu.restype = ctypes.c_int
         L.ss2d_dwconv3x3_silu.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_void_p]
+        L.ss2d_cross_scan_1b1.restype = ctypes.c_int
+        L.ss2d_cross_scan_1b1.argtypes = ([ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_int64] * 3
+                                          + [ctypes.c_void_p])
+        L.ss2d_core_fwd.restype = ctypes.c_int
+        L.ss2d_core_fwd.argtypes = [ctypes.POINTER(CoreParams), ctypes.c_void_p]
         if L.ss2d_abi_version() != ABI_VERSION:
             raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L

@@ -1,0 +1,60 @@
+"""Fused SS2D core operator: CrossScan -> selective scan -> CrossMerge in one HIP kernel (d_state = 1).
+
+Stands in for the three operator calls of SS2Dv2.forward_corev2 (classification/models/vmamba.py:604,
+625-633, 638) when the model has one state per channel; the projections between them remain the caller's.
+"""
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.SS2D_F32, torch.bfloat16: _lib.SS2D_BF16, torch.float16: _lib.SS2D_F16}
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True):
+    """x (B,D,H,W); delta (4,D,B,L) view; Bs, Cs (4,B,L) views (last stride 1), all of x.dtype and already in the
+    scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32.
+
+    Raises Ss2dError with status SS2D_ENOTSUP when the shape has no fused kernel (image too large for the LDS
+    planes, unaligned delta rows): callers fall back to the three separate operators.
+    """
+    _check(x.is_cuda, "ss2d_core: vmamba_amd runs on the GPU only")
+    _check(x.dim() == 4, "x must be (B, D, H, W)")
+    _check(x.dtype in _DTYPE_CODE, f"ss2d_core not implemented for input type '{x.dtype}'")
+    B, D, H, W = x.shape
+    L = H * W
+    for name, t in (("delta", delta), ("B", Bs), ("C", Cs)):
+        _check(t.is_cuda and t.dtype == x.dtype, f"{name} must be a GPU tensor of x's dtype")
+        _check(t.stride(-1) == 1 or t.size(-1) == 1, f"{name} must be contiguous in its last dimension")
+    _check(tuple(delta.shape) == (4, D, B, L), "delta must have shape (4, dim, batch, L)")
+    _check(tuple(Bs.shape) == (4, B, L) and tuple(Cs.shape) == (4, B, L), "B and C must have shape (4, batch, L)")
+    _check(As.dtype == torch.float32 and As.is_cuda and As.numel() == 4 * D, "A must be (4*dim) float32 (one state)")
+    As = As.contiguous()
+    if Ds is not None:
+        _check(Ds.dtype == torch.float32 and Ds.is_cuda and tuple(Ds.shape) == (4 * D,), "D must be (4*dim) float32")
+        Ds = Ds.contiguous()
+    if delta_bias is not None:
+        _check(delta_bias.dtype == torch.float32 and delta_bias.is_cuda and tuple(delta_bias.shape) == (4 * D,),
+               "delta_bias must be (4*dim) float32")
+        delta_bias = delta_bias.contiguous()
+    x = x.contiguous()
+    y = torch.empty((B, D, L), device=x.device, dtype=torch.float32)
+    p = _lib.CoreParams()
+    p.batch, p.dim, p.height, p.width = B, D, H, W
+    p.in_dtype = _DTYPE_CODE[x.dtype]
+    p.delta_softplus = 1 if delta_softplus else 0
+    p.x, p.delta, p.A, p.B, p.C = x.data_ptr(), delta.data_ptr(), As.data_ptr(), Bs.data_ptr(), Cs.data_ptr()
+    p.D = Ds.data_ptr() if Ds is not None else None
+    p.delta_bias = delta_bias.data_ptr() if delta_bias is not None else None
+    p.y = y.data_ptr()
+    p.delta_dir_stride, p.delta_dim_stride, p.delta_batch_stride = delta.stride(0), delta.stride(1), delta.stride(2)
+    p.B_dir_stride, p.B_batch_stride = Bs.stride(0), Bs.stride(1)
+    p.C_dir_stride, p.C_batch_stride = Cs.stride(0), Cs.stride(1)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_core_fwd(p, torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_core_fwd")
+    return y

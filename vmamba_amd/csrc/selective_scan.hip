@@ -18,16 +18,9 @@
 // (kVec); otherwise element-wise with bounds checks.  Positions past the end of a row are fed
 // as dl = 0, u = 0, i.e. the identity pair (1, 0), so the state at the end of the last pass is
 // the state at the last real position.
-#include "ss2d_common.h"
+#include "scan_common.h"
 
 namespace ss2d {
-
-constexpr int kItems = 8;                    // consecutive positions per lane per pass
-constexpr int kPass = kWave * kItems;        // 512 positions per wavefront pass
-constexpr int kWavesPerWg = kBlock / kWave;  // 4
-constexpr int kPassesPerChunk = SS2D_SCAN_CHUNK / kPass;  // 4
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 
 struct ScanArgs {
     const void *u, *delta, *B, *C;
@@ -40,268 +33,10 @@ struct ScanArgs {
     uint32_t B_span_bytes, C_span_bytes;   // flat kernel: extent of B / C reachable through the strides
 };
 
-// ---- 8-wide loads / stores ------------------------------------------------------------
-// Eight consecutive elements of a row as they sit in registers before widening: 4 dwords for 16-bit
-// types, 8 for fp32.  Keeping loads in this form lets a pass issue the NEXT pass's loads before it
-// starts computing (software prefetch), which is what keeps enough bytes in flight per wavefront.
-template <typename T> struct Raw8 { uint32_t w[sizeof(T) * 2]; };
-
-// Items at positions >= L come back as `fill`.
-template <typename T, bool kVec>
-__device__ __forceinline__ Raw8<T> load_raw(const T *__restrict__ row, int pos, int L, float fill = 0.0f) {
-    Raw8<T> r;
-    if constexpr (kVec) {
-        // the host guarantees 16-byte alignment and L % (16/sizeof(T)) == 0, so a vector is either
-        // entirely inside the row or entirely outside
-        if constexpr (sizeof(T) == 2) {
-            const uint32_t fill2 = (uint32_t)from_f32<T>(fill).bits * 0x10001u;
-            uint4 v = make_uint4(fill2, fill2, fill2, fill2);
-            if (pos < L) v = *reinterpret_cast<const uint4 *>(row + pos);
-            r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z; r.w[3] = v.w;
-        } else {
-            const uint32_t f = f32_to_bits(fill);
-            uint4 lo = make_uint4(f, f, f, f), hi = lo;
-            if (pos < L) lo = *reinterpret_cast<const uint4 *>(row + pos);
-            if (pos + 4 < L) hi = *reinterpret_cast<const uint4 *>(row + pos + 4);
-            r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w;
-            r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
-        }
-    } else {
-        if constexpr (sizeof(T) == 2) {
-            const uint32_t fb = from_f32<T>(fill).bits;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t lo = (pos + 2 * i < L) ? row[pos + 2 * i].bits : fb;
-                const uint32_t hi = (pos + 2 * i + 1 < L) ? row[pos + 2 * i + 1].bits : fb;
-                r.w[i] = lo | (hi << 16);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kItems; ++i) r.w[i] = f32_to_bits((pos + i < L) ? row[pos + i] : fill);
-        }
-    }
-    return r;
-}
-
-// Eight in-range, 16-byte-aligned elements, no bounds check.
-template <typename T>
-__device__ __forceinline__ Raw8<T> load_raw_unchecked(const T *__restrict__ row, int pos) {
-    Raw8<T> r;
-    const uint4 lo = *reinterpret_cast<const uint4 *>(row + pos);
-    r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w;
-    if constexpr (sizeof(T) == 4) {
-        const uint4 hi = *reinterpret_cast<const uint4 *>(row + pos + 4);
-        r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
-    }
-    return r;
-}
-
-template <typename T>
-__device__ __forceinline__ void unpack_raw(const Raw8<T> &r, float (&v)[kItems]) {
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[2 * i] = to_f32(T{(uint16_t)(r.w[i] & 0xffffu)});
-            v[2 * i + 1] = to_f32(T{(uint16_t)(r.w[i] >> 16)});
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < kItems; ++i) v[i] = bits_to_f32(r.w[i]);
-    }
-}
-
-template <typename T, bool kVec>
-__device__ __forceinline__ void load_items(const T *__restrict__ row, int pos, int L, float (&v)[kItems],
-                                           float fill = 0.0f) {
-    unpack_raw<T>(load_raw<T, kVec>(row, pos, L, fill), v);
-}
-
-template <typename T, bool kVec>
-__device__ __forceinline__ void store_items(T *__restrict__ row, int pos, int L, const float (&v)[kItems]) {
-    if constexpr (kVec) {
-        if constexpr (sizeof(T) == 2) {
-            if (pos < L) {
-                uint32_t w[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    w[i] = (uint32_t)from_f32<T>(v[2 * i]).bits | ((uint32_t)from_f32<T>(v[2 * i + 1]).bits << 16);
-                *reinterpret_cast<uint4 *>(row + pos) = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        } else {
-            if (pos < L) *reinterpret_cast<float4 *>(row + pos) = make_float4(v[0], v[1], v[2], v[3]);
-            if (pos + 4 < L) *reinterpret_cast<float4 *>(row + pos + 4) = make_float4(v[4], v[5], v[6], v[7]);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < kItems; ++i)
-            if (pos + i < L) row[pos + i] = from_f32<T>(v[i]);
-    }
-}
-
-constexpr int kBufferRsrcWord3 = 0x00020000;   // raw buffer, 32-bit data format (gfx9 family)
-
-template <typename T>
-__device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset) {
-    if constexpr (sizeof(T) == 2) {
-        return to_f32(T{(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)(elem_offset * 2u), 0, 0)});
-    } else {
-        return bits_to_f32((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(elem_offset * 4u), 0, 0));
-    }
-}
-
-// delta -> dl for the 8 items of a lane.
-//   kSoftplus: dl = softplus(raw + bias) = ln2 * log2(1 + 2^((raw + bias) * log2e)) with the two hardware
-//   transcendentals.  w = 1 + t loses the low bits of a small t; c = t - (w - 1) is exactly that loss (t < 1), and
-//   log(1 + t) = log(w) + c/w with c/w ~ c.  Arguments above 20 return the argument itself (the reference's
-//   threshold); that select sits behind a wave-uniform vote because it is almost never taken.
-//   A raw value of -inf (the fill for positions past the end of a row) gives t = 0, dl = 0: the identity pair.
-//   !kSoftplus: dl = raw + bias; the caller zeroes positions past the end.
-constexpr float kSoftplusThreshold = 20.0f;
-
-template <bool kSoftplus>
-__device__ __forceinline__ void delta_transform(const float (&raw)[kItems], const float (&bias)[kItems],
-                                                float (&dl)[kItems]) {
-    if constexpr (kSoftplus) {
-        float zmax = -__builtin_inff();
-#pragma unroll
-        for (int i = 0; i < kItems; ++i) {
-            const float z = fmaf(raw[i], kLog2e, bias[i] * kLog2e);
-            zmax = __builtin_fmaxf(zmax, z);
-            const float t = __builtin_amdgcn_exp2f(z);
-            const float w = 1.0f + t;
-            float c = t - (w - 1.0f);
-            c = t < 1.0f ? c : 0.0f;
-            dl[i] = fmaf(kLn2, __builtin_amdgcn_logf(w), c);
-        }
-        if (__builtin_amdgcn_ballot_w64(zmax > kSoftplusThreshold * kLog2e) != 0) {
-#pragma unroll
-            for (int i = 0; i < kItems; ++i) {
-                const float x = raw[i] + bias[i];
-                dl[i] = x > kSoftplusThreshold ? x : dl[i];
-            }
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < kItems; ++i) dl[i] = raw[i] + bias[i];
-    }
-}
-
-// Inclusive scan of (a,h) over the 64 lanes; returns this lane's EXCLUSIVE prefix in
-// (a_ex,h_ex) and the wave total, uniform, in (a_tot,h_tot).
-__device__ __forceinline__ void wave_scan_pairs(float a, float h, float &a_ex, float &h_ex, float &a_tot,
-                                                float &h_tot) {
-#define SS2D_SCAN_STEP(CTRL, MASK)                        \
-    {                                                     \
-        const float ap = dpp_move<CTRL, MASK>(1.0f, a);   \
-        const float hp = dpp_move<CTRL, MASK>(0.0f, h);   \
-        h = fmaf(a, hp, h);                               \
-        a = a * ap;                                       \
-    }
-    SS2D_SCAN_STEP(kDppRowShr1, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr2, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr4, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr8, 0xF)
-    SS2D_SCAN_STEP(kDppRowBcast15, 0xA)
-    SS2D_SCAN_STEP(kDppRowBcast31, 0xC)
-#undef SS2D_SCAN_STEP
-    a_ex = dpp_move<kDppWaveShr1>(1.0f, a);
-    h_ex = dpp_move<kDppWaveShr1>(0.0f, h);
-    a_tot = read_lane(a, kWave - 1);
-    h_tot = read_lane(h, kWave - 1);
-}
-
-// One state of one pass: lane-local scan of its 8 items, wave scan of the lane totals, then
-// the state entering the lane (from `carry`, the state entering the pass) is pushed through
-// the items and C*h is accumulated into y.  Returns the pass totals.
-__device__ __forceinline__ void scan_state_pass(const float (&dl)[kItems], const float (&du)[kItems],
-                                                const float (&Bv)[kItems], const float (&Cv)[kItems], float A_log2e,
-                                                float carry, float (&y)[kItems], float &a_tot, float &h_tot) {
-    float ac[kItems], hh[kItems];
-#pragma unroll
-    for (int i = 0; i < kItems; ++i) {
-        const float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
-        const float b = Bv[i] * du[i];
-        ac[i] = i == 0 ? a : ac[i - 1] * a;
-        hh[i] = i == 0 ? b : fmaf(a, hh[i - 1], b);
-    }
-    float a_ex, h_ex;
-    wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
-    const float s_in = fmaf(a_ex, carry, h_ex);
-#pragma unroll
-    for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
-}
-
-// The fill the delta loads use past the end of a row (see delta_transform).
-template <bool kSoftplus> __device__ __forceinline__ constexpr float delta_fill() {
-    return kSoftplus ? -__builtin_inff() : 0.0f;
-}
-
-// Widen u and delta, apply bias/softplus, and start the output with the D*u skip term.  `n_valid` is how many
-// of the 8 items lie inside the row.
-template <typename in_t, bool kSoftplus>
-__device__ __forceinline__ void prepare_delta_u(const Raw8<in_t> &u_raw, const Raw8<in_t> &dl_raw, int n_valid,
-                                                float bias, float Dv, float (&dl)[kItems], float (&du)[kItems],
-                                                float (&y)[kItems]) {
-    float uv[kItems], raw[kItems], bias_items[kItems];
-    unpack_raw<in_t>(u_raw, uv);
-    unpack_raw<in_t>(dl_raw, raw);
-#pragma unroll
-    for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
-    delta_transform<kSoftplus>(raw, bias_items, dl);
-#pragma unroll
-    for (int i = 0; i < kItems; ++i) {
-        if constexpr (!kSoftplus) dl[i] = (i < n_valid) ? dl[i] : 0.0f;   // identity pair past the end of the row
-        du[i] = dl[i] * uv[i];                                            // u is 0 past the end
-        y[i] = Dv * uv[i];
-    }
-}
-
-template <typename in_t, bool kVec, bool kSoftplus>
-__device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_row, int pos, int L, float bias,
-                                             float Dv, float (&dl)[kItems], float (&du)[kItems], float (&y)[kItems]) {
-    const Raw8<in_t> u_raw = load_raw<in_t, kVec>(u_row, pos, L);
-    const Raw8<in_t> dl_raw = load_raw<in_t, kVec>(dl_row, pos, L, delta_fill<kSoftplus>());
-    prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
-}
-
 // ---- one wavefront per row ------------------------------------------------------------
 // kN == 1: the single state lives in registers and inputs are fetched in bursts.
 // kN == 0: any dstate; the per-wave states (running product, h) live in LDS, 2*dstate floats per wave: they
 //          are wave-uniform, and keeping 3*dstate of them in vector registers (tried for dstate 16) spills.
-// kGran consecutive elements through a buffer descriptor (32-bit offsets, hardware range check).
-template <typename T, int kGran>
-__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, uint32_t uniform_elem_offset,
-                                             float (&v)[kGran]) {
-    // elem_offset: per lane; uniform_elem_offset: the same for the whole wavefront (rides in a scalar register)
-    const int byte_off = (int)(elem_offset * (uint32_t)sizeof(T));
-    const int soff = (int)(uniform_elem_offset * (uint32_t)sizeof(T));
-    constexpr int kBytes = kGran * (int)sizeof(T);
-    uint32_t w[kBytes >= 4 ? kBytes / 4 : 1];
-    if constexpr (kBytes == 2) {
-        w[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_off, soff, 0);
-    } else if constexpr (kBytes == 4) {
-        w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_off, soff, 0);
-    } else if constexpr (kBytes == 8) {
-        const auto t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, byte_off, soff, 0);
-        w[0] = t[0]; w[1] = t[1];
-    } else if constexpr (kBytes == 16) {
-        const auto t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, soff, 0);
-        w[0] = t[0]; w[1] = t[1]; w[2] = t[2]; w[3] = t[3];
-    } else {
-        static_assert(kBytes == 32, "8 fp32 elements");
-        const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, soff, 0);
-        const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, soff, 0);
-        w[0] = t0[0]; w[1] = t0[1]; w[2] = t0[2]; w[3] = t0[3]; w[4] = t1[0]; w[5] = t1[1]; w[6] = t1[2]; w[7] = t1[3];
-    }
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-        for (int i = 0; i < kGran; ++i) v[i] = to_f32(T{(uint16_t)(w[i / 2] >> (16 * (i % 2)))});
-    } else {
-#pragma unroll
-        for (int i = 0; i < kGran; ++i) v[i] = bits_to_f32(w[i]);
-    }
-}
-
 template <typename in_t, typename out_t, int kN, bool kVec, bool kSoftplus>
 __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
