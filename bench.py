@@ -39,6 +39,11 @@ def scan_bytes(B, KD, L, N, K, s_in, s_out):
     return B * KD * L * (2 * s_in + s_out) + 2 * B * K * N * L * s_in + 4 * KD * (N + 2)
 
 
+def core_bytes(B, D, L, s_in, K=4):
+    """Algorithmic bytes of one fused-core launch: x in, the K delta rows in, merged fp32 y out; B, C rows; A, D, bias."""
+    return B * D * L * (s_in + K * s_in + 4) + 2 * B * K * L * s_in + 4 * K * D * 3
+
+
 def time_op(fn, reps, warm=5):
     import torch
     for _ in range(warm):
@@ -58,6 +63,7 @@ def kernel_lines(reps):
     BASELINE config 3 / config 4 operator shapes."""
     import torch
     import vmamba_amd as va
+    from vmamba_amd.core import core_fits, ss2d_core_hip
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(0)
     out = []
@@ -83,12 +89,22 @@ def kernel_lines(reps):
         t_sc = time_op(lambda: va.selective_scan_fn(u, delta, A, Bm, Cm, Dv, bias, True), reps)
         t_cm = time_op(lambda: va.cross_merge_fn(ys5), reps)
         b_cs, b_sc, b_cm = 5 * E * 2, scan_bytes(B, K * D, L, N, K, 2, 4), 5 * E * 4
+        fused = {}
+        if N == 1 and core_fits(H, W, x.dtype):
+            # the same work as ONE kernel; delta and B / C direction-major, batch-innermost
+            delta_k = delta.view(B, K, D, L).permute(1, 2, 0, 3).contiguous()
+            B_k, C_k = Bm.view(B, K, L).permute(1, 0, 2).contiguous(), Cm.view(B, K, L).permute(1, 0, 2).contiguous()
+            A1 = A.view(-1)
+            t_f = time_op(lambda: ss2d_core_hip(x, delta_k, B_k, C_k, A1, Dv, bias, True), reps)
+            b_f = core_bytes(B, D, L, 2)
+            fused = dict(core_fused_us=t_f * 1e6, core_fused_GBs=b_f / t_f / 1e9, core_fused_bytes=b_f)
+            del delta_k, B_k, C_k
         out.append(dict(shape=name, B=B, D=D, H=H, W=W, N=N,
                         cross_scan_us=t_cs * 1e6, cross_scan_GBs=b_cs / t_cs / 1e9,
                         scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9,
                         cross_merge_us=t_cm * 1e6, cross_merge_GBs=b_cm / t_cm / 1e9,
                         core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
-                        scan_bytes=b_sc))
+                        scan_bytes=b_sc, **fused))
         log("kernels", out[-1])
         del x, delta, Bm, Cm, xs, u, ys, ys5
     return out

@@ -52,9 +52,12 @@ def test_forward_core_fp32(d_model, d_state, ratio, H, W):
     x = torch.randn(2, ref.d_inner, H, W, generator=torch.Generator().manual_seed(1))
     with torch.no_grad():
         want = ref.forward_core(x)
-        got = hip.forward_core(x.to(DEV)).cpu()
-    assert got.shape == want.shape == x.shape and got.dtype == x.dtype
-    assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)
+    for fused in (True, False):       # one fused kernel (one-state models) / the three operators
+        hip.fused_core = fused
+        with torch.no_grad():
+            got = hip.forward_core(x.to(DEV)).cpu()
+        assert got.shape == want.shape == x.shape and got.dtype == x.dtype
+        assert torch.allclose(got, want, rtol=1e-3, atol=1e-3), f"fused={fused}"
 
 
 def test_forward_core_bf16_activations():
@@ -66,8 +69,11 @@ def test_forward_core_bf16_activations():
     x = torch.randn(4, 96, 56, 56, generator=torch.Generator().manual_seed(2)).bfloat16()
     with torch.no_grad():
         want = ref.forward_core(x).float()
-        got = hip.forward_core(x.to(DEV)).float().cpu()
-    assert torch.allclose(got, want, rtol=2e-2, atol=2e-2)
+    for fused in (True, False):
+        hip.fused_core = fused
+        with torch.no_grad():
+            got = hip.forward_core(x.to(DEV)).float().cpu()
+        assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), f"fused={fused}"
 
 
 def test_block_with_gate_matches():

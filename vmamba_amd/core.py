@@ -15,6 +15,18 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
+def core_fits(H, W, dtype):
+    """True when ss2d_core_fwd takes an H x W image of this dtype: at least 8 positions, and the LDS arrays of one
+    image (two fp32 merge planes and two copies of the x map, each with one spare word per 32) within 64 KiB."""
+    if dtype not in _DTYPE_CODE:
+        return False
+    L = H * W
+    es = 4 if dtype == torch.float32 else 2
+    plane = L + (L >> 5) + 2
+    xmap = plane if es == 4 else L + 2 * (L >> 6) + 2
+    return L >= 8 and 2 * plane * 4 + 2 * xmap * es <= 64 * 1024
+
+
 def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True):
     """x (B,D,H,W); delta (4,D,B,L) view; Bs, Cs (4,B,L) views (last stride 1), all of x.dtype and already in the
     scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32.

@@ -237,15 +237,17 @@ __device__ __forceinline__ void load_delta_u(const in_t *u_row, const in_t *dl_r
     prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
 }
 
-// kGran consecutive elements through a buffer descriptor (32-bit offsets, hardware range check).
+// kGran consecutive elements through a buffer descriptor (32-bit offsets, hardware range check), as loaded:
+// kGran * sizeof(T) bytes in 32-bit words (a lone 16-bit element sits in the low half of its word).
+template <typename T, int kGran> constexpr int gather_words() { return kGran * (int)sizeof(T) >= 4 ? kGran * (int)sizeof(T) / 4 : 1; }
+
 template <typename T, int kGran>
-__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, uint32_t uniform_elem_offset,
-                                             float (&v)[kGran]) {
+__device__ __forceinline__ void gather_group_raw(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, uint32_t uniform_elem_offset,
+                                                 uint32_t (&w)[gather_words<T, kGran>()]) {
     // elem_offset: per lane; uniform_elem_offset: the same for the whole wavefront (rides in a scalar register)
     const int byte_off = (int)(elem_offset * (uint32_t)sizeof(T));
     const int soff = (int)(uniform_elem_offset * (uint32_t)sizeof(T));
     constexpr int kBytes = kGran * (int)sizeof(T);
-    uint32_t w[kBytes >= 4 ? kBytes / 4 : 1];
     if constexpr (kBytes == 2) {
         w[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_off, soff, 0);
     } else if constexpr (kBytes == 4) {
@@ -262,6 +264,10 @@ __device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32
         const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, soff, 0);
         w[0] = t0[0]; w[1] = t0[1]; w[2] = t0[2]; w[3] = t0[3]; w[4] = t1[0]; w[5] = t1[1]; w[6] = t1[2]; w[7] = t1[3];
     }
+}
+
+template <typename T, int kGran>
+__device__ __forceinline__ void unpack_group(const uint32_t (&w)[gather_words<T, kGran>()], float (&v)[kGran]) {
     if constexpr (sizeof(T) == 2) {
 #pragma unroll
         for (int i = 0; i < kGran; ++i) v[i] = to_f32(T{(uint16_t)(w[i / 2] >> (16 * (i % 2)))});
@@ -269,6 +275,14 @@ __device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32
 #pragma unroll
         for (int i = 0; i < kGran; ++i) v[i] = bits_to_f32(w[i]);
     }
+}
+
+template <typename T, int kGran>
+__device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset, uint32_t uniform_elem_offset,
+                                             float (&v)[kGran]) {
+    uint32_t w[gather_words<T, kGran>()];
+    gather_group_raw<T, kGran>(rsrc, elem_offset, uniform_elem_offset, w);
+    unpack_group<T, kGran>(w, v);
 }
 
 }  // namespace ss2d

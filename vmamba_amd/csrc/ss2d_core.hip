@@ -4,17 +4,26 @@
 // The unfused path writes the four scan-ordered copies of x (xs), reads them back in the scan, writes the four
 // scan outputs (ys) and reads them back in the merge: 62 bytes per activation element at bf16-in / fp32-out.
 // Here a workgroup owns one channel d of CB images.  Its four wavefronts are the four scan directions:
-//   * the CB x maps are loaded once into LDS (odd row pitch); every wavefront reads u for ITS direction from
-//     there -- row-major, column-major, or either reversed -- so xs never exists;
+//   * the CB x maps are loaded once and kept in LDS twice, in row-major order (xR) and in column-major order
+//     (xT).  Direction 0 walks xR forwards, 2 walks it backwards, 1 walks xT forwards, 3 backwards: every
+//     wavefront reads the u of ITS scan order with plain index arithmetic, and xs never exists;
 //   * delta (from dt_proj) and the B / C rows (from x_proj) are streamed from HBM / L2 exactly as in the scan
 //     kernels: 8 positions per lane, DPP wavefront scan, state carried in a register, softplus fused;
-//   * each wavefront adds its outputs into two fp32 LDS planes at the position the merge wants them: plane A
-//     (row-major index) collects directions 0 and 2, plane B (column-major index, odd pitch) directions 1 and 3.
-//     Each plane entry receives exactly two adds onto an initial 0, so the result is fl(y0 + y2) resp. fl(y1 + y3)
-//     whatever order the LDS atomics land in -- the association order of cross_merge_fwd
-//     (classification/models/csm_triton.py:61-62) -- and ys never exists;
+//   * each wavefront puts its outputs into an fp32 LDS plane at the position the merge wants them: plane A
+//     (row-major index) collects directions 0 and 2, plane B (column-major index) directions 1 and 3.  Every
+//     plane entry has exactly two writers, one forward and one backward direction; whichever comes first
+//     stores, the other adds, giving fl(y0 + y2) resp. fl(y1 + y3) -- the association order of cross_merge_fwd
+//     (classification/models/csm_triton.py:61-62) -- and ys never exists.  LDS float atomics are an order of
+//     magnitude slower than plain LDS traffic on this chip, so the order is fixed by construction instead: the
+//     four wavefronts advance pass by pass, in each pass the forward directions update the planes, a barrier,
+//     then the backward directions, a barrier; "who is first" follows from the pass in which the other
+//     direction reaches the same entry;
 //   * finally out[r] = A[r] + B[t(r)] is written once.
 // HBM traffic per element: x (s_in) + 4 delta (4 s_in) + out (s_out) = 14 bytes instead of 62.
+//
+// LDS banks: a lane owns 8 consecutive positions, so for a fixed item the 64 lanes touch addresses 8 apart, which
+// would fold onto 4 of the 32 banks.  All four LDS arrays therefore skip one 4-byte word after every 32 words
+// (lds_index): lanes 0..31 of one access then fall into 32 different banks.
 //
 // The CB images of a workgroup are walked as one stream per direction (restart by a = 0 at each image start, as
 // in the flat scan kernel), which needs their delta rows adjacent in memory: delta is therefore taken with
@@ -28,114 +37,190 @@ struct CoreArgs {
     const void *x, *delta, *Bm, *Cm;
     const float *A, *Dv, *bias;
     void *y;
-    int32_t B, D, H, W, L, CB, Wp, Hp, softplus, vec_ok;
+    int32_t B, D, H, W, L, CB, softplus, vec_ok;
     int64_t dl_ks, dl_ds, dl_bs;        // delta strides over direction, channel, batch (elements)
     int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
     uint32_t B_span_bytes, C_span_bytes;
 };
 
-// Walks the spatial position that scan position j of direction kDir reads / writes.
-//   directions 0, 2: row-major index s = h*W + w  -> (q, r) = (h, w), inner extent W
-//   directions 1, 3: column-major index s = w*H + h -> (q, r) = (w, h), inner extent H
-//   directions 0, 1 walk s upwards from 0, directions 2, 3 downwards from L-1.
-template <int kDir>
-struct Walker {
-    int q, r;
-    __device__ __forceinline__ void init(int j, int L, FastDiv div_inner) {
-        const uint32_t s = (kDir < 2) ? (uint32_t)j : (uint32_t)(L - 1 - j);
-        uint32_t qq, rr;
-        divmod(s, div_inner, qq, rr);
-        q = (int)qq; r = (int)rr;
-    }
-    __device__ __forceinline__ void restart(int outer, int inner) {       // first scan position of an image
-        q = (kDir < 2) ? 0 : outer - 1;
-        r = (kDir < 2) ? 0 : inner - 1;
-    }
-    __device__ __forceinline__ void step(int inner) {
-        if (kDir < 2) { ++r; const bool c = r == inner; r = c ? 0 : r; q += c ? 1 : 0; }
-        else { --r; const bool c = r < 0; r = c ? inner - 1 : r; q -= c ? 1 : 0; }
-    }
+// Index of logical element a in an LDS array of kBytes-wide elements that skips one word after every 32 words.
+template <int kBytes> __host__ __device__ __forceinline__ constexpr int lds_index(int a) {
+    static_assert(kBytes == 2 || kBytes == 4, "16-bit or 32-bit elements");
+    return kBytes == 4 ? a + (a >> 5) : a + ((a >> 6) << 1);
+}
+// Elements to allocate for n logical elements (a multiple of 16 bytes).
+template <int kBytes> __host__ __device__ __forceinline__ constexpr int lds_extent(int n) {
+    return (lds_index<kBytes>(n) + 8) & ~7;
+}
+
+constexpr int kCoreBurst = 4;     // passes whose delta / B / C loads are in flight per wavefront
+
+// What one pass of one lane loads from memory, as it arrives.
+template <typename in_t, int kGran>
+struct CorePassLoads {
+    static constexpr int kGroups = kItems / kGran;
+    static constexpr int kWords = gather_words<in_t, kGran>();
+    Raw8<in_t> dl;
+    uint32_t b[kGroups][kWords], c[kGroups][kWords];
+    uint32_t i0, j0;      // image and position of the lane's first item
 };
 
-template <typename in_t, int kDir, bool kSoftplus, int kGran>
-__device__ __forceinline__ void core_scan_direction(const CoreArgs &p, int d, int b0, int nb, const in_t *xmap, float *planeA,
-                                                    float *planeB, FastDiv divL, FastDiv divW, FastDiv divH) {
+template <typename in_t, bool kSoftplus, int kGran>
+__global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD) {
+    extern __shared__ __align__(16) float core_smem[];
+    constexpr int kEs = (int)sizeof(in_t);
     constexpr int kGroups = kItems / kGran;
-    constexpr bool kRowMajor = (kDir % 2) == 0;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int L = p.L, H = p.H, W = p.W, Wp = p.Wp, Hp = p.Hp;
-    const int inner = kRowMajor ? W : H, outer = kRowMajor ? H : W;
-    const FastDiv div_inner = kRowMajor ? divW : divH;
-    const int Lp = H * Wp, WHp = W * Hp;
+    using Loads = CorePassLoads<in_t, kGran>;
+    const int L = p.L, H = p.H;
+    const int n_max = p.CB * L;
+    const int plane_ext = lds_extent<4>(n_max), map_ext = lds_extent<kEs>(n_max);
+    float *planeA = core_smem;                           // fl(y0 + y2), row-major index
+    float *planeB = planeA + plane_ext;                  // fl(y1 + y3), column-major index
+    in_t *xR = reinterpret_cast<in_t *>(planeB + plane_ext);
+    in_t *xT = xR + map_ext;
+
+    uint32_t bt, d;
+    divmod(blockIdx.x, divD, bt, d);                     // neighbouring workgroups share B / C rows (same images)
+    const int b0 = (int)bt * p.CB;
+    const int nb = min(p.CB, p.B - b0);
     const int n_el = nb * L;
-    const int kd = kDir * p.D + d;
-    const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + kDir * p.dl_ks + d * p.dl_ds + b0 * p.dl_bs;
+
+    // ---- this wavefront's direction ---------------------------------------------------------------------------
+    const int lane = threadIdx.x & (kWave - 1);
+    const int dir = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const bool reverse = dir >= 2;
+    const in_t *xs = (dir & 1) ? xT : xR;
+    float *plane = (dir & 1) ? planeB : planeA;
+    const int kd = dir * p.D + (int)d;
+    const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + dir * p.dl_ks + (int64_t)d * p.dl_ds + b0 * p.dl_bs;
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bm), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Cm), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
-    const uint32_t B_soff = (uint32_t)(kDir * p.B_ks + b0 * p.B_bs), C_soff = (uint32_t)(kDir * p.C_ks + b0 * p.C_bs);
+    const uint32_t B_soff = (uint32_t)(dir * p.B_ks + b0 * p.B_bs), C_soff = (uint32_t)(dir * p.C_ks + b0 * p.C_bs);
     const float A_log2e = p.A[kd] * kLog2e;
     const float Dv = p.Dv ? p.Dv[kd] : 0.0f;
     const float bias = p.bias ? p.bias[kd] : 0.0f;
-    float *plane = kRowMajor ? planeA : planeB;
-    const int plane_img = kRowMajor ? L : WHp;          // plane elements per image
-    const int plane_pitch = kRowMajor ? W : Hp;
-
-    float h_carry = 0.0f;
     const int n_pass = (n_el + kPass - 1) / kPass;
-    for (int pass = 0; pass < n_pass; ++pass) {
+
+    auto issue = [&](int pass, Loads &r) {
         const int e0 = pass * kPass + lane * kItems;
-        const bool full = e0 + kItems <= n_el;
-        float raw[kItems];
-        if (full && p.vec_ok) load_items<in_t, true>(dl_base, e0, n_el, raw, delta_fill<kSoftplus>());
-        else load_items<in_t, false>(dl_base, e0, n_el, raw, delta_fill<kSoftplus>());
-
-        uint32_t i0, j0;
-        divmod((uint32_t)min(e0, n_el - 1), divL, i0, j0);
-        const int k = kGran == kItems ? kItems : min(kItems, L - (int)j0);     // items before the next image starts
-
-        // u from the LDS maps, and where each output goes in the merge planes
-        Walker<kDir> wk;
-        wk.init((int)j0, L, div_inner);
-        int img = (int)i0;
-        float uv[kItems];
-        int paddr[kItems];
+        if (e0 + kItems <= n_el && p.vec_ok) r.dl = load_raw<in_t, true>(dl_base, e0, n_el, delta_fill<kSoftplus>());
+        else r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
+        divmod((uint32_t)min(e0, n_el - 1), divL, r.i0, r.j0);
+        const int k = kGran == kItems ? kItems : min(kItems, L - (int)r.j0);   // items before the next image starts
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) {
-            if constexpr (kGran != kItems) {
-                if (i % kGran == 0) {                       // an image can only start at a group boundary
-                    const bool wrap = i == k;
-                    if (wrap) { wk.restart(outer, inner); }
-                    img += wrap ? 1 : 0;
+        for (int gi = 0; gi < kGroups; ++gi) {
+            const bool in_a = kGran == kItems ? true : gi * kGran < k;
+            const uint32_t ig = r.i0 + (in_a ? 0u : 1u);
+            const uint32_t jg = in_a ? r.j0 + gi * kGran : (uint32_t)(gi * kGran - k);
+            gather_group_raw<in_t, kGran>(B_rsrc, ig * (uint32_t)p.B_bs + jg, B_soff, r.b[gi]);
+            gather_group_raw<in_t, kGran>(C_rsrc, ig * (uint32_t)p.C_bs + jg, C_soff, r.c[gi]);
+        }
+    };
+
+    // the first passes' loads fly while the maps are staged
+    Loads regs[kCoreBurst];
+#pragma unroll
+    for (int q = 0; q < kCoreBurst; ++q)
+        if (q < n_pass) issue(q, regs[q]);
+
+    // ---- stage: copy the maps into xR / xT ------------------------------------------------------------------------
+    const in_t *xin = reinterpret_cast<const in_t *>(p.x);
+    if constexpr (kGran == kItems && sizeof(in_t) == 2) {
+        // rows are multiples of 8 elements (and 16-byte aligned, host-checked through kGran): 16-byte loads
+        const int n_vec = n_el / kItems;
+        for (int base = 0; base < n_vec; base += 2 * kBlock) {
+            uint4 v[2];
+            uint32_t ii[2], rr[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int vi = base + u * kBlock + (int)threadIdx.x;
+                divmod((uint32_t)min(vi, n_vec - 1) * kItems, divL, ii[u], rr[u]);
+                v[u] = *reinterpret_cast<const uint4 *>(xin + ((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int vi = base + u * kBlock + (int)threadIdx.x;
+                if (vi < n_vec) {
+                    const uint32_t w32[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+                    uint32_t h, w;
+                    divmod(rr[u], divW, h, w);
+                    const int at_r = vi * kItems;
+                    int at_t = (int)(ii[u] * L + w * H + h);
+#pragma unroll
+                    for (int i = 0; i < kItems; ++i) {
+                        const in_t e = in_t{(uint16_t)(w32[i / 2] >> (16 * (i % 2)))};
+                        xR[lds_index<kEs>(at_r + i)] = e;
+                        xT[lds_index<kEs>(at_t)] = e;
+                        ++w;                                   // next column, wrapping to the next row
+                        at_t += H;
+                        if ((int)w == p.W) { w = 0; ++h; at_t = (int)(ii[u] * L + h); }
+                    }
                 }
             }
-            const bool valid = e0 + i < n_el;
-            const int xoff = img * Lp + (kRowMajor ? wk.q * Wp + wk.r : wk.r * Wp + wk.q);
-            uv[i] = valid ? to_f32(xmap[valid ? xoff : 0]) : 0.0f;
-            paddr[i] = img * plane_img + wk.q * plane_pitch + wk.r;
-            wk.step(inner);
         }
-
-        float dl[kItems], bias_items[kItems];
+    } else {
+        constexpr int kChunk = 8;
+        for (int base = 0; base < n_el; base += kChunk * kBlock) {
+            in_t v[kChunk];
+            uint32_t ii[kChunk], rr[kChunk];
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
-        delta_transform<kSoftplus>(raw, bias_items, dl);
+            for (int u = 0; u < kChunk; ++u) {
+                const int idx = base + u * kBlock + (int)threadIdx.x;
+                divmod((uint32_t)min(idx, n_el - 1), divL, ii[u], rr[u]);
+                v[u] = xin[((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]];
+            }
+#pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const int idx = base + u * kBlock + (int)threadIdx.x;
+                if (idx < n_el) {
+                    uint32_t h, w;
+                    divmod(rr[u], divW, h, w);
+                    xR[lds_index<kEs>(idx)] = v[u];
+                    xT[lds_index<kEs>((int)(ii[u] * L + w * H + h))] = v[u];
+                }
+            }
+        }
+    }
+    __syncthreads();
 
-        // B, C rows of (direction, image): group gathers
-        float Bv[kItems], Cv[kItems];
+    // ---- scan: 8 positions per lane per pass, loads kCoreBurst passes ahead ---------------------------------------
+    // Returns the pass's outputs in yv and their plane positions in at (logical index in this direction's order).
+    auto compute = [&](int pass, const Loads &r, float &h_carry, float (&yv)[kItems], int (&at)[kItems], int &img_of_b) {
+        const int e0 = pass * kPass + lane * kItems;
+        const int j0 = (int)r.j0, i0 = (int)r.i0;
+        const int k = kGran == kItems ? kItems : min(kItems, L - j0);
+        float raw[kItems], Bv[kItems], Cv[kItems];
+        unpack_raw<in_t>(r.dl, raw);
         bool first[kGroups];
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             const bool in_a = kGran == kItems ? true : gi * kGran < k;
-            const uint32_t ig = i0 + (in_a ? 0u : 1u);
-            const uint32_t jg = in_a ? j0 + gi * kGran : (uint32_t)(gi * kGran - k);
-            first[gi] = jg == 0;
+            first[gi] = (in_a ? j0 + gi * kGran : gi * kGran - k) == 0;
             float bg[kGran], cg[kGran];
-            gather_group<in_t, kGran>(B_rsrc, ig * (uint32_t)p.B_bs + jg, B_soff, bg);
-            gather_group<in_t, kGran>(C_rsrc, ig * (uint32_t)p.C_bs + jg, C_soff, cg);
+            unpack_group<in_t, kGran>(r.b[gi], bg);
+            unpack_group<in_t, kGran>(r.c[gi], cg);
 #pragma unroll
             for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
         }
-
+        // u from LDS.  Forwards the logical index is the stream position e0 + i; backwards it is img*L + L-1-j.
+        const int step = reverse ? -1 : 1;
+        const int at_a = reverse ? i0 * L + L - 1 - j0 : e0;                 // items of image i0:     at_a + step*i
+        const int at_b = reverse ? (i0 + 1) * L + L - 1 + k : e0;            // items of image i0 + 1: at_b + step*i
+        img_of_b = k;
+        float uv[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const bool valid = e0 + i < n_el;
+            int a = ((kGran == kItems || i < k) ? at_a : at_b) + step * i;
+            a = valid ? a : 0;
+            at[i] = a;
+            const in_t v = xs[lds_index<kEs>(a)];
+            uv[i] = valid ? to_f32(v) : 0.0f;
+        }
+        float dl[kItems], bias_items[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
+        delta_transform<kSoftplus>(raw, bias_items, dl);
         float ac[kItems], hh[kItems];
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
@@ -151,57 +236,69 @@ __device__ __forceinline__ void core_scan_direction(const CoreArgs &p, int d, in
         const float s_in = fmaf(a_ex, h_carry, h_ex);
         h_carry = fmaf(a_tot, h_carry, h_tot);
 #pragma unroll
+        for (int i = 0; i < kItems; ++i) yv[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), Dv * uv[i]);
+    };
+
+    // Plane update of one pass.  An entry at logical index a of image img is written by the forward direction in
+    // pass a / 512 and by the backward direction in pass (2*img*L + L-1 - a) / 512 (its stream position there is
+    // the mirror image of a within the image).  The earlier pass stores, the later one adds; in the same pass the
+    // forward direction goes first (the barrier between the two halves of a pass orders them).
+    auto update_plane = [&](int pass, const Loads &r, const float (&yv)[kItems], const int (&at)[kItems], int k) {
+        const int e0 = pass * kPass + lane * kItems;
+        const int i0 = (int)r.i0;
+#pragma unroll
         for (int i = 0; i < kItems; ++i) {
-            const float yv = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), Dv * uv[i]);
-            if (e0 + i < n_el) __hip_atomic_fetch_add(plane + paddr[i], yv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (e0 + i < n_el) {
+                const int img = (kGran == kItems || i < k) ? i0 : i0 + 1;
+                const int other_pos = reverse ? at[i] : 2 * img * L + L - 1 - at[i];     // the other direction's stream position
+                const int other_pass = (int)((uint32_t)other_pos / (uint32_t)kPass);
+                const bool add = reverse ? other_pass <= pass : other_pass < pass;
+                float *slot = plane + lds_index<4>(at[i]);
+                const float old = *slot;
+                *slot = add ? old + yv[i] : yv[i];
+            }
+        }
+    };
+
+    float h_carry = 0.0f;
+    for (int pass0 = 0; pass0 < n_pass; pass0 += kCoreBurst) {
+#pragma unroll
+        for (int q = 0; q < kCoreBurst; ++q) {
+            const int pass = pass0 + q;
+            if (pass < n_pass) {                     // uniform over the workgroup: every wavefront meets every barrier
+                float yv[kItems];
+                int at[kItems], k;
+                compute(pass, regs[q], h_carry, yv, at, k);
+                if (!reverse) update_plane(pass, regs[q], yv, at, k);
+                __syncthreads();
+                if (reverse) update_plane(pass, regs[q], yv, at, k);
+                __syncthreads();
+                if (pass + kCoreBurst < n_pass) issue(pass + kCoreBurst, regs[q]);
+            }
         }
     }
-}
 
-template <typename in_t, bool kSoftplus, int kGran>
-__global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divH,
-                                                           FastDiv divD) {
-    extern __shared__ __align__(16) float core_smem[];
-    const int L = p.L, H = p.H, W = p.W;
-    const int Lp = H * p.Wp, WHp = W * p.Hp;
-    float *planeA = core_smem;                           // [CB][L]
-    float *planeB = planeA + p.CB * L;                   // [CB][W*Hp]
-    in_t *xmap = reinterpret_cast<in_t *>(planeB + p.CB * WHp);   // [CB][H*Wp]
-
-    uint32_t bt, d;
-    divmod(blockIdx.x, divD, bt, d);                     // neighbouring workgroups share B / C rows (same images)
-    const int b0 = (int)bt * p.CB;
-    const int nb = min(p.CB, p.B - b0);
-    const int n_el = nb * L;
-
-    for (int idx = threadIdx.x; idx < p.CB * (L + WHp); idx += kBlock) core_smem[idx] = 0.0f;
-    const in_t *xin = reinterpret_cast<const in_t *>(p.x);
-    for (int idx = threadIdx.x; idx < n_el; idx += kBlock) {
-        uint32_t i, r, h, w;
-        divmod((uint32_t)idx, divL, i, r);
-        divmod(r, divW, h, w);
-        xmap[i * Lp + h * p.Wp + w] = xin[((size_t)(b0 + i) * p.D + d) * L + r];
-    }
-    __syncthreads();
-
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    switch (wave) {
-        case 0: core_scan_direction<in_t, 0, kSoftplus, kGran>(p, (int)d, b0, nb, xmap, planeA, planeB, divL, divW, divH); break;
-        case 1: core_scan_direction<in_t, 1, kSoftplus, kGran>(p, (int)d, b0, nb, xmap, planeA, planeB, divL, divW, divH); break;
-        case 2: core_scan_direction<in_t, 2, kSoftplus, kGran>(p, (int)d, b0, nb, xmap, planeA, planeB, divL, divW, divH); break;
-        default: core_scan_direction<in_t, 3, kSoftplus, kGran>(p, (int)d, b0, nb, xmap, planeA, planeB, divL, divW, divH); break;
-    }
-    __syncthreads();
-
+    // ---- merge: out[r] = A[r] + B[t(r)] ---------------------------------------------------------------------------
     float *yo = reinterpret_cast<float *>(p.y);
-    for (int idx = threadIdx.x; idx < n_el; idx += kBlock) {
-        uint32_t i, r, h, w;
-        divmod((uint32_t)idx, divL, i, r);
-        divmod(r, divW, h, w);
-        const float v = planeA[i * L + r] + planeB[i * WHp + w * p.Hp + h];
-        yo[((size_t)(b0 + i) * p.D + d) * L + r] = v;
+    for (int base = 0; base < n_el; base += 4 * kBlock) {
+        float v[4];
+        size_t off[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int idx = min(base + u * kBlock + (int)threadIdx.x, n_el - 1);
+            uint32_t i, r, h, w;
+            divmod((uint32_t)idx, divL, i, r);
+            divmod(r, divW, h, w);
+            v[u] = planeA[lds_index<4>(idx)] + planeB[lds_index<4>((int)(i * L + w * H + h))];
+            off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (base + u * kBlock + (int)threadIdx.x < n_el) yo[off[u]] = v[u];
     }
 }
+
+constexpr size_t kCoreMaxLds = 64 * 1024;
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
 
@@ -216,11 +313,14 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     CB = (CB + align_rows - 1) / align_rows * align_rows;
     if (CB >= a.B) CB = a.B;                                  // a single tile starts at image 0
     if (CB > 1 && a.dl_bs != L) CB = 1;                       // adjacent delta rows need the batch-innermost layout
+    auto lds_bytes = [&](int64_t cb) {
+        const int n = (int)(cb * L);
+        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)lds_extent<(int)sizeof(in_t)>(n) * sizeof(in_t);
+    };
+    while (CB > 1 && lds_bytes(CB) > kCoreMaxLds) CB = CB > align_rows ? CB - align_rows : 1;
+    const size_t smem = lds_bytes(CB);
+    if (smem > kCoreMaxLds) return SS2D_ENOTSUP;
     a.CB = (int)CB;
-    a.Wp = a.W | 1;
-    a.Hp = a.H | 1;
-    const size_t smem = (size_t)CB * ((size_t)L + (size_t)a.W * a.Hp) * sizeof(float) + (size_t)CB * a.H * a.Wp * sizeof(in_t);
-    if (smem > 64 * 1024) return SS2D_ENOTSUP;
     // 16-byte loads of the delta stream need every (direction, channel, first image of a workgroup) start aligned;
     // otherwise the kernel loads element-wise
     const int64_t vec = 16 / (int64_t)sizeof(in_t);
@@ -235,10 +335,9 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t tiles = (a.B + CB - 1) / CB;
     const int64_t n_wg = tiles * a.D;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-    const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dH = make_fastdiv((uint32_t)a.H),
-                  dD = make_fastdiv((uint32_t)a.D);
+    const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dD = make_fastdiv((uint32_t)a.D);
 #define SS2D_CORE_LAUNCH(SP, G) \
-    hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dH, dD)
+    hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD)
     if (a.softplus) {
         if (g == 8) SS2D_CORE_LAUNCH(true, 8); else if (g == 4) SS2D_CORE_LAUNCH(true, 4); else SS2D_CORE_LAUNCH(true, 1);
     } else {
@@ -274,7 +373,7 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     const int64_t B_span = (3 * a.B_ks + (int64_t)(a.B - 1) * a.B_bs + L) * eb, C_span = (3 * a.C_ks + (int64_t)(a.B - 1) * a.C_bs + L) * eb;
     if (B_span >= 0x7fffffffll || C_span >= 0x7fffffffll) return SS2D_ENOTSUP;
     a.B_span_bytes = (uint32_t)B_span; a.C_span_bytes = (uint32_t)C_span;
-    a.CB = 1; a.Wp = 0; a.Hp = 0; a.vec_ok = 0;
+    a.CB = 1; a.vec_ok = 0;
 
     hipStream_t s = (hipStream_t)stream;
     if (q->in_dtype == SS2D_F32) return launch_core<float>(a, s);

@@ -20,7 +20,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .csm import cross_merge_fn, cross_scan_fn
+from .core import core_fits, ss2d_core_hip
+from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
 from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip
@@ -83,9 +84,10 @@ class SS2D(nn.Module):
 
     def __init__(self, d_model=96, d_state=1, ssm_ratio=1.0, dt_rank="auto", d_conv=3, conv_bias=False, bias=False,
                  disable_z=True, dt_min=0.001, dt_max=0.1, dt_scale=1.0, dt_init_floor=1e-4, channel_first=True,
-                 layers=HipLayers):
+                 layers=HipLayers, fused_core=True):
         super().__init__()
         self.channel_first = channel_first
+        self.fused_core = fused_core
         self.layers = layers
         Linear = Linear2d if channel_first else nn.Linear
         self.k_group = 4
@@ -118,6 +120,7 @@ class SS2D(nn.Module):
         K = self.k_group
         consts = dict(
             As=-self.A_logs.float().exp(), Ds=self.Ds.float(), dt_bias=self.dt_projs_bias.reshape(-1).float(),
+            Wx_all=self.x_proj_weight.reshape(1, -1, self.d_inner).expand(batch, -1, -1).contiguous(),
             Wx=self.x_proj_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, -1, self.d_inner).contiguous(),
             Wdt=self.dt_projs_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, self.d_inner, -1).contiguous())
         if not torch.is_grad_enabled():
@@ -139,10 +142,30 @@ class SS2D(nn.Module):
         dts = torch.bmm(consts["Wdt"], dts.reshape(B * K, R, L)).view(B, K * D, L)
         return dts, Bs, Cs
 
+    def forward_core_fused(self, x, consts):
+        """One state per channel: the three operators as ONE kernel (ss2d_core_fwd).
+
+        A projection is a per-position contraction, so x_proj is applied to x in its natural order for all four
+        directions at once, and only its small output (R + 2 rows per direction instead of D) is put into scan
+        order -- direction-major and batch-innermost, which makes dt_proj ONE GEMM per direction over all B*L
+        positions and hands the kernel delta rows of consecutive images side by side.
+        """
+        B, D, H, W = x.shape
+        K, L, R = self.k_group, H * W, self.dt_rank
+        C = R + 2
+        proj = torch.bmm(consts["Wx_all"], x.view(B, D, L))                                   # (B, K*C, L)
+        x_dbl = proj.new_empty((K, C, B, L))
+        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl.permute(2, 0, 1, 3))
+        delta = torch.bmm(self.dt_projs_weight, x_dbl[:, :R].reshape(K, R, B * L)).view(K, D, B, L)
+        return ss2d_core_hip(x, delta, x_dbl[:, R], x_dbl[:, R + 1], consts["As"].view(-1), consts["Ds"],
+                             consts["dt_bias"], True)
+
     def forward_core(self, x):
         B, D, H, W = x.shape
         K, L = self.k_group, H * W
         consts = self._inference_constants(B)
+        if self.d_state == 1 and self.fused_core and core_fits(H, W, x.dtype):
+            return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
         dts, Bs, Cs = self.project(xs, consts)
         ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
