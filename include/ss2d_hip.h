@@ -190,6 +190,17 @@ typedef struct ss2d_core_params {
 
 int ss2d_core_fwd(const ss2d_core_params *params, void *stream);
 
+/*
+ * dt_proj of the SS2D core: the per-direction rank-R -> D projection between x_proj and the scan.
+ * Replaces the grouped conv1d / einsum of SS2Dv2.forward_corev2 (classification/models/vmamba.py:608-609, 614-615):
+ *   delta[k, d, n] = sum_r weight[k, d, r] * x[k*x_dir_stride + r*x_rank_stride + n]
+ *   weight (K, D, R) contiguous; delta (K, D, N) contiguous; x rows contiguous along n (N = batch * L positions).
+ * dtype SS2D_BF16 or SS2D_F16 for all three tensors; products accumulate in fp32 on the matrix cores and are
+ * rounded once to dtype, as in the library GEMM.  SS2D_F32 and R > 48 return SS2D_ENOTSUP (use a library GEMM).
+ */
+int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, int R, int64_t N, int64_t x_dir_stride,
+                 int64_t x_rank_stride, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

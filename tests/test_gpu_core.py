@@ -180,3 +180,43 @@ def test_cross_scan_1b1_empty_and_bad_args():
         va.cross_scan_fn(torch.zeros(2, 3, 3, 4, 4, device=DEV), one_by_one=True)
     with pytest.raises(NotImplementedError):
         va.cross_scan_fn(torch.zeros(2, 4, 3, 4, 4), one_by_one=True)
+
+
+# ---- dt_proj on the matrix cores -----------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("K,D,R,N", [(4, 96, 6, 2 * 3136), (4, 192, 12, 3 * 784), (4, 384, 24, 5 * 196), (4, 768, 48, 7 * 49),
+                                     (2, 40, 3, 77), (1, 100, 17, 1000), (3, 33, 8, 32), (4, 8, 40, 5)])
+def test_dt_proj_matches_fp32_matmul(K, D, R, N, dtype):
+    """One rounding of an fp32-accumulated sum of exact 16-bit products: against the fp32 matmul of the same
+    16-bit operands the result is within one rounding of the output type (plus fp32 summation-order noise)."""
+    from vmamba_amd.core import dt_proj_hip
+    _announce("dt_proj", K, D, R, N, dtype)
+    g = torch.Generator().manual_seed(K * 1000 + D + R)
+    x = torch.randn(K, R, N, generator=g).to(dtype)
+    w = (torch.randn(K, D, R, generator=g) * R ** -0.5).to(dtype)
+    want = torch.bmm(w.float(), x.float())
+    got = dt_proj_hip(x.to(DEV), w.to(DEV))
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == (K, D, N)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11          # half an ulp, relative
+    err = (got.cpu().float() - want).abs()
+    assert bool((err <= eps * want.abs() * 1.01 + 1e-6).all()), f"max err {err.max().item()}"
+    # rows taken through strides: the dts slice of a (K, C, N) projection output
+    C = R + 2
+    x_dbl = torch.randn(K, C, N, generator=g).to(dtype).to(DEV)
+    got2 = dt_proj_hip(x_dbl[:, :R], w.to(DEV))
+    want2 = torch.bmm(w.float(), x_dbl[:, :R].cpu().float())
+    err2 = (got2.cpu().float() - want2).abs()
+    assert bool((err2 <= eps * want2.abs() * 1.01 + 1e-6).all())
+
+
+def test_dt_proj_rejections():
+    from vmamba_amd.core import dt_proj_hip
+    with pytest.raises(RuntimeError):
+        dt_proj_hip(torch.zeros(4, 6, 64, device=DEV), torch.zeros(4, 96, 6, device=DEV))              # fp32: library GEMM
+    with pytest.raises(_lib.Ss2dError) as e:
+        dt_proj_hip(torch.zeros(1, 64, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(1, 8, 64, device=DEV, dtype=torch.bfloat16))
+    assert e.value.code == _lib.SS2D_ENOTSUP
+    assert dt_proj_hip(torch.zeros(4, 6, 0, device=DEV, dtype=torch.bfloat16),
+                       torch.zeros(4, 96, 6, device=DEV, dtype=torch.bfloat16)).shape == (4, 96, 0)

@@ -15,7 +15,8 @@ SCAN_CHUNK = 2048
 ABI_VERSION = 1
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
-           "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd")
+           "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
+           "ss2d_dt_proj")
 
 
 class ScanParams(ctypes.Structure):
@@ -81,6 +82,9 @@ def lib():
                                           + [ctypes.c_void_p])
         L.ss2d_core_fwd.restype = ctypes.c_int
         L.ss2d_core_fwd.argtypes = [ctypes.POINTER(CoreParams), ctypes.c_void_p]
+        L.ss2d_dt_proj.restype = ctypes.c_int
+        L.ss2d_dt_proj.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_int64] * 3 + [ctypes.c_int]
+                                   + [ctypes.c_void_p])
         if L.ss2d_abi_version() != ABI_VERSION:
             raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L

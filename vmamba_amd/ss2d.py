@@ -20,7 +20,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .core import core_fits, ss2d_core_hip
+from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
@@ -156,7 +156,11 @@ class SS2D(nn.Module):
         proj = torch.bmm(consts["Wx_all"], x.view(B, D, L))                                   # (B, K*C, L)
         x_dbl = proj.new_empty((K, C, B, L))
         cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl.permute(2, 0, 1, 3))
-        delta = torch.bmm(self.dt_projs_weight, x_dbl[:, :R].reshape(K, R, B * L)).view(K, D, B, L)
+        dts = x_dbl[:, :R].reshape(K, R, B * L)
+        if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
+            delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, B, L)
+        else:
+            delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, B, L)
         return ss2d_core_hip(x, delta, x_dbl[:, R], x_dbl[:, R + 1], consts["As"].view(-1), consts["Ds"],
                              consts["dt_bias"], True)
 
