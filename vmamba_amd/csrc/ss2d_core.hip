@@ -101,19 +101,27 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     const float bias = p.bias ? p.bias[kd] : 0.0f;
     const int n_pass = (n_el + kPass - 1) / kPass;
 
+    // Image and position of this lane's first item in the pass issued next: passes are issued strictly in order, so
+    // the pair just advances by 512 positions each time (no division in the loop).
+    uint32_t next_i, next_j, step_i, step_j;
+    divmod((uint32_t)(lane * kItems), divL, next_i, next_j);
+    divmod((uint32_t)kPass, divL, step_i, step_j);
     auto issue = [&](int pass, Loads &r) {
         const int e0 = pass * kPass + lane * kItems;
         if (e0 + kItems <= n_el && p.vec_ok) r.dl = load_raw<in_t, true>(dl_base, e0, n_el, delta_fill<kSoftplus>());
         else r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
-        divmod((uint32_t)min(e0, n_el - 1), divL, r.i0, r.j0);
+        r.i0 = next_i; r.j0 = next_j;
+        next_i += step_i; next_j += step_j;
+        if (next_j >= (uint32_t)L) { next_j -= (uint32_t)L; next_i += 1; }
         const int k = kGran == kItems ? kItems : min(kItems, L - (int)r.j0);   // items before the next image starts
+        const uint32_t B_a = r.i0 * (uint32_t)p.B_bs + r.j0, C_a = r.i0 * (uint32_t)p.C_bs + r.j0;   // image i0
+        const uint32_t B_b = B_a + (uint32_t)p.B_bs - (uint32_t)(r.j0 + k), C_b = C_a + (uint32_t)p.C_bs - (uint32_t)(r.j0 + k);
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             const bool in_a = kGran == kItems ? true : gi * kGran < k;
-            const uint32_t ig = r.i0 + (in_a ? 0u : 1u);
-            const uint32_t jg = in_a ? r.j0 + gi * kGran : (uint32_t)(gi * kGran - k);
-            gather_group_raw<in_t, kGran>(B_rsrc, ig * (uint32_t)p.B_bs + jg, B_soff, r.b[gi]);
-            gather_group_raw<in_t, kGran>(C_rsrc, ig * (uint32_t)p.C_bs + jg, C_soff, r.c[gi]);
+            // image i0: position j0 + gi*kGran; image i0 + 1: position gi*kGran - k
+            gather_group_raw<in_t, kGran>(B_rsrc, (in_a ? B_a : B_b) + gi * kGran, B_soff, r.b[gi]);
+            gather_group_raw<in_t, kGran>(C_rsrc, (in_a ? C_a : C_b) + gi * kGran, C_soff, r.c[gi]);
         }
     };
 
@@ -184,38 +192,53 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     __syncthreads();
 
     // ---- scan: 8 positions per lane per pass, loads kCoreBurst passes ahead ---------------------------------------
-    // Returns the pass's outputs in yv and their plane positions in at (logical index in this direction's order).
-    auto compute = [&](int pass, const Loads &r, float &h_carry, float (&yv)[kItems], int (&at)[kItems], int &img_of_b) {
+    // Where one group of kGran consecutive positions (never split between images) sits in the LDS arrays.
+    struct GroupSlot {
+        int plane_idx;     // index into the plane of the group's lowest logical index
+        bool valid, add;   // inside the stream; add to the plane entry (the other direction was there first) or store
+    };
+
+    // One pass: the outputs in yv (scan order) and the plane slots of its groups.
+    auto compute = [&](int pass, const Loads &r, float &h_carry, float (&yv)[kItems], GroupSlot (&slot)[kGroups]) {
         const int e0 = pass * kPass + lane * kItems;
         const int j0 = (int)r.j0, i0 = (int)r.i0;
         const int k = kGran == kItems ? kItems : min(kItems, L - j0);
-        float raw[kItems], Bv[kItems], Cv[kItems];
+        const int img_base = i0 * L;
+        float raw[kItems], Bv[kItems], Cv[kItems], uv[kItems];
         unpack_raw<in_t>(r.dl, raw);
         bool first[kGroups];
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             const bool in_a = kGran == kItems ? true : gi * kGran < k;
-            first[gi] = (in_a ? j0 + gi * kGran : gi * kGran - k) == 0;
+            const int jg = in_a ? j0 + gi * kGran : gi * kGran - k;          // position of the group in its image
+            const int img_off = in_a ? img_base : img_base + L;              // img * L
+            first[gi] = jg == 0;
             float bg[kGran], cg[kGran];
             unpack_group<in_t, kGran>(r.b[gi], bg);
             unpack_group<in_t, kGran>(r.c[gi], cg);
 #pragma unroll
             for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
-        }
-        // u from LDS.  Forwards the logical index is the stream position e0 + i; backwards it is img*L + L-1-j.
-        const int step = reverse ? -1 : 1;
-        const int at_a = reverse ? i0 * L + L - 1 - j0 : e0;                 // items of image i0:     at_a + step*i
-        const int at_b = reverse ? (i0 + 1) * L + L - 1 + k : e0;            // items of image i0 + 1: at_b + step*i
-        img_of_b = k;
-        float uv[kItems];
+            // The group's kGran logical indices in this direction's order are consecutive and kGran-aligned (L and
+            // every group start are multiples of kGran): forwards they are the stream positions e0 + gi*kGran + t,
+            // backwards img*L + L-1 - (jg + t), i.e. the block starting at img*L + L - jg - kGran read downwards.
+            const bool valid = e0 + gi * kGran < n_el;
+            int base = reverse ? img_off + L - jg - kGran : e0 + gi * kGran;
+            base = valid ? base : 0;
+            // the other direction reaches this block at the mirrored stream position of the same image
+            const int other_pos = reverse ? base : 2 * img_off + L - 1 - base;
+            const int other_pass = (int)((uint32_t)other_pos / (uint32_t)kPass);
+            slot[gi].valid = valid;
+            slot[gi].add = reverse ? other_pass <= pass : other_pass < pass;
+            slot[gi].plane_idx = lds_index<4>(base);
+            const in_t *src = xs + lds_index<kEs>(base);                     // no pad word inside an aligned block
+            float um[kGran];
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) {
-            const bool valid = e0 + i < n_el;
-            int a = ((kGran == kItems || i < k) ? at_a : at_b) + step * i;
-            a = valid ? a : 0;
-            at[i] = a;
-            const in_t v = xs[lds_index<kEs>(a)];
-            uv[i] = valid ? to_f32(v) : 0.0f;
+            for (int c = 0; c < kGran; ++c) um[c] = to_f32(src[c]);
+#pragma unroll
+            for (int t = 0; t < kGran; ++t) {
+                const float v = reverse ? um[kGran - 1 - t] : um[t];
+                uv[gi * kGran + t] = valid ? v : 0.0f;
+            }
         }
         float dl[kItems], bias_items[kItems];
 #pragma unroll
@@ -224,10 +247,11 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         float ac[kItems], hh[kItems];
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
-            if constexpr (!kSoftplus) dl[i] = (e0 + i < n_el) ? dl[i] : 0.0f;
+            // past the end of the stream delta was filled so that dl = 0 (softplus) or is zeroed here; u is 0 there
+            if constexpr (!kSoftplus) dl[i] = slot[i / kGran].valid ? dl[i] : 0.0f;
             float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
             if (i % kGran == 0) a = first[i / kGran] ? 0.0f : a;
-            const float bb = (e0 + i < n_el) ? Bv[i] * (dl[i] * uv[i]) : 0.0f;
+            const float bb = slot[i / kGran].valid ? Bv[i] * (dl[i] * uv[i]) : 0.0f;
             ac[i] = i == 0 ? a : ac[i - 1] * a;
             hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
         }
@@ -243,19 +267,17 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     // pass a / 512 and by the backward direction in pass (2*img*L + L-1 - a) / 512 (its stream position there is
     // the mirror image of a within the image).  The earlier pass stores, the later one adds; in the same pass the
     // forward direction goes first (the barrier between the two halves of a pass orders them).
-    auto update_plane = [&](int pass, const Loads &r, const float (&yv)[kItems], const int (&at)[kItems], int k) {
-        const int e0 = pass * kPass + lane * kItems;
-        const int i0 = (int)r.i0;
+    auto update_plane = [&](const float (&yv)[kItems], const GroupSlot (&slot)[kGroups]) {
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) {
-            if (e0 + i < n_el) {
-                const int img = (kGran == kItems || i < k) ? i0 : i0 + 1;
-                const int other_pos = reverse ? at[i] : 2 * img * L + L - 1 - at[i];     // the other direction's stream position
-                const int other_pass = (int)((uint32_t)other_pos / (uint32_t)kPass);
-                const bool add = reverse ? other_pass <= pass : other_pass < pass;
-                float *slot = plane + lds_index<4>(at[i]);
-                const float old = *slot;
-                *slot = add ? old + yv[i] : yv[i];
+        for (int gi = 0; gi < kGroups; ++gi) {
+            if (slot[gi].valid) {
+                float *dst = plane + slot[gi].plane_idx;
+#pragma unroll
+                for (int c = 0; c < kGran; ++c) {
+                    const float y = reverse ? yv[gi * kGran + kGran - 1 - c] : yv[gi * kGran + c];
+                    const float old = dst[c];
+                    dst[c] = slot[gi].add ? old + y : y;
+                }
             }
         }
     };
@@ -267,11 +289,11 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             const int pass = pass0 + q;
             if (pass < n_pass) {                     // uniform over the workgroup: every wavefront meets every barrier
                 float yv[kItems];
-                int at[kItems], k;
-                compute(pass, regs[q], h_carry, yv, at, k);
-                if (!reverse) update_plane(pass, regs[q], yv, at, k);
+                GroupSlot slot[kGroups];
+                compute(pass, regs[q], h_carry, yv, slot);
+                if (!reverse) update_plane(yv, slot);
                 __syncthreads();
-                if (reverse) update_plane(pass, regs[q], yv, at, k);
+                if (reverse) update_plane(yv, slot);
                 __syncthreads();
                 if (pass + kCoreBurst < n_pass) issue(pass + kCoreBurst, regs[q]);
             }
