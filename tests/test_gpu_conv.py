@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 SHAPES = [(2, 96, 56, 56), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (1, 8, 3, 3), (2, 40, 9, 13), (1, 96, 1, 1),
-          (2, 12, 5, 6), (1, 7, 4, 4), (1, 32, 1, 70)]
+          (2, 12, 5, 6), (1, 7, 4, 4), (1, 32, 1, 70), (1, 16, 2, 200), (1, 64, 20, 128)]
 
 
 def _tol(dtype):

@@ -20,6 +20,12 @@ constexpr int kDwCh = 32;            // channels per workgroup tile
 constexpr int kDwPitch = kDwPos + 8; // LDS row pitch in elements: keeps 16-byte alignment, spreads banks
 
 __device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+// SiLU for results that are rounded to a 16-bit type afterwards: the two hardware transcendentals (each good to one
+// fp32 ulp) instead of the library expf and an IEEE division -- a quarter of the instructions, far below 16-bit
+// rounding.  exp2 overflows to +inf for very negative v, where rcp gives 0 and the product -0: SiLU's limit.
+__device__ __forceinline__ float silu_fast(float v) {
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
+}
 
 template <typename T> __device__ __forceinline__ void unpack8(const uint4 raw, float (&v)[8]) {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_kernel(const T *__rest
         for (int ci = 0; ci < 8; ++ci) {
             float v = acc[ci] + (bias ? bv[ci] : 0.0f);
             T o = from_f32<T>(v);
-            if (kSilu) o = from_f32<T>(silu_f32(to_f32(o)));
+            if (kSilu) o = from_f32<T>(silu_fast(to_f32(o)));
             tile[(cv * 8 + ci) * kDwPitch + p] = o.bits;
         }
     }
@@ -105,6 +111,127 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_kernel(const T *__rest
             *reinterpret_cast<uint4 *>(yo) = *reinterpret_cast<const uint4 *>(src);
         } else {
             for (int i = 0; i < 8 && rr + i < L; ++i) yo[i] = T{src[i]};
+        }
+    }
+}
+
+// Row-tile variant of the same operation for images up to kDwMaxW wide: a workgroup owns TH full rows x 32 channels.
+// The input rows (plus one halo row above and below and one zero column either side) are copied ONCE into LDS with
+// 16-byte loads -- the nine taps then come out of LDS as contiguous 16-byte reads instead of nine trips through the
+// vector memory pipeline, which is what bounds the kernel above.  Results are parked channel-major in a second LDS
+// tile and written as 16 bytes per lane along the row-major positions, which are contiguous in (B,D,H,W).
+constexpr int kDwMaxW = 128;
+
+template <typename T, bool kSilu>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restrict__ x, const T *__restrict__ weight,
+                                                                const T *__restrict__ bias, T *__restrict__ y, int D,
+                                                                int H, int W, int TH, int row_tiles, int ch_tiles,
+                                                                int out_pitch, FastDiv divW, FastDiv divWp) {
+    extern __shared__ __align__(16) uint16_t dw_smem[];
+    const int Wp = W + 2;
+    uint16_t *in_tile = dw_smem;                                 // [TH + 2][W + 2][32]
+    uint16_t *out_tile = dw_smem + (TH + 2) * Wp * kDwCh;        // [32][out_pitch]
+    uint32_t wg = blockIdx.x;
+    const uint32_t ct = wg % ch_tiles; wg /= ch_tiles;
+    const uint32_t rt = wg % row_tiles;
+    const uint32_t b = wg / row_tiles;
+    const int h0 = (int)rt * TH;
+    const int rows = min(TH, H - h0);
+    const int c_base = (int)ct * kDwCh;
+    const int cv = threadIdx.x % 4;
+    const int c0 = c_base + cv * 8;                              // this lane's 8 channels, in every phase
+
+    // ---- input rows h0-1 .. h0+rows into LDS; outside the image (and channels >= D) zeros.  The image sits behind a
+    // buffer descriptor and pieces outside it are pointed past its end, where the hardware returns 0: the loads
+    // are unconditional, so a thread's six are in flight together instead of one latency after the other.
+    const T *xb = x + (size_t)b * H * W * D;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xb), 0, H * W * D * 2, 0x00020000);
+    const int n_in = (rows + 2) * Wp;
+    constexpr int kLoadsInFlight = 6;
+    for (int e0 = threadIdx.x / 4; e0 < n_in; e0 += kLoadsInFlight * (kBlock / 4)) {
+        uint4 v[kLoadsInFlight];
+#pragma unroll
+        for (int u = 0; u < kLoadsInFlight; ++u) {
+            const int e = e0 + u * (kBlock / 4);
+            uint32_t rr, cc;
+            divmod((uint32_t)e, divWp, rr, cc);
+            const int h = h0 - 1 + (int)rr, w = (int)cc - 1;
+            const bool inside = e < n_in && h >= 0 && h < H && w >= 0 && w < W && c0 < D;
+            const uint32_t off = inside ? (uint32_t)((h * W + w) * D + c0) * 2u : 0x7ffffff0u;
+            const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+            v[u] = make_uint4(t[0], t[1], t[2], t[3]);
+        }
+#pragma unroll
+        for (int u = 0; u < kLoadsInFlight; ++u) {
+            const int e = e0 + u * (kBlock / 4);
+            if (e < n_in) *reinterpret_cast<uint4 *>(in_tile + (size_t)e * kDwCh + cv * 8) = v[u];
+        }
+    }
+    // the 72 weights of the 8 channels: 9 consecutive 16-byte vectors
+    float wt[8][9];
+    float bv[8];
+    {
+        const int cw = min(c0, D - 8);                           // keep the loads in range; lanes with c0 >= D store nothing
+        const uint4 *wp = reinterpret_cast<const uint4 *>(weight + (size_t)cw * 9);
+        float flat[72];
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            float t8[8];
+            unpack8<T>(wp[k], t8);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) flat[k * 8 + i] = t8[i];
+        }
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci)
+#pragma unroll
+            for (int t = 0; t < 9; ++t) wt[ci][t] = flat[ci * 9 + t];
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci) bv[ci] = 0.0f;
+        if (bias) unpack8<T>(*reinterpret_cast<const uint4 *>(bias + cw), bv);
+    }
+    __syncthreads();
+
+    // ---- nine taps per output from LDS
+    const int n_out = rows * W;
+    for (int pidx = threadIdx.x / 4; pidx < n_out; pidx += kBlock / 4) {
+        uint32_t ph, pw;
+        divmod((uint32_t)pidx, divW, ph, pw);
+        float acc[8];
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci) acc[ci] = 0.0f;
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                float xv[8];
+                unpack8<T>(*reinterpret_cast<const uint4 *>(in_tile + ((size_t)(ph + kh) * Wp + pw + kw) * kDwCh + cv * 8), xv);
+#pragma unroll
+                for (int ci = 0; ci < 8; ++ci) acc[ci] = fmaf(wt[ci][kh * 3 + kw], xv[ci], acc[ci]);
+            }
+#pragma unroll
+        for (int ci = 0; ci < 8; ++ci) {
+            T o = from_f32<T>(acc[ci] + bv[ci]);
+            if (kSilu) o = from_f32<T>(silu_fast(to_f32(o)));
+            out_tile[(cv * 8 + ci) * out_pitch + pidx] = o.bits;
+        }
+    }
+    __syncthreads();
+
+    // ---- write back: the tile's positions are contiguous per channel in (B, D, H, W)
+    const int L = H * W;
+    const int pieces = (n_out + 7) / 8;
+    const bool vec = ((h0 * W) % 8 == 0) && (L % 8 == 0);
+    for (int e = threadIdx.x; e < kDwCh * pieces; e += kBlock) {
+        const int c = e / pieces, piece = e - c * pieces;
+        const int cg = c_base + c;
+        if (cg < D) {
+            T *yo = y + ((size_t)b * D + cg) * L + (size_t)h0 * W + piece * 8;
+            const uint16_t *src = out_tile + c * out_pitch + piece * 8;
+            if (vec && piece * 8 + 8 <= n_out) {
+                *reinterpret_cast<uint4 *>(yo) = *reinterpret_cast<const uint4 *>(src);
+            } else {
+                for (int i = 0; i < 8 && piece * 8 + i < n_out; ++i) yo[i] = T{src[i]};
+            }
         }
     }
 }
@@ -148,6 +275,27 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
     const int64_t L = (int64_t)H * W;
     auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     if constexpr (sizeof(T) == 2) {
+        if (in_channel_last && D % 8 == 0 && W <= kDwMaxW && al16(x) && al16(w) && al16(y) && (!bias || al16(bias))) {
+            // TH rows per workgroup: about 224 positions, LDS within 64 KiB
+            int TH = 224 / W;
+            TH = TH < 1 ? 1 : (TH > H ? H : TH);
+            const int out_pitch = ((TH * W + 7) / 8) * 8 + 8;
+            const size_t smem = ((size_t)(TH + 2) * (W + 2) * kDwCh + (size_t)kDwCh * out_pitch) * sizeof(uint16_t);
+            const int row_tiles = (H + TH - 1) / TH, ch_tiles = (D + kDwCh - 1) / kDwCh;
+            const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
+            if (smem <= 64 * 1024 && n_wg <= 0x7fffffff && (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
+                if (apply_silu) {
+                    hipLaunchKernelGGL((dwconv3x3_rows_kernel<T, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream,
+                                       (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles,
+                                       out_pitch, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)));
+                } else {
+                    hipLaunchKernelGGL((dwconv3x3_rows_kernel<T, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream,
+                                       (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles,
+                                       out_pitch, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)));
+                }
+                return launch_status();
+            }
+        }
         if (in_channel_last && D % 8 == 0 && al16(x) && al16(w) && al16(y) && (!bias || al16(bias))) {
             const int pos_tiles = (int)((L + kDwPos - 1) / kDwPos), ch_tiles = (D + kDwCh - 1) / kDwCh;
             const int64_t n_wg = (int64_t)B * pos_tiles * ch_tiles;

@@ -181,7 +181,10 @@ class SS2D(nn.Module):
         """out_norm on the merged (B, D, L) map, in the block's layout (vmamba.py:641-646)."""
         return self.layers.out_norm(self.out_norm, y.view(B, D, H, W), self.channel_first, dtype)
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """``residual`` (same layout as x) is added to the result; channel-last blocks without an out_proj bias fold
+        the addition into the out_proj GEMM (one pass over the activation fewer than the block's separate add,
+        vmamba.py:1228, and one rounding instead of two)."""
         x = self.in_proj(x)
         z = None
         if not self.disable_z:
@@ -191,4 +194,8 @@ class SS2D(nn.Module):
         y = self.forward_core(x)
         if z is not None:
             y = y * z
-        return self.out_proj(y)
+        if residual is None:
+            return self.out_proj(y)
+        if self.channel_first or self.out_proj.bias is not None:
+            return residual + self.out_proj(y)
+        return torch.addmm(residual.reshape(-1, self.d_model), y.reshape(-1, self.d_inner), self.out_proj.weight.t()).view(residual.shape)

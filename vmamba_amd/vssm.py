@@ -55,7 +55,7 @@ class VSSBlock(nn.Module):
         self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
     def forward(self, x):
-        x = x + self.op(self.norm(x))
+        x = self.op(self.norm(x), residual=x)
         return x + self.mlp(self.norm2(x))
 
 
