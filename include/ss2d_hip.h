@@ -191,6 +191,27 @@ typedef struct ss2d_core_params {
 int ss2d_core_fwd(const ss2d_core_params *params, void *stream);
 
 /*
+ * CrossScan / CrossMerge for every layout and mode of the reference operators (cross_scan_fn / cross_merge_fn,
+ * classification/models/csm_triton.py:501-517; semantics of the flex kernel :278-400 and of the torch functions
+ * :22-179).  Flags are named from the scan's side, as in the reference, for both operations:
+ *   x_channel_last   0: x is (B,[4,]C,H,W)      1: x is (B,H,W,[4,]C)        ("in_channel_first" negated)
+ *   y_channel_last   0: y is (B,4,C,H*W)        1: y is (B,H*W,4,C)          ("out_channel_first" negated)
+ *   one_by_one       x has one slice per direction (the bracketed 4) instead of one shared map
+ *   scans            0: row-major, column-major, both reversed;  1: row-major four times;  2: row-major twice,
+ *                    reversed twice
+ * scan:   y_k[route_k(h,w)] = x_(k)[h,w]                       (a permutation / replication; any 1/2/4/8-byte type)
+ * merge:  x[h,w] = sum_k y_k[route_k(h,w)]  (one_by_one: x_k[h,w] = y_k[route_k(h,w)], no sum), dtype F32/BF16/F16.
+ *         Rounding: scans 0 and 2 add pairwise, (y0 + y2) + (y1 + y3), each add rounded to dtype (order = PAIRWISE,
+ *         the torch functions) or left to right (order = LEFT_TO_RIGHT, the Triton kernel); scans 1 accumulates the
+ *         four terms in fp32 and rounds once (a torch reduction, csm_triton.py:64).
+ * The default combination (0, 0, 0, 0) is also served by the tiled kernels behind ss2d_cross_scan / ss2d_cross_merge.
+ */
+int ss2d_cross_scan_flex(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                         int y_channel_last, int one_by_one, int scans, void *stream);
+int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H, int W, int dtype, int x_channel_last,
+                          int y_channel_last, int one_by_one, int scans, int order, void *stream);
+
+/*
  * dt_proj of the SS2D core: the per-direction rank-R -> D projection between x_proj and the scan.
  * Replaces the grouped conv1d / einsum of SS2Dv2.forward_corev2 (classification/models/vmamba.py:608-609, 614-615):
  *   delta[k, d, n] = sum_r weight[k, d, r] * x[k*x_dir_stride + r*x_rank_stride + n]

@@ -10,6 +10,8 @@ Follows, without importing them:
   cross_scan   classification/models/csm_triton.py:22-29 and :532-541
   cross_scan_1b1  classification/models/csm_triton.py:88-99 (one-by-one, scans = 0)
   cross_merge  classification/models/csm_triton.py:56-62 and :543-551
+  cross_scan_flex / cross_merge_flex  every layout / mode of csm_triton.py:22-179, stated as index gathers
+                  over the routes of the flex kernel (:308-328)
   selective_scan  kernels/selective_scan/test_selective_scan.py:168-234
                   (selective_scan_ref; same arithmetic as csms6s.py:25-68 but
                   the bias add and softplus happen after the widening to fp32,
@@ -32,6 +34,59 @@ def cross_scan_1b1(x):
     col = lambda v: v.transpose(2, 3).reshape(B, C, H * W)
     return torch.stack([x[:, 0].reshape(B, C, H * W), col(x[:, 1]),
                         x[:, 2].reshape(B, C, H * W).flip(-1), col(x[:, 3]).flip(-1)], dim=1)
+
+
+def scan_routes(H, W, scans):
+    """(4, L) int64: routes[k, r] = scan position at which direction k visits row-major spatial index r."""
+    L = H * W
+    r = torch.arange(L)
+    col = (r % W) * H + r // W
+    if scans == 0:
+        return torch.stack([r, col, L - 1 - r, L - 1 - col])
+    if scans == 1:
+        return torch.stack([r, r, r, r])
+    if scans == 2:
+        return torch.stack([r, r, L - 1 - r, L - 1 - r])
+    raise ValueError(scans)
+
+
+def cross_scan_flex(x, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0):
+    """x (B,[4,]C,H,W) | (B,H,W,[4,]C) -> y (B,4,C,L) | (B,L,4,C):  y_k[route_k(r)] = x_(k)[r]."""
+    if in_channel_first:
+        B, C, H, W = x.shape[0], x.shape[-3], x.shape[-2], x.shape[-1]
+        xs = x.reshape(B, -1, C, H * W)
+    else:
+        B, H, W, C = x.shape[0], x.shape[1], x.shape[2], x.shape[-1]
+        xs = x.reshape(B, H * W, -1, C).permute(0, 2, 3, 1)
+    xs = xs.expand(B, 4, C, H * W)
+    routes = scan_routes(H, W, scans)
+    y = x.new_empty((B, 4, C, H * W))
+    for k in range(4):
+        y[:, k, :, routes[k]] = xs[:, k]
+    return y if out_channel_first else y.permute(0, 3, 1, 2).contiguous()
+
+
+def cross_merge_flex(y, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0, left_to_right=False):
+    """y (B,4,C,H,W) | (B,H,W,4,C) -> x (B,[4,]C,L) | (B,L,[4,]C):  x[r] = sum_k y_k[route_k(r)] (one_by_one: no sum).
+    scans 0, 2: (y0 + y2) + (y1 + y3) rounded per add (or left to right); scans 1: a 4-term reduction."""
+    if out_channel_first:
+        B, _, C, H, W = y.shape
+        ys = y.reshape(B, 4, C, H * W)
+    else:
+        B, H, W, _, C = y.shape
+        ys = y.reshape(B, H * W, 4, C).permute(0, 2, 3, 1)
+    routes = scan_routes(H, W, scans)
+    g = [ys[:, k][..., routes[k]] for k in range(4)]
+    if one_by_one:
+        x = torch.stack(g, dim=1)                                   # (B, 4, C, L)
+        return x if in_channel_first else x.permute(0, 3, 1, 2).contiguous()
+    if scans == 1:
+        x = torch.stack(g, dim=1).sum(1)                            # the reference's y.sum(1)
+    elif left_to_right:
+        x = ((g[0] + g[1]) + g[2]) + g[3]
+    else:
+        x = (g[0] + g[2]) + (g[1] + g[3])
+    return x if in_channel_first else x.permute(0, 2, 1).contiguous()
 
 
 def cross_merge(ys):

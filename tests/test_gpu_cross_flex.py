@@ -1,0 +1,94 @@
+"""GPU parity of CrossScan / CrossMerge in every layout and mode (channel-first / channel-last on either side,
+one-by-one, scans 0 / 1 / 2) through the C ABI against the CPU oracle.  Bit-exact: the scan is a permutation, and
+the merge's additions are rounded in the oracle's order."""
+import itertools
+
+import pytest
+import torch
+
+from oracle import torch_ref
+import vmamba_amd as va
+from vmamba_amd import _lib
+from vmamba_amd.csm import cross_merge_flex_hip
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+MODES = list(itertools.product([True, False], [True, False], [False, True], [0, 1, 2]))
+SHAPES = [(2, 3, 5, 7), (1, 8, 14, 14), (2, 96, 7, 7), (1, 2, 1, 9), (1, 1, 33, 2)]
+
+
+def _x_shape(B, C, H, W, icf, obo):
+    if icf:
+        return (B, 4, C, H, W) if obo else (B, C, H, W)
+    return (B, H, W, 4, C) if obo else (B, H, W, C)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8], ids=str)
+@pytest.mark.parametrize("icf,ocf,obo,scans", MODES)
+def test_cross_scan_every_mode_bit_exact(icf, ocf, obo, scans, dtype):
+    print("CASE scan-flex", icf, ocf, obo, scans, dtype, flush=True)
+    for (B, C, H, W) in SHAPES:
+        g = torch.Generator().manual_seed(B + C + H + W)
+        x = (torch.randn(_x_shape(B, C, H, W, icf, obo), generator=g) * 40).to(dtype)
+        want = torch_ref.cross_scan_flex(x, icf, ocf, obo, scans)
+        got = va.cross_scan_fn(x.to(DEV), icf, ocf, obo, scans)
+        torch.cuda.synchronize()
+        assert got.shape == want.shape and torch.equal(got.cpu(), want), (B, C, H, W)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("icf,ocf,obo,scans", MODES)
+def test_cross_merge_every_mode_bit_exact(icf, ocf, obo, scans, dtype):
+    print("CASE merge-flex", icf, ocf, obo, scans, dtype, flush=True)
+    for (B, C, H, W) in SHAPES:
+        g = torch.Generator().manual_seed(B * 7 + C + H + W)
+        y = torch.randn((B, 4, C, H, W) if ocf else (B, H, W, 4, C), generator=g).to(dtype)
+        want = torch_ref.cross_merge_flex(y, icf, ocf, obo, scans)
+        got = va.cross_merge_fn(y.to(DEV), icf, ocf, obo, scans)
+        torch.cuda.synchronize()
+        assert got.shape == want.shape and got.dtype == dtype
+        if scans == 1 and not obo and dtype == torch.float32:
+            # a four-term fp32 reduction: the library's order of additions is not specified
+            assert torch.allclose(got.cpu(), want, rtol=3e-7, atol=1e-7), (B, C, H, W)
+        else:
+            assert torch.equal(got.cpu(), want), (B, C, H, W)
+
+
+def test_cross_merge_flex_left_to_right_order():
+    y = torch.randn(2, 7, 5, 4, 6, generator=torch.Generator().manual_seed(1)).bfloat16()
+    want = torch_ref.cross_merge_flex(y, False, False, False, 0, left_to_right=True)
+    got = cross_merge_flex_hip(y.to(DEV), False, False, False, 0, order=_lib.MERGE_LEFT_TO_RIGHT)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("icf,ocf,obo,scans", MODES)
+def test_flex_modes_round_trip_and_autograd(icf, ocf, obo, scans):
+    """merge(scan(x)) = 4x (one-by-one: x) exactly on small integers; the backward of each operator is the other."""
+    B, C, H, W = 2, 3, 4, 5
+    x = torch.randint(-8, 8, _x_shape(B, C, H, W, icf, obo), generator=torch.Generator().manual_seed(2)).float().to(DEV)
+    x.requires_grad_(True)
+    y = va.cross_scan_fn(x, icf, ocf, obo, scans)
+    y5 = y.view(B, 4, C, H, W) if ocf else y.view(B, H, W, 4, C)
+    back = va.cross_merge_fn(y5, icf, ocf, obo, scans)
+    assert torch.equal(back.reshape(x.shape), x.detach() * (1 if obo else 4))
+    gy = torch.randint(-8, 8, y.shape, generator=torch.Generator().manual_seed(3)).float().to(DEV)
+    (gx,) = torch.autograd.grad(y, x, gy)
+    want = va.cross_merge_fn((gy.view(B, 4, C, H, W) if ocf else gy.view(B, H, W, 4, C)), icf, ocf, obo, scans)
+    assert torch.equal(gx, want.reshape(x.shape))
+    # <scan(x), gy> = <x, merge(gy)>
+    assert (y.detach() * gy).sum().item() == (x.detach() * gx).sum().item()
+
+
+def test_flex_rejections():
+    with pytest.raises(NotImplementedError):
+        va.cross_scan_fn(torch.zeros(1, 2, 3, 3, device=DEV), scans=3)
+    with pytest.raises(ValueError):
+        va.cross_scan_fn(torch.zeros(1, 2, 3, 3, device=DEV), one_by_one=True, in_channel_first=False)
+    with pytest.raises(ValueError):
+        va.cross_merge_fn(torch.zeros(1, 3, 2, 3, 3, device=DEV), in_channel_first=False)
+    assert va.cross_scan_fn(torch.zeros(0, 3, 3, 2, device=DEV), in_channel_first=False, out_channel_first=False).shape == (0, 9, 4, 2)
+    L = _lib.lib()
+    assert L.ss2d_cross_scan_flex(None, None, 1, 1, 1, 1, 2, 2, 0, 0, 0, None) == _lib.SS2D_EINVAL
+    assert L.ss2d_cross_scan_flex(None, None, 1, 1, 1, 1, 2, 0, 0, 0, 3, None) == _lib.SS2D_EINVAL
+    assert L.ss2d_cross_merge_flex(None, None, 1, 1, 1, 1, 7, 0, 0, 0, 0, 0, None) == _lib.SS2D_EINVAL

@@ -78,6 +78,98 @@ def test_cross_scan_1b1_pins():
         assert torch.equal(yz[:, k], orc.cross_scan(z[:, k])[:, k])
 
 
+def _flat_offsets(B, C, H, W, x_cl, y_cl, one_by_one):
+    """Flat element offsets of x[b,(k),c,r] and y[b,k,c,j], as the flex kernel computes its pointers
+    (classification/models/csm_triton.py:330-384): channel-first = (B,[4,]C,L) / (B,4,C,L), channel-last =
+    (B,L,[4,]C) / (B,L,4,C)."""
+    L, K = H * W, (4 if one_by_one else 1)
+
+    def xo(b, k, c, r):
+        kk = k if one_by_one else 0
+        return ((b * L + r) * K + kk) * C + c if x_cl else ((b * K + kk) * C + c) * L + r
+
+    def yo(b, k, c, j):
+        return ((b * L + j) * 4 + k) * C + c if y_cl else ((b * 4 + k) * C + c) * L + j
+    return xo, yo
+
+
+def _route(k, scans, h, w, H, W):
+    """csm_triton.py:308-328: none; trans; flip; trans + flip | none x4 | none, none, flip, flip."""
+    L = H * W
+    if scans == 0:
+        return [h * W + w, w * H + h, L - 1 - (h * W + w), L - 1 - (w * H + h)][k]
+    if scans == 1:
+        return h * W + w
+    return h * W + w if k < 2 else L - 1 - (h * W + w)
+
+
+@pytest.mark.parametrize("scans", [0, 1, 2])
+@pytest.mark.parametrize("one_by_one", [False, True])
+@pytest.mark.parametrize("x_cl,y_cl", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_cross_flex_against_flat_offset_loops(x_cl, y_cl, one_by_one, scans):
+    """The tensor formulation against element-by-element loops over flat offsets, for every layout and mode; the
+    default mode is also tied to the functions the known-answer cases pin."""
+    B, C, H, W = 2, 3, 3, 4
+    L, K = H * W, (4 if one_by_one else 1)
+    xo, yo = _flat_offsets(B, C, H, W, x_cl, y_cl, one_by_one)
+    x_flat = torch.arange(B * K * C * L, dtype=torch.float32) + 1
+    shape = ((B, H, W) + ((4,) if one_by_one else ()) + (C,)) if x_cl else ((B,) + ((4,) if one_by_one else ()) + (C, H, W))
+    x = x_flat.view(shape)
+    want = torch.zeros(B * 4 * C * L)
+    for b in range(B):
+        for k in range(4):
+            for c in range(C):
+                for h in range(H):
+                    for w in range(W):
+                        want[yo(b, k, c, _route(k, scans, h, w, H, W))] = x_flat[xo(b, k, c, h * W + w)]
+    got = torch_ref.cross_scan_flex(x, not x_cl, not y_cl, one_by_one, scans)
+    assert got.shape == ((B, L, 4, C) if y_cl else (B, 4, C, L))
+    assert torch.equal(got.reshape(-1), want)
+    # merge: x[b,(k),c,r] = sum_k y[b,k,c,route_k(r)]
+    y_flat = torch.arange(B * 4 * C * L, dtype=torch.float32) * 3 + 2
+    y = y_flat.view((B, H, W, 4, C) if y_cl else (B, 4, C, H, W))
+    wantm = torch.zeros(B * K * C * L)
+    for b in range(B):
+        for c in range(C):
+            for h in range(H):
+                for w in range(W):
+                    terms = [y_flat[yo(b, k, c, _route(k, scans, h, w, H, W))] for k in range(4)]
+                    if one_by_one:
+                        for k in range(4):
+                            wantm[xo(b, k, c, h * W + w)] = terms[k]
+                    else:
+                        wantm[xo(b, 0, c, h * W + w)] = sum(terms)
+    gotm = torch_ref.cross_merge_flex(y, not x_cl, not y_cl, one_by_one, scans)
+    assert gotm.shape == (((B, L) + ((4,) if one_by_one else ()) + (C,)) if x_cl else ((B,) + ((4,) if one_by_one else ()) + (C, L)))
+    assert torch.equal(gotm.reshape(-1), wantm)            # small integers: every order of addition is exact
+    if not (x_cl or y_cl or scans):
+        if one_by_one:
+            assert torch.equal(got, torch_ref.cross_scan_1b1(x))
+        else:
+            assert torch.equal(got, orc.cross_scan(x)) and torch.equal(gotm, orc.cross_merge(y))
+
+
+@pytest.mark.parametrize("scans", [0, 1, 2])
+def test_cross_merge_flex_rounding(scans):
+    """bf16: scans 0 / 2 round every pairwise add; scans 1 is the library reduction over the four copies."""
+    g = torch.Generator().manual_seed(9)
+    y = (torch.randn(2, 4, 3, 5, 6, generator=g) * 3).bfloat16()
+    B, K, C, H, W = y.shape
+    routes = torch_ref.scan_routes(H, W, scans)
+    t = [y.view(B, 4, C, -1)[:, k][..., routes[k]] for k in range(4)]
+    got = torch_ref.cross_merge_flex(y, scans=scans)
+    if scans == 1:
+        assert torch.equal(got, y.view(B, 4, C, -1).sum(1))
+    else:
+        want = ((t[0].float() + t[2].float()).bfloat16().float() + (t[1].float() + t[3].float()).bfloat16().float()).bfloat16()
+        assert torch.equal(got, want)
+        ltr = torch_ref.cross_merge_flex(y, scans=scans, left_to_right=True)
+        w2 = t[0]
+        for k in (1, 2, 3):
+            w2 = (w2.float() + t[k].float()).bfloat16()
+        assert torch.equal(ltr, w2)
+
+
 def test_cross_scan_empty():
     assert orc.cross_scan(torch.zeros(0, 3, 4, 4)).shape == (0, 4, 3, 16)
     assert orc.cross_scan(torch.zeros(2, 0, 4, 4)).shape == (2, 4, 0, 16)

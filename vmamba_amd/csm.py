@@ -1,10 +1,11 @@
 """CrossScan / CrossMerge operator API, mirroring classification/models/csm_triton.py:501-517.
 
-``cross_scan_fn`` and ``cross_merge_fn`` keep the reference's signatures.  The combination the
-SS2D core uses -- channel-first in and out, not one-by-one, ``scans=0`` (vmamba.py:603, 632) --
-runs on the HIP kernels in libss2d_hip.so through the C ABI, and so does the one-by-one CrossScan
-(forward only).  Other layouts / scan modes raise NotImplementedError; CPU tensors raise as well:
-this package has no CPU path.
+``cross_scan_fn`` and ``cross_merge_fn`` keep the reference's signatures and serve every layout and
+mode of the reference (channel-first / channel-last on either side, one-by-one, ``scans`` 0/1/2)
+on the HIP kernels in libss2d_hip.so through the C ABI: the combination the SS2D core uses --
+channel-first in and out, not one-by-one, ``scans=0`` (vmamba.py:603, 632) -- and the
+channel-first one-by-one scan on tiled kernels, everything else on the generic "flex" kernels.
+``force_torch=True`` and CPU tensors raise: this package has no PyTorch or CPU path.
 
 Both operators are each other's adjoint (csm_triton.py:208-225, 249-273), so autograd is
 supported with the same two kernels.
@@ -25,13 +26,58 @@ def _require_gpu(t, what):
         raise NotImplementedError(f"{what}: vmamba_amd runs on the GPU only (got a {t.device.type} tensor)")
 
 
-def _require_default_mode(what, in_channel_first, out_channel_first, one_by_one, scans, force_torch, allow_1b1=False):
+def _require_hip(what, scans, force_torch):
     if force_torch:
         raise NotImplementedError(f"{what}: force_torch=True asks for the PyTorch implementation, which this package does not ship")
-    if not (in_channel_first and out_channel_first and (allow_1b1 or not one_by_one) and scans == 0):
-        raise NotImplementedError(
-            f"{what}: only in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0 has a HIP kernel "
-            f"(got {in_channel_first}, {out_channel_first}, {one_by_one}, {scans})")
+    if scans not in (0, 1, 2):
+        raise NotImplementedError(f"{what}: scans must be 0 (cross), 1 (unidirectional) or 2 (bidirectional), got {scans}")
+
+
+def _flex_dims(t, channel_first, one_by_one, what):
+    """(B, C, H, W) of an x-side / merge-input tensor: (B,[4,]C,H,W) or (B,H,W,[4,]C)."""
+    want = 5 if one_by_one else 4
+    if t.dim() != want or (one_by_one and t.shape[1 if channel_first else 3] != 4):
+        raise ValueError(f"{what}: expected a {'(B,4,C,H,W)' if channel_first else '(B,H,W,4,C)'} tensor"
+                         f"{'' if one_by_one else ' without the direction axis'}, got {tuple(t.shape)}")
+    if channel_first:
+        return t.shape[0], t.shape[-3], t.shape[-2], t.shape[-1]
+    return t.shape[0], t.shape[-1], t.shape[1], t.shape[2]
+
+
+def cross_scan_flex_hip(x, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0):
+    """Any layout / mode of CrossScan (ss2d_cross_scan_flex); bit-exact for any 1/2/4/8-byte dtype."""
+    _require_gpu(x, "cross_scan")
+    B, C, H, W = _flex_dims(x, in_channel_first, one_by_one, "cross_scan")
+    x = x.contiguous()
+    y = x.new_empty((B, 4, C, H * W) if out_channel_first else (B, H * W, 4, C))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_cross_scan_flex(x.data_ptr(), y.data_ptr(), B, C, H, W, x.element_size(),
+                                             0 if in_channel_first else 1, 0 if out_channel_first else 1,
+                                             1 if one_by_one else 0, scans, _stream(x))
+    _lib.check(rc, "ss2d_cross_scan_flex")
+    return y
+
+
+def cross_merge_flex_hip(y, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0,
+                         order=_lib.MERGE_PAIRWISE):
+    """Any layout / mode of CrossMerge (ss2d_cross_merge_flex): y (B,4,C,H,W) | (B,H,W,4,C) ->
+    (B,[4,]C,L) | (B,L,[4,]C)."""
+    _require_gpu(y, "cross_merge")
+    B, C, H, W = _flex_dims(y, out_channel_first, True, "cross_merge")
+    if y.dtype not in _DTYPE_CODE:
+        raise TypeError(f"cross_merge: unsupported dtype {y.dtype}")
+    y = y.contiguous()
+    L = H * W
+    if one_by_one:
+        x = y.new_empty((B, 4, C, L) if in_channel_first else (B, L, 4, C))
+    else:
+        x = y.new_empty((B, C, L) if in_channel_first else (B, L, C))
+    with torch.cuda.device(y.device):
+        rc = _lib.lib().ss2d_cross_merge_flex(y.data_ptr(), x.data_ptr(), B, C, H, W, _DTYPE_CODE[y.dtype],
+                                              0 if in_channel_first else 1, 0 if out_channel_first else 1,
+                                              1 if one_by_one else 0, scans, order, _stream(y))
+    _lib.check(rc, "ss2d_cross_merge_flex")
+    return x
 
 
 def cross_scan_hip(x):
@@ -111,23 +157,62 @@ class CrossMergeHip(torch.autograd.Function):
         return cross_scan_hip(grad_out.reshape(B, C, H, W)).view(B, 4, C, H, W)
 
 
-class CrossScan1b1Hip(torch.autograd.Function):
+class CrossScanFlexHip(torch.autograd.Function):
+    """Any mode; the two operators are each other's adjoint for every mode (csm_triton.py:208-225, 249-273)."""
     @staticmethod
-    def forward(ctx, x):
-        return cross_scan_1b1_hip(x)
+    def forward(ctx, x, in_channel_first, out_channel_first, one_by_one, scans):
+        ctx.mode = (in_channel_first, out_channel_first, one_by_one, scans)
+        ctx.dims = _flex_dims(x, in_channel_first, one_by_one, "cross_scan")
+        if in_channel_first and out_channel_first and one_by_one and scans == 0:
+            return cross_scan_1b1_hip(x)
+        return cross_scan_flex_hip(x, in_channel_first, out_channel_first, one_by_one, scans)
 
     @staticmethod
     def backward(ctx, grad_y):
-        raise NotImplementedError("one-by-one cross_scan: forward only (its adjoint, the one-by-one merge, has no HIP kernel)")
+        icf, ocf, obo, scans = ctx.mode
+        B, C, H, W = ctx.dims
+        g = grad_y.reshape(B, 4, C, H, W) if ocf else grad_y.reshape(B, H, W, 4, C)
+        gx = cross_merge_flex_hip(g, icf, ocf, obo, scans)
+        if obo:
+            gx = gx.view(B, 4, C, H, W) if icf else gx.view(B, H, W, 4, C)
+        else:
+            gx = gx.view(B, C, H, W) if icf else gx.view(B, H, W, C)
+        return gx, None, None, None, None
+
+
+class CrossMergeFlexHip(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, y, in_channel_first, out_channel_first, one_by_one, scans):
+        ctx.mode = (in_channel_first, out_channel_first, one_by_one, scans)
+        ctx.dims = _flex_dims(y, out_channel_first, True, "cross_merge")
+        return cross_merge_flex_hip(y, in_channel_first, out_channel_first, one_by_one, scans)
+
+    @staticmethod
+    def backward(ctx, grad_x):
+        icf, ocf, obo, scans = ctx.mode
+        B, C, H, W = ctx.dims
+        if obo:
+            g = grad_x.reshape(B, 4, C, H, W) if icf else grad_x.reshape(B, H, W, 4, C)
+        else:
+            g = grad_x.reshape(B, C, H, W) if icf else grad_x.reshape(B, H, W, C)
+        gy = cross_scan_flex_hip(g, icf, ocf, obo, scans)
+        return (gy.view(B, 4, C, H, W) if ocf else gy.view(B, H, W, 4, C)), None, None, None, None
 
 
 def cross_scan_fn(x, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0, force_torch=False):
-    # x: (B, C, H, W) -> y: (B, 4, C, L);  one_by_one: x (B, 4, C, H, W)
-    _require_default_mode("cross_scan_fn", in_channel_first, out_channel_first, one_by_one, scans, force_torch, allow_1b1=True)
-    return CrossScan1b1Hip.apply(x) if one_by_one else CrossScanHip.apply(x)
+    # x: (B, C, H, W) | (B, H, W, C) | (B, 4, C, H, W) | (B, H, W, 4, C)
+    # y: (B, 4, C, L) | (B, L, 4, C)
+    # scans: 0: cross scan; 1 unidirectional; 2: bidirectional;
+    _require_hip("cross_scan_fn", scans, force_torch)
+    if in_channel_first and out_channel_first and (not one_by_one) and scans == 0:
+        return CrossScanHip.apply(x)
+    return CrossScanFlexHip.apply(x, in_channel_first, out_channel_first, one_by_one, scans)
 
 
 def cross_merge_fn(y, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0, force_torch=False):
-    # y: (B, 4, C, H, W) -> (B, C, L)
-    _require_default_mode("cross_merge_fn", in_channel_first, out_channel_first, one_by_one, scans, force_torch)
-    return CrossMergeHip.apply(y)
+    # y: (B, 4, C, H, W) | (B, H, W, 4, C)
+    # x: (B, C, H * W) | (B, H * W, C) | (B, 4, C, H * W) | (B, H * W, 4, C)
+    _require_hip("cross_merge_fn", scans, force_torch)
+    if in_channel_first and out_channel_first and (not one_by_one) and scans == 0:
+        return CrossMergeHip.apply(y)
+    return CrossMergeFlexHip.apply(y, in_channel_first, out_channel_first, one_by_one, scans)

@@ -1,0 +1,183 @@
+// CrossScan / CrossMerge for every layout and scan mode of the reference's "flex" kernel
+// (classification/models/csm_triton.py:278-400; torch semantics :22-179):
+//   x layout   channel-first (B,[4,]C,H,W)  or channel-last (B,H,W,[4,]C)
+//   y layout   channel-first (B,4,C,L)      or channel-last (B,L,4,C)
+//   one_by_one: x carries its own slice per direction instead of one map shared by the four
+//   scans      0: the four cross-scan routes (row-major, column-major, both reversed)
+//              1: four times the row-major route           2: row-major twice, reversed twice
+// The combination the SS2D core uses (both channel-first, shared map, scans = 0) has its own tiled kernels
+// (cross_scan.hip, cross_merge.hip); this file covers all the others with one kernel per operation: a thread per
+// OUTPUT element in the output's memory order (so stores are coalesced), the source found through the route.
+// Reads are coalesced whenever the route keeps the innermost dimension (every channel-last source, and the
+// non-transposing routes of channel-first sources); the transposing routes of channel-first sources gather through L2.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+struct FlexArgs {
+    const void *src;
+    void *dst;
+    int32_t B, C, H, W, L, x_cl, y_cl, one_by_one, scans, order;
+    int64_t total;
+    FastDiv divC, divL, divW, divH;
+};
+
+// scan position of direction k for the row-major spatial index r (csm_triton.py:308-328)
+__device__ __forceinline__ uint32_t flex_route(int k, int scans, uint32_t r, const FlexArgs &p) {
+    const bool reversed = scans == 1 ? false : k >= 2;
+    const bool transposed = scans == 0 && (k & 1);
+    uint32_t j = r;
+    if (transposed) {
+        uint32_t h, w;
+        divmod(r, p.divW, h, w);
+        j = w * (uint32_t)p.H + h;
+    }
+    return reversed ? (uint32_t)p.L - 1 - j : j;
+}
+// its inverse: the row-major spatial index that direction k visits at scan position j
+__device__ __forceinline__ uint32_t flex_route_inv(int k, int scans, uint32_t j, const FlexArgs &p) {
+    const bool reversed = scans == 1 ? false : k >= 2;
+    const bool transposed = scans == 0 && (k & 1);
+    uint32_t s = reversed ? (uint32_t)p.L - 1 - j : j;
+    if (transposed) {
+        uint32_t w, h;
+        divmod(s, p.divH, w, h);
+        s = h * (uint32_t)p.W + w;
+    }
+    return s;
+}
+
+__device__ __forceinline__ int64_t flex_x_offset(const FlexArgs &p, uint32_t b, int k, uint32_t c, uint32_t r) {
+    const int K = p.one_by_one ? 4 : 1, kk = p.one_by_one ? k : 0;
+    return p.x_cl ? (((int64_t)b * p.L + r) * K + kk) * p.C + c : (((int64_t)b * K + kk) * p.C + c) * p.L + r;
+}
+__device__ __forceinline__ int64_t flex_y_offset(const FlexArgs &p, uint32_t b, int k, uint32_t c, uint32_t j) {
+    return p.y_cl ? (((int64_t)b * p.L + j) * 4 + k) * p.C + c : (((int64_t)b * 4 + k) * p.C + c) * p.L + j;
+}
+
+// y (in its own memory order) <- x
+template <typename U>
+__global__ __launch_bounds__(kBlock) void cross_scan_flex_kernel(const FlexArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= p.total) return;
+    uint32_t b, k, c, j;
+    if (p.y_cl) {                           // (B, L, 4, C)
+        const int64_t q = idx / p.C;
+        c = (uint32_t)(idx - q * p.C);
+        k = (uint32_t)(q & 3);
+        const uint32_t bl = (uint32_t)(q >> 2);
+        divmod(bl, p.divL, b, j);
+    } else {                                // (B, 4, C, L)
+        const int64_t q = idx / p.L;
+        j = (uint32_t)(idx - q * p.L);
+        uint32_t bk;
+        divmod((uint32_t)q, p.divC, bk, c);
+        b = bk >> 2; k = bk & 3;
+    }
+    const uint32_t r = flex_route_inv((int)k, p.scans, j, p);
+    reinterpret_cast<U *>(p.dst)[idx] = reinterpret_cast<const U *>(p.src)[flex_x_offset(p, b, (int)k, c, r)];
+}
+
+template <typename T> __device__ __forceinline__ T flex_add(T a, T b) { return from_f32<T>(to_f32(a) + to_f32(b)); }
+
+// x (in its own memory order) <- y
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cross_merge_flex_kernel(const FlexArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= p.total) return;
+    const int K = p.one_by_one ? 4 : 1;
+    uint32_t b, k = 0, c, r;
+    if (p.x_cl) {                           // (B, L, [4,] C)
+        const int64_t q = idx / p.C;
+        c = (uint32_t)(idx - q * p.C);
+        uint32_t bl = (uint32_t)q;
+        if (p.one_by_one) { k = bl & 3; bl >>= 2; }
+        divmod(bl, p.divL, b, r);
+    } else {                                // (B, [4,] C, L)
+        const int64_t q = idx / p.L;
+        r = (uint32_t)(idx - q * p.L);
+        uint32_t bk;
+        divmod((uint32_t)q, p.divC, bk, c);
+        if (p.one_by_one) { b = bk >> 2; k = bk & 3; } else { b = bk; }
+    }
+    (void)K;
+    const T *y = reinterpret_cast<const T *>(p.src);
+    T *x = reinterpret_cast<T *>(p.dst);
+    if (p.one_by_one) {
+        x[idx] = y[flex_y_offset(p, b, (int)k, c, flex_route((int)k, p.scans, r, p))];
+        return;
+    }
+    T v[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) v[kk] = y[flex_y_offset(p, b, kk, c, flex_route(kk, p.scans, r, p))];
+    T out;
+    if (p.scans == 1) {
+        // the reference sums the four copies with a reduction (csm_triton.py:64, 75): fp32 accumulation, one rounding
+        out = from_f32<T>(((to_f32(v[0]) + to_f32(v[1])) + to_f32(v[2])) + to_f32(v[3]));
+    } else if (p.order == SS2D_MERGE_PAIRWISE) {
+        out = flex_add(flex_add(v[0], v[2]), flex_add(v[1], v[3]));
+    } else {
+        out = flex_add(flex_add(flex_add(v[0], v[1]), v[2]), v[3]);
+    }
+    x[idx] = out;
+}
+
+static int flex_fill(FlexArgs &a, int B, int C, int H, int W, int x_cl, int y_cl, int one_by_one, int scans) {
+    if (B < 0 || C < 0 || H < 0 || W < 0) return SS2D_EINVAL;
+    if ((x_cl | 1) != 1 || (y_cl | 1) != 1 || (one_by_one | 1) != 1 || scans < 0 || scans > 2) return SS2D_EINVAL;
+    const int64_t L = (int64_t)H * W;
+    if (L > 0x3fffffff || (int64_t)B * 4 * C > 0x7fffffff || (int64_t)B * L * 4 > 0x7fffffff) return SS2D_ENOTSUP;
+    a.B = B; a.C = C; a.H = H; a.W = W; a.L = (int32_t)L;
+    a.x_cl = x_cl; a.y_cl = y_cl; a.one_by_one = one_by_one; a.scans = scans; a.order = 0;
+    a.divC = make_fastdiv((uint32_t)(C > 0 ? C : 1)); a.divL = make_fastdiv((uint32_t)(L > 0 ? L : 1));
+    a.divW = make_fastdiv((uint32_t)(W > 0 ? W : 1)); a.divH = make_fastdiv((uint32_t)(H > 0 ? H : 1));
+    return SS2D_OK;
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_cross_scan_flex(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                                    int y_channel_last, int one_by_one, int scans, void *stream) {
+    using namespace ss2d;
+    FlexArgs a;
+    const int rc = flex_fill(a, B, C, H, W, x_channel_last, y_channel_last, one_by_one, scans);
+    if (rc != SS2D_OK) return rc;
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return SS2D_EINVAL;
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    a.src = x; a.dst = y;
+    a.total = (int64_t)B * 4 * C * a.L;
+    const int64_t n_wg = (a.total + kBlock - 1) / kBlock;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (elem_bytes) {
+        case 1: hipLaunchKernelGGL((cross_scan_flex_kernel<uint8_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((cross_scan_flex_kernel<uint16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((cross_scan_flex_kernel<uint32_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+        default: hipLaunchKernelGGL((cross_scan_flex_kernel<uint64_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+    }
+    return launch_status();
+}
+
+extern "C" int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H, int W, int dtype, int x_channel_last,
+                                     int y_channel_last, int one_by_one, int scans, int order, void *stream) {
+    using namespace ss2d;
+    FlexArgs a;
+    const int rc = flex_fill(a, B, C, H, W, x_channel_last, y_channel_last, one_by_one, scans);
+    if (rc != SS2D_OK) return rc;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (order != SS2D_MERGE_PAIRWISE && order != SS2D_MERGE_LEFT_TO_RIGHT) return SS2D_EINVAL;
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    a.src = y; a.dst = x; a.order = order;
+    a.total = (int64_t)B * (one_by_one ? 4 : 1) * C * a.L;
+    const int64_t n_wg = (a.total + kBlock - 1) / kBlock;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case SS2D_F32: hipLaunchKernelGGL((cross_merge_flex_kernel<float>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+        case SS2D_BF16: hipLaunchKernelGGL((cross_merge_flex_kernel<bf16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+        default: hipLaunchKernelGGL((cross_merge_flex_kernel<f16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+    }
+    return launch_status();
+}
