@@ -115,6 +115,19 @@ def kernel_lines(reps):
                         cross_merge_us=t_cm * 1e6, cross_merge_GBs=b_cm / t_cm / 1e9,
                         core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
                         scan_bytes=b_sc, **fused))
+        if name == "stage1":
+            # the other layouts / modes of the two operators (generic kernels), same shape; bytes = 5 E s as above
+            flex = {}
+            x_cl = x.permute(0, 2, 3, 1).contiguous()
+            y_cl = ys5.permute(0, 3, 4, 1, 2).contiguous()
+            for tag, (icf, ocf, scans) in dict(cl_cl_s0=(False, False, 0), cf_cl_s0=(True, False, 0),
+                                               cl_cf_s0=(False, True, 0), cf_cf_s2=(True, True, 2)).items():
+                xi, yi = (x if icf else x_cl), (ys5 if ocf else y_cl)
+                t_s = time_op(lambda: va.cross_scan_fn(xi, icf, ocf, False, scans), reps)
+                t_m = time_op(lambda: va.cross_merge_fn(yi, icf, ocf, False, scans), reps)
+                flex[tag] = dict(scan_us=t_s * 1e6, scan_GBs=b_cs / t_s / 1e9, merge_us=t_m * 1e6, merge_GBs=b_cm / t_m / 1e9)
+            out[-1]["flex_modes"] = flex
+            del x_cl, y_cl
         log("kernels", out[-1])
         del x, delta, Bm, Cm, xs, u, ys, ys5
     return out

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 MODES = list(itertools.product([True, False], [True, False], [False, True], [0, 1, 2]))
-SHAPES = [(2, 3, 5, 7), (1, 8, 14, 14), (2, 96, 7, 7), (1, 2, 1, 9), (1, 1, 33, 2)]
+SHAPES = [(2, 3, 5, 7), (1, 8, 14, 14), (2, 96, 7, 7), (1, 2, 1, 9), (1, 1, 33, 2), (2, 5, 8, 16)]
 
 
 def _x_shape(B, C, H, W, icf, obo):
@@ -24,7 +24,7 @@ def _x_shape(B, C, H, W, icf, obo):
     return (B, H, W, 4, C) if obo else (B, H, W, C)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8], ids=str)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8, torch.float64], ids=str)
 @pytest.mark.parametrize("icf,ocf,obo,scans", MODES)
 def test_cross_scan_every_mode_bit_exact(icf, ocf, obo, scans, dtype):
     print("CASE scan-flex", icf, ocf, obo, scans, dtype, flush=True)

@@ -18,7 +18,7 @@ struct FlexArgs {
     const void *src;
     void *dst;
     int32_t B, C, H, W, L, x_cl, y_cl, one_by_one, scans, order;
-    int64_t total;
+    uint32_t total;          // output elements (or channel vectors); host-checked < 2^32
     FastDiv divC, divL, divW, divH;
 };
 
@@ -58,66 +58,96 @@ __device__ __forceinline__ int64_t flex_y_offset(const FlexArgs &p, uint32_t b, 
 // y (in its own memory order) <- x
 template <typename U>
 __global__ __launch_bounds__(kBlock) void cross_scan_flex_kernel(const FlexArgs p) {
-    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
     if (idx >= p.total) return;
-    uint32_t b, k, c, j;
+    uint32_t b, k, c, j, q;
     if (p.y_cl) {                           // (B, L, 4, C)
-        const int64_t q = idx / p.C;
-        c = (uint32_t)(idx - q * p.C);
-        k = (uint32_t)(q & 3);
-        const uint32_t bl = (uint32_t)(q >> 2);
-        divmod(bl, p.divL, b, j);
+        divmod(idx, p.divC, q, c);
+        k = q & 3;
+        divmod(q >> 2, p.divL, b, j);
     } else {                                // (B, 4, C, L)
-        const int64_t q = idx / p.L;
-        j = (uint32_t)(idx - q * p.L);
+        divmod(idx, p.divL, q, j);
         uint32_t bk;
-        divmod((uint32_t)q, p.divC, bk, c);
+        divmod(q, p.divC, bk, c);
         b = bk >> 2; k = bk & 3;
     }
     const uint32_t r = flex_route_inv((int)k, p.scans, j, p);
     reinterpret_cast<U *>(p.dst)[idx] = reinterpret_cast<const U *>(p.src)[flex_x_offset(p, b, (int)k, c, r)];
 }
 
+// Channel-first on both sides with routes that do not transpose (scans 1 and 2): y_k is x_(k) copied or reversed
+// along L, so a thread moves 16 bytes; reversed routes read the mirrored 16 bytes and swap the elements inside.
+template <int kElemBytes> __device__ __forceinline__ uint4 flex_reverse16(uint4 v) {
+    if constexpr (kElemBytes == 8) return make_uint4(v.z, v.w, v.x, v.y);
+    uint4 r = make_uint4(v.w, v.z, v.y, v.x);
+    if constexpr (kElemBytes <= 2) {
+        r.x = (r.x >> 16) | (r.x << 16); r.y = (r.y >> 16) | (r.y << 16);
+        r.z = (r.z >> 16) | (r.z << 16); r.w = (r.w >> 16) | (r.w << 16);
+    }
+    if constexpr (kElemBytes == 1) {
+        r.x = ((r.x & 0x00ff00ffu) << 8) | ((r.x >> 8) & 0x00ff00ffu); r.y = ((r.y & 0x00ff00ffu) << 8) | ((r.y >> 8) & 0x00ff00ffu);
+        r.z = ((r.z & 0x00ff00ffu) << 8) | ((r.z >> 8) & 0x00ff00ffu); r.w = ((r.w & 0x00ff00ffu) << 8) | ((r.w >> 8) & 0x00ff00ffu);
+    }
+    return r;
+}
+
+template <int kElemBytes>
+__global__ __launch_bounds__(kBlock) void cross_scan_rows_vec_kernel(const FlexArgs p, uint32_t Lv, FastDiv divLv) {
+    const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;          // over (B, 4, C, L / vec)
+    if (idx >= p.total) return;
+    uint32_t q, jv, bk, c;
+    divmod(idx, divLv, q, jv);
+    divmod(q, p.divC, bk, c);
+    const uint32_t b = bk >> 2, k = bk & 3;
+    const bool reversed = p.scans == 2 && k >= 2;
+    const uint32_t K = p.one_by_one ? 4 : 1, kk = p.one_by_one ? k : 0;
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.src) + ((size_t)(b * K + kk) * p.C + c) * Lv;
+    uint4 v = src[reversed ? Lv - 1 - jv : jv];
+    if (reversed) v = flex_reverse16<kElemBytes>(v);
+    reinterpret_cast<uint4 *>(p.dst)[idx] = v;
+}
+
 template <typename T> __device__ __forceinline__ T flex_add(T a, T b) { return from_f32<T>(to_f32(a) + to_f32(b)); }
 
 // x (in its own memory order) <- y
-template <typename T>
+template <typename T> __device__ __forceinline__ T flex_combine(const T (&v)[4], int scans, int order) {
+    if (scans == 1)     // the reference sums the four copies with a reduction (csm_triton.py:64, 75): fp32, one rounding
+        return from_f32<T>(((to_f32(v[0]) + to_f32(v[1])) + to_f32(v[2])) + to_f32(v[3]));
+    if (order == SS2D_MERGE_PAIRWISE) return flex_add(flex_add(v[0], v[2]), flex_add(v[1], v[3]));
+    return flex_add(flex_add(flex_add(v[0], v[1]), v[2]), v[3]);
+}
+
+// x (in its own memory order) <- y.  kVec elements of T per thread along the channel axis (kVec > 1 only when both
+// sides are channel-last; C then counts vectors).
+template <typename T, int kVec>
 __global__ __launch_bounds__(kBlock) void cross_merge_flex_kernel(const FlexArgs p) {
-    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
     if (idx >= p.total) return;
-    const int K = p.one_by_one ? 4 : 1;
-    uint32_t b, k = 0, c, r;
+    uint32_t b, k = 0, c, r, q;
     if (p.x_cl) {                           // (B, L, [4,] C)
-        const int64_t q = idx / p.C;
-        c = (uint32_t)(idx - q * p.C);
-        uint32_t bl = (uint32_t)q;
-        if (p.one_by_one) { k = bl & 3; bl >>= 2; }
-        divmod(bl, p.divL, b, r);
+        divmod(idx, p.divC, q, c);
+        if (p.one_by_one) { k = q & 3; q >>= 2; }
+        divmod(q, p.divL, b, r);
     } else {                                // (B, [4,] C, L)
-        const int64_t q = idx / p.L;
-        r = (uint32_t)(idx - q * p.L);
+        divmod(idx, p.divL, q, r);
         uint32_t bk;
-        divmod((uint32_t)q, p.divC, bk, c);
+        divmod(q, p.divC, bk, c);
         if (p.one_by_one) { b = bk >> 2; k = bk & 3; } else { b = bk; }
     }
-    (void)K;
-    const T *y = reinterpret_cast<const T *>(p.src);
-    T *x = reinterpret_cast<T *>(p.dst);
+    struct alignas(sizeof(T) * kVec) Vec { T e[kVec]; };
+    const Vec *y = reinterpret_cast<const Vec *>(p.src);
+    Vec *x = reinterpret_cast<Vec *>(p.dst);
     if (p.one_by_one) {
         x[idx] = y[flex_y_offset(p, b, (int)k, c, flex_route((int)k, p.scans, r, p))];
         return;
     }
-    T v[4];
+    Vec v[4], out;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) v[kk] = y[flex_y_offset(p, b, kk, c, flex_route(kk, p.scans, r, p))];
-    T out;
-    if (p.scans == 1) {
-        // the reference sums the four copies with a reduction (csm_triton.py:64, 75): fp32 accumulation, one rounding
-        out = from_f32<T>(((to_f32(v[0]) + to_f32(v[1])) + to_f32(v[2])) + to_f32(v[3]));
-    } else if (p.order == SS2D_MERGE_PAIRWISE) {
-        out = flex_add(flex_add(v[0], v[2]), flex_add(v[1], v[3]));
-    } else {
-        out = flex_add(flex_add(flex_add(v[0], v[1]), v[2]), v[3]);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const T t[4] = {v[0].e[i], v[1].e[i], v[2].e[i], v[3].e[i]};
+        out.e[i] = flex_combine(t, p.scans, p.order);
     }
     x[idx] = out;
 }
@@ -146,10 +176,40 @@ extern "C" int ss2d_cross_scan_flex(const void *x, void *y, int B, int C, int H,
     if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
     if (!x || !y) return SS2D_EINVAL;
     a.src = x; a.dst = y;
-    a.total = (int64_t)B * 4 * C * a.L;
-    const int64_t n_wg = (a.total + kBlock - 1) / kBlock;
-    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    // both sides channel-last: the copy moves whole channel rows, so it is done in 16-byte pieces when they divide C
+    if (x_channel_last && y_channel_last && ((int64_t)C * elem_bytes) % 16 == 0 &&
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0) {
+        a.C = (int32_t)((int64_t)C * elem_bytes / 16);
+        a.divC = make_fastdiv((uint32_t)a.C);
+        elem_bytes = 16;
+    }
     hipStream_t s = (hipStream_t)stream;
+    // both sides channel-first, no transposing route: 16-byte pieces along L
+    const int vec = 16 / elem_bytes;
+    if (!x_channel_last && !y_channel_last && scans != 0 && elem_bytes < 16 && a.L % vec == 0 &&
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0) {
+        const uint32_t Lv = (uint32_t)(a.L / vec);
+        const int64_t total_v = (int64_t)B * 4 * C * Lv;
+        if (total_v > 0xffffffffll) return SS2D_ENOTSUP;
+        a.total = (uint32_t)total_v;
+        const uint32_t n = (uint32_t)((total_v + kBlock - 1) / kBlock);
+        const FastDiv dLv = make_fastdiv(Lv);
+        switch (elem_bytes) {
+            case 1: hipLaunchKernelGGL((cross_scan_rows_vec_kernel<1>), dim3(n), dim3(kBlock), 0, s, a, Lv, dLv); break;
+            case 2: hipLaunchKernelGGL((cross_scan_rows_vec_kernel<2>), dim3(n), dim3(kBlock), 0, s, a, Lv, dLv); break;
+            case 4: hipLaunchKernelGGL((cross_scan_rows_vec_kernel<4>), dim3(n), dim3(kBlock), 0, s, a, Lv, dLv); break;
+            default: hipLaunchKernelGGL((cross_scan_rows_vec_kernel<8>), dim3(n), dim3(kBlock), 0, s, a, Lv, dLv); break;
+        }
+        return launch_status();
+    }
+    const int64_t total = (int64_t)B * 4 * a.C * a.L;
+    if (total > 0xffffffffll) return SS2D_ENOTSUP;
+    a.total = (uint32_t)total;
+    const int64_t n_wg = (total + kBlock - 1) / kBlock;
+    if (elem_bytes == 16) {
+        hipLaunchKernelGGL((cross_scan_flex_kernel<uint4>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a);
+        return launch_status();
+    }
     switch (elem_bytes) {
         case 1: hipLaunchKernelGGL((cross_scan_flex_kernel<uint8_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
         case 2: hipLaunchKernelGGL((cross_scan_flex_kernel<uint16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
@@ -170,14 +230,24 @@ extern "C" int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H
     if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
     if (!x || !y) return SS2D_EINVAL;
     a.src = y; a.dst = x; a.order = order;
-    a.total = (int64_t)B * (one_by_one ? 4 : 1) * C * a.L;
-    const int64_t n_wg = (a.total + kBlock - 1) / kBlock;
-    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-    hipStream_t s = (hipStream_t)stream;
-    switch (dtype) {
-        case SS2D_F32: hipLaunchKernelGGL((cross_merge_flex_kernel<float>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
-        case SS2D_BF16: hipLaunchKernelGGL((cross_merge_flex_kernel<bf16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
-        default: hipLaunchKernelGGL((cross_merge_flex_kernel<f16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a); break;
+    const int eb = dtype == SS2D_F32 ? 4 : 2, vec = 16 / eb;
+    const bool use_vec = x_channel_last && y_channel_last && C % vec == 0 &&
+                         ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    if (use_vec) {
+        a.C = C / vec;
+        a.divC = make_fastdiv((uint32_t)a.C);
     }
+    const int64_t total = (int64_t)B * (one_by_one ? 4 : 1) * a.C * a.L;
+    if (total > 0xffffffffll) return SS2D_ENOTSUP;
+    a.total = (uint32_t)total;
+    const int64_t n_wg = (total + kBlock - 1) / kBlock;
+    hipStream_t s = (hipStream_t)stream;
+#define SS2D_FLEX_MERGE(T, V) hipLaunchKernelGGL((cross_merge_flex_kernel<T, V>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, a)
+    switch (dtype) {
+        case SS2D_F32: if (use_vec) SS2D_FLEX_MERGE(float, 4); else SS2D_FLEX_MERGE(float, 1); break;
+        case SS2D_BF16: if (use_vec) SS2D_FLEX_MERGE(bf16_t, 8); else SS2D_FLEX_MERGE(bf16_t, 1); break;
+        default: if (use_vec) SS2D_FLEX_MERGE(f16_t, 8); else SS2D_FLEX_MERGE(f16_t, 1); break;
+    }
+#undef SS2D_FLEX_MERGE
     return launch_status();
 }
