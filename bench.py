@@ -175,6 +175,9 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="replay the forward as one captured HIP graph (validated against eager) instead of eager "
                          "launches; measured equal within noise at batch 128, so eager is the default")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="skip PyTorch's TunableOp pass: by default the first (untimed) forward lets PyTorch-ROCm time the "
+                         "hipBLASLt / rocBLAS solutions for each GEMM shape of the model and keep the fastest (~12 s)")
     ap.add_argument("--layout", choices=["channel_first", "channel_last"], default="channel_last",
                     help="activation layout of the harness outside the SS2D core (same weights, same math)")
     args = ap.parse_args()
@@ -226,10 +229,34 @@ def main():
             torch.cuda.synchronize()
         return graph, out
 
+    gemm_mode = "library-default GEMM solutions"
     with torch.no_grad():
         model(x)
         torch.cuda.synchronize()
         log("first forward done")
+        if not args.no_gemm_tuning:
+            # The projection / MLP GEMMs stay PyTorch-ROCm library calls; TunableOp only picks, per GEMM shape, the
+            # fastest of the library's own solutions.  Tuning happens in this one untimed forward.
+            try:
+                import torch.cuda.tunable as tunable
+                tunable.enable(True)
+                tunable.tuning_enable(True)
+                for setter, value in (("set_filename", "/tmp/vmamba_amd_tunableop.csv"), ("set_max_tuning_duration", 30),
+                                      ("set_max_tuning_iterations", 20)):
+                    if hasattr(tunable, setter):
+                        getattr(tunable, setter)(value)
+                t_tune = time.perf_counter()
+                model(x)
+                torch.cuda.synchronize()
+                tunable.tuning_enable(False)
+                gemm_mode = "GEMM solutions picked by PyTorch TunableOp"
+                log(f"GEMM tuning forward: {time.perf_counter() - t_tune:.1f} s, {len(tunable.get_results())} shapes")
+            except Exception as e:      # an optimisation of library calls, never a requirement
+                log(f"TunableOp unavailable ({type(e).__name__}: {e}); library-default GEMM solutions")
+                try:
+                    tunable.enable(False)
+                except Exception:
+                    pass
         graph = None
         if args.graph:
             try:
@@ -278,7 +305,8 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
-                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}; SS2D core on HIP kernels"},
+                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}, {gemm_mode}; "
+                               f"SS2D core on HIP kernels"},
         "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "kernels": kernels,
     }))
 

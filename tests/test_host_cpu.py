@@ -44,3 +44,44 @@ def test_reference_core_runs_on_cpu():
     with torch.no_grad():
         y = m(torch.randn(1, 8, 5, 6))
     assert y.shape == (1, 8, 5, 6) and torch.isfinite(y).all()
+
+
+def test_vssm_state_dict_uses_reference_key_names_and_loads_legacy_checkpoints():
+    """State-dict keys are the reference's (classification/models/vmamba.py:1356-1363, 1402-1437, 1487-1490), and the
+    key prefixes of its older training code are renamed on load (vmamba.py:1557-1564)."""
+    import torch
+    from oracle.ss2d_core_ref import reference_vmamba_tiny
+    from vmamba_amd.vssm import VSSM
+
+    torch.manual_seed(0)
+    small = dict(depths=(1, 2), dims=(16, 32), num_classes=5)
+    src = VSSM(**small, channel_first=False, layers=__import__("oracle.ss2d_core_ref", fromlist=["TorchLayers"]).TorchLayers)
+    keys = set(src.state_dict().keys())
+    block = {"norm.weight", "norm.bias", "op.x_proj_weight", "op.A_logs", "op.Ds", "op.dt_projs_weight", "op.dt_projs_bias",
+             "op.in_proj.weight", "op.conv2d.weight", "op.out_norm.weight", "op.out_norm.bias", "op.out_proj.weight",
+             "norm2.weight", "norm2.bias", "mlp.fc1.weight", "mlp.fc1.bias", "mlp.fc2.weight", "mlp.fc2.bias"}
+    want = {f"patch_embed.{i}.{p}" for i in (0, 2, 5, 7) for p in ("weight", "bias")}
+    want |= {f"layers.{i}.blocks.{j}.{k}" for (i, j) in ((0, 0), (1, 0), (1, 1)) for k in block}
+    want |= {f"layers.0.downsample.{i}.{p}" for i in (1, 3) for p in ("weight", "bias")}
+    want |= {f"classifier.{m}.{p}" for m in ("norm", "head") for p in ("weight", "bias")}
+    assert keys == want
+    assert len(reference_vmamba_tiny().state_dict()) == 276
+
+    # a checkpoint written with the old names
+    legacy = {}
+    for k, v in src.state_dict().items():
+        k = k.replace(".norm.", ".ln_1.") if ".blocks." in k and ".norm." in k and ".op." not in k else k
+        k = k.replace(".op.", ".self_attention.")
+        k = k.replace("patch_embed.0.", "patch_embed.proj.").replace("patch_embed.2.", "patch_embed.norm.")
+        k = k.replace("classifier.norm.", "norm.").replace("classifier.head.", "head.")
+        legacy[k] = v.clone()
+    assert set(legacy) != keys
+    dst = VSSM(**small, channel_first=False, layers=src.layers[0].blocks[0].op.layers)
+    result = dst.load_state_dict(legacy, strict=True)
+    assert not result.missing_keys and not result.unexpected_keys
+    for (ka, a), (kb, b) in zip(src.state_dict().items(), dst.state_dict().items()):
+        assert ka == kb and torch.equal(a, b)
+    # channel-first models store 1x1-conv weights; a channel-last checkpoint loads into them (vmamba.py:47-49)
+    cf = VSSM(**small, channel_first=True, layers=src.layers[0].blocks[0].op.layers)
+    cf.load_state_dict(src.state_dict(), strict=True)
+    assert torch.equal(cf.layers[0].blocks[0].mlp.fc1.weight, src.layers[0].blocks[0].mlp.fc1.weight)

@@ -7,7 +7,14 @@ same weights run in two activation layouts: ``channel_first=True`` ("ln2d": (B,C
 LayerNorm2d) and ``channel_first=False`` ("ln": (B,H,W,C), nn.Linear, nn.LayerNorm).  The norm
 layers come from ``layers`` (default: this package's HIP LayerNorm kernels); convolutions, the projection and
 MLP GEMMs and activations are stock torch; drop-path is the identity at inference.
+
+Module names -- hence state_dict keys -- are the reference's (``patch_embed.{0,2,5,7}``,
+``layers.{i}.blocks.{j}.{norm,op,norm2,mlp}``, ``layers.{i}.downsample.{1,3}``, ``classifier.{norm,head}``), and
+``VSSM._load_from_state_dict`` applies the reference's renames for checkpoints written by its older training code
+(vmamba.py:1531-1570), so a released VMamba checkpoint of this architecture loads with ``load_state_dict``.
 """
+from collections import OrderedDict
+
 import torch
 import torch.nn as nn
 
@@ -76,11 +83,30 @@ class VSSM(nn.Module):
             down = (nn.Sequential(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
                                   Norm(dims[i + 1]))
                     if i + 1 < len(dims) else nn.Identity())
-            stages.append(nn.Sequential(*blocks, down))
+            stages.append(nn.Sequential(OrderedDict(blocks=nn.Sequential(*blocks), downsample=down)))
         self.layers = nn.ModuleList(stages)
-        self.classifier = nn.Sequential(Norm(dims[-1]), _to_cf(cf), nn.AdaptiveAvgPool2d(1), nn.Flatten(1),
-                                        nn.Linear(dims[-1], num_classes))
+        self.classifier = nn.Sequential(OrderedDict(
+            norm=Norm(dims[-1]), permute=_to_cf(cf), avgpool=nn.AdaptiveAvgPool2d(1), flatten=nn.Flatten(1),
+            head=nn.Linear(dims[-1], num_classes)))
         self.apply(self._init_weights)
+
+    # key prefixes of checkpoints from the reference's previous training code -> current names (vmamba.py:1557-1564)
+    LEGACY_KEYS = (("patch_embed.proj", "patch_embed.0"), ("patch_embed.norm", "patch_embed.2"),
+                   ("norm", "classifier.norm"), ("head", "classifier.head"))
+    LEGACY_BLOCK_KEYS = (("ln_1", "norm"), ("self_attention", "op"))
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        def rename(src, dst):
+            for key in [k for k in state_dict if k.startswith(prefix + src)]:
+                state_dict[prefix + dst + key[len(prefix + src):]] = state_dict.pop(key)
+
+        for i, stage in enumerate(self.layers):
+            for j in range(len(stage.blocks)):
+                for src, dst in self.LEGACY_BLOCK_KEYS:
+                    rename(f"layers.{i}.blocks.{j}.{src}", f"layers.{i}.blocks.{j}.{dst}")
+        for src, dst in self.LEGACY_KEYS:
+            rename(src, dst)
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     @staticmethod
     def _init_weights(m):
