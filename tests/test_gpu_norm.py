@@ -51,7 +51,7 @@ def test_layer_norm_rows_without_affine_and_known_answers():
 
 # B, C, H, W
 CF = [(2, 96, 56, 56), (2, 48, 5, 7), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (1, 1000, 3, 3), (2, 7, 9, 4), (1, 96, 1, 1),
-      (1, 1300, 3, 5), (1, 97, 8, 9), (2, 200, 3, 70), (1, 500, 6, 6)]
+      (1, 1300, 3, 5), (1, 97, 8, 9), (2, 200, 3, 70), (1, 500, 6, 6), (2, 768, 6, 6), (3, 40, 2, 2), (1, 136, 4, 9)]
 
 
 @pytest.mark.parametrize("B,C,H,W", CF)

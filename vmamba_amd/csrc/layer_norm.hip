@@ -213,14 +213,24 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_reg_kernel(const in_t *_
     const int p = threadIdx.x % kTP, g = threadIdx.x / kTP;
     const int l = l0 + p;
     const bool valid = l < L;
-    const in_t *xb = x + (size_t)b * C * L + l;
+    // The image sits behind a buffer descriptor and elements outside it (position past L, channel past C) are
+    // pointed beyond its end, where the hardware returns 0: every load is unconditional, so the kVPT loads of a lane
+    // are all in flight together (a select on the loaded value makes the compiler branch around each load and
+    // wait for it).  Host-checked: C * L * sizeof(in_t) < 2 GiB.
+    const in_t *xb = x + (size_t)b * C * L;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<in_t *>(xb), 0, C * L * (int)sizeof(in_t), 0x00020000);
 
     float v[kVPT];
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < kVPT; ++i) {
         const int c = g + i * kG;
-        v[i] = (valid && c < C) ? to_f32(xb[(size_t)c * L]) : 0.0f;
+        const uint32_t off = (valid && c < C) ? (uint32_t)(c * L + l) * (uint32_t)sizeof(in_t) : 0x7ffffff0u;
+        if constexpr (sizeof(in_t) == 4) {
+            v[i] = bits_to_f32((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)off, 0, 0));
+        } else {
+            v[i] = to_f32(in_t{(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(x_rsrc, (int)off, 0, 0)});
+        }
         s += v[i];
     }
     red[0][g][p] = s;
@@ -284,6 +294,118 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_reg_kernel(const in_t *_
     }
 }
 
+// Quad variant of the register kernel for fp32 channel-first input (the merged scan output feeding out_norm): a lane
+// owns FOUR consecutive positions, so every load is 16 bytes (the address pipeline is priced per instruction, and the
+// 4-byte loads of the variant above leave it the bottleneck on short images).  Threads are laid out quads x groups;
+// group g holds channels g, g+kG, ... of its four positions.  Sums cross the groups of a wavefront by lane
+// exchanges and the wavefronts through a few floats of LDS.
+template <typename w_t, typename out_t, bool kOutChannelLast, int kQ, int kG, int kCPL>
+__global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float *__restrict__ x, const w_t *__restrict__ weight,
+                                                                    const w_t *__restrict__ bias, out_t *__restrict__ y, int C,
+                                                                    int L, int tiles_per_image, int Cp, float eps) {
+    static_assert(kQ * kG == kBlock && kQ <= kWave, "one thread per (position quad, group)");
+    constexpr int kTP = 4 * kQ;                      // positions per workgroup
+    constexpr int kWaves = kBlock / kWave;
+    extern __shared__ __align__(16) unsigned char lnq_smem[];
+    __shared__ float red[2][kWaves][kTP];
+    const uint32_t b = blockIdx.x / tiles_per_image;
+    const int l0 = (int)(blockIdx.x - b * tiles_per_image) * kTP;
+    const int q = threadIdx.x % kQ, g = threadIdx.x / kQ;
+    const int wave = threadIdx.x / kWave;
+    const int l = l0 + 4 * q;
+    const bool valid = l < L;                        // L % 4 == 0 (host-checked): a quad is inside or outside
+    const float *xb = x + (size_t)b * C * L;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(xb), 0, C * L * 4, 0x00020000);
+
+    float v[kCPL][4];
+    float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < kCPL; ++i) {
+        const int c = g + i * kG;
+        // outside the image: pointed past the end of the buffer, where the hardware returns 0 (loads stay unconditional)
+        const uint32_t off = (valid && c < C) ? (uint32_t)(c * L + l) * 4u : 0x7ffffff0u;
+        const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { v[i][j] = bits_to_f32(t[j]); s[j] += v[i][j]; }
+    }
+    auto reduce_groups = [&](float (&acc)[4], int which) {
+#pragma unroll
+        for (int m = kQ; m < kWave; m *= 2)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] += __shfl_xor(acc[j], m, kWave);
+        if ((threadIdx.x & (kWave - 1)) < kQ) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) red[which][wave][4 * q + j] = acc[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) t += red[which][w][4 * q + j];
+            acc[j] = t;
+        }
+    };
+    reduce_groups(s, 0);
+    float mean[4], qq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mean[j] = s[j] / (float)C;
+#pragma unroll
+    for (int i = 0; i < kCPL; ++i) {
+        const bool live = g + i * kG < C;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float d = v[i][j] - mean[j];
+            qq[j] = live ? fmaf(d, d, qq[j]) : qq[j];
+        }
+    }
+    reduce_groups(qq, 1);
+    float rstd[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rstd[j] = rsqrtf(qq[j] / (float)C + eps);
+
+    if constexpr (!kOutChannelLast) {
+        out_t *yb = y + (size_t)b * C * L + l;
+#pragma unroll
+        for (int i = 0; i < kCPL; ++i) {
+            const int c = g + i * kG;
+            if (valid && c < C) {
+                const float wv = weight ? to_f32(weight[c]) : 1.0f, bv = bias ? to_f32(bias[c]) : 0.0f;
+                out_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = from_f32<out_t>(fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv));
+                out_t *dst = yb + (size_t)c * L;
+                if constexpr (sizeof(out_t) == 4) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+                } else {
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2((uint32_t)o[0].bits | ((uint32_t)o[1].bits << 16),
+                                                                 (uint32_t)o[2].bits | ((uint32_t)o[3].bits << 16));
+                }
+            }
+        }
+    } else {
+        out_t *ot = reinterpret_cast<out_t *>(lnq_smem);          // [kTP][Cp]
+#pragma unroll
+        for (int i = 0; i < kCPL; ++i) {
+            const int c = g + i * kG;
+            if (c < C) {
+                const float wv = weight ? to_f32(weight[c]) : 1.0f, bv = bias ? to_f32(bias[c]) : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ot[(4 * q + j) * Cp + c] = from_f32<out_t>(fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv));
+            }
+        }
+        __syncthreads();
+        const int nl = min(kTP, L - l0);
+        out_t *yb = y + ((size_t)b * L + l0) * C;
+        constexpr int kPiece = 16 / (int)sizeof(out_t);            // elements per 16-byte piece; C % kPiece == 0 (host)
+        const int pieces = C / kPiece;
+        for (int idx = threadIdx.x; idx < nl * pieces; idx += kBlock) {
+            const int pp = idx / pieces, cc = (idx - pp * pieces) * kPiece;
+            *reinterpret_cast<uint4 *>(yb + (size_t)pp * C + cc) = *reinterpret_cast<const uint4 *>(ot + pp * Cp + cc);
+        }
+    }
+}
+
 // ---- host side ----------------------------------------------------------------------------------
 static bool ln_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -340,7 +462,7 @@ static int launch_ln_cf_reg(const void *x, const void *w, const void *b, void *y
                             int out_channel_last, hipStream_t stream) {
     const int tiles = (L + kTP - 1) / kTP;
     const int64_t n_wg = (int64_t)B * tiles;
-    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    if (n_wg > 0x7fffffff || (int64_t)C * L * (int64_t)sizeof(in_t) >= 0x7ffffff0ll) return SS2D_ENOTSUP;
     // LDS pitch of the turn-round tile: lanes walk positions, so consecutive rows must land in different banks
     int Cp = sizeof(out_t) == 2 ? ((C + 1) & ~1) : (C | 1);
     if (sizeof(out_t) == 2 && (Cp / 2) % 2 == 0) Cp += 2;
@@ -355,9 +477,40 @@ static int launch_ln_cf_reg(const void *x, const void *w, const void *b, void *y
     return launch_status();
 }
 
+template <typename w_t, typename out_t, int kQ, int kG, int kCPL>
+static int launch_ln_cf_quad(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
+                             int out_channel_last, hipStream_t stream) {
+    constexpr int kTP = 4 * kQ;
+    const int tiles = (L + kTP - 1) / kTP;
+    const int64_t n_wg = (int64_t)B * tiles;
+    // LDS pitch of the turn-round tile: rows 16-byte aligned, and four rows apart never in the same banks
+    const int piece = 16 / (int)sizeof(out_t);
+    const int Cp = ((C + piece - 1) / piece) * piece + piece;
+    if (out_channel_last) {
+        const size_t smem = (size_t)kTP * Cp * sizeof(out_t);
+        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<w_t, out_t, true, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
+                           stream, (const float *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+    } else {
+        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<w_t, out_t, false, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), 0,
+                           stream, (const float *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+    }
+    return launch_status();
+}
+
 template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
                         int out_channel_last, hipStream_t stream) {
+    if constexpr (sizeof(in_t) == 4) {
+        // fp32 input, quads of positions: 16-byte loads (and 16-byte channel-last stores)
+        const bool quad_ok = L % 4 == 0 && ln_aligned16(x) && (int64_t)C * L * 4 < 0x7ffffff0ll && (int64_t)B * ((L + 15) / 16) <= 0x7fffffff &&
+                             (out_channel_last ? (C % (16 / (int)sizeof(out_t)) == 0 && ln_aligned16(y)) : ln_aligned16(y));
+        if (quad_ok) {
+            if (C <= 96) return launch_ln_cf_quad<w_t, out_t, 16, 16, 6>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 192) return launch_ln_cf_quad<w_t, out_t, 16, 16, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 384) return launch_ln_cf_quad<w_t, out_t, 8, 32, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 768) return launch_ln_cf_quad<w_t, out_t, 4, 64, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+        }
+    }
     if (C <= 96) return launch_ln_cf_reg<in_t, w_t, out_t, 64, 4, 24>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     if (C <= 192) return launch_ln_cf_reg<in_t, w_t, out_t, 64, 4, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     if (C <= 384) return launch_ln_cf_reg<in_t, w_t, out_t, 32, 8, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
