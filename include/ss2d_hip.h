@@ -119,6 +119,37 @@ typedef struct ss2d_scan_params {
 int ss2d_selective_scan_fwd(const ss2d_scan_params *params, void *stream);
 
 /*
+ * Selective-scan backward.  Replaces selective_scan_bwd + selective_scan_bwd_kernel
+ * (kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:233-355,
+ *  .../selective_scan_bwd_kernel_oflex.cuh); inputs as in the forward plus
+ *   dout   (batch, dim, seqlen)   dout_dtype: SS2D_F32 or in_dtype (strides in elements, sequence stride 1)
+ * and caller-allocated outputs
+ *   du, ddelta  (batch, dim, seqlen) contiguous, in_dtype; ddelta is per CHANNEL (with delta_dim < dim the caller
+ *               sums the dim/delta_dim channels of a delta row, as selective_scan_oflex.cpp:347-352 does)
+ *   dA (dim, dstate), dB, dC (batch, n_groups, dstate, seqlen), dD (dim), ddelta_bias (dim): fp32, contiguous,
+ *               ZERO-INITIALISED by the caller (accumulated with atomics over the rows that share them);
+ *               dD / ddelta_bias NULL exactly when D / delta_bias is NULL.
+ * The forward states are recomputed inside the kernel, so the forward's `x` output is not needed.
+ * Returns SS2D_ENOTSUP when ceil(seqlen/512) * dstate exceeds ~3000 (per-pass states kept in LDS).
+ */
+typedef struct ss2d_scan_bwd_params {
+    int32_t batch, dim, seqlen, dstate, n_groups, delta_dim;
+    int32_t in_dtype, dout_dtype;
+    int32_t delta_softplus;
+    int32_t reserved;
+    const void *u, *delta, *A, *B, *C, *D, *delta_bias, *dout;
+    void *du, *ddelta, *dA, *dB, *dC, *dD, *ddelta_bias;
+    int64_t u_batch_stride, u_d_stride;
+    int64_t delta_batch_stride, delta_d_stride;
+    int64_t A_d_stride, A_dstate_stride;
+    int64_t B_batch_stride, B_group_stride, B_dstate_stride;
+    int64_t C_batch_stride, C_group_stride, C_dstate_stride;
+    int64_t dout_batch_stride, dout_d_stride;
+} ss2d_scan_bwd_params;
+
+int ss2d_selective_scan_bwd(const ss2d_scan_bwd_params *params, void *stream);
+
+/*
  * LayerNorm over the channel axis, the step after CrossMerge (out_norm) and the block norms of the model.
  * Replaces the torch calls of LayerNorm2d.forward (classification/models/vmamba.py:52-57: permute,
  * F.layer_norm, permute) and of nn.LayerNorm on (B,H,W,C) activations, including the transposition

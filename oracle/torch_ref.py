@@ -159,3 +159,40 @@ def selective_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=Fa
         y = y + u32 * D.float()[None, :, None]
     out = y if out_float else y.to(dtype_in)
     return (out, h) if return_last_state else out
+
+
+def selective_scan_f64(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False):
+    """The same recurrence in float64, differentiable by autograd (no dtype round trips): the gradient oracle."""
+    batch, dim, L = u.shape
+    G, N = B.shape[1], B.shape[2]
+    dl = delta
+    if delta.shape[1] != dim:
+        rep = dim // delta.shape[1]
+        dl = dl.repeat_interleave(rep, dim=1)
+        if delta_bias is not None:
+            delta_bias = delta_bias.repeat_interleave(rep)
+    if delta_bias is not None:
+        dl = dl + delta_bias[None, :, None]
+    if delta_softplus:
+        dl = F.softplus(dl)
+    Bf = B.repeat_interleave(dim // G, dim=1)
+    Cf = C.repeat_interleave(dim // G, dim=1)
+    decay = torch.exp(torch.einsum("bdl,dn->bdln", dl, A))
+    drive = torch.einsum("bdl,bdnl,bdl->bdln", dl, Bf, u)
+    h = torch.zeros(batch, dim, N, dtype=u.dtype)
+    ys = []
+    for t in range(L):
+        h = decay[:, :, t] * h + drive[:, :, t]
+        ys.append(torch.einsum("bdn,bdn->bd", h, Cf[..., t]))
+    y = torch.stack(ys, dim=2)
+    if D is not None:
+        y = y + u * D[None, :, None]
+    return y
+
+
+def selective_scan_grads(u, delta, A, B, C, D, delta_bias, dout, delta_softplus):
+    """[du, ddelta, dA, dB, dC, dD, ddelta_bias] of sum(y * dout) by float64 autograd (None where the input is None)."""
+    leaves = [None if t is None else t.detach().double().requires_grad_(True) for t in (u, delta, A, B, C, D, delta_bias)]
+    y = selective_scan_f64(*leaves, delta_softplus=delta_softplus)
+    y.backward(dout.double())
+    return [None if t is None else t.grad for t in leaves]

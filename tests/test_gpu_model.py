@@ -99,3 +99,33 @@ def test_vmamba_tiny_logits_match_reference_core(channel_first):
         got = hip(x.to(DEV)).cpu()
     assert got.shape == (2, 1000)
     assert torch.allclose(got, want, rtol=2e-3, atol=2e-3)
+
+
+def test_small_vssm_trains_on_the_gpu():
+    """One training step: gradients of a small model on the GPU (HIP scan / cross-scan / cross-merge backward, torch
+    autograd for the rest) against the all-torch CPU model with the same weights."""
+    print("CASE vssm-train", flush=True)
+    from oracle.ss2d_core_ref import TorchLayers
+    torch.manual_seed(11)
+    cfg = dict(depths=(1, 1), dims=(16, 32), num_classes=7)
+    ref = VSSM(**cfg, channel_first=True, ss2d_cls=RefSS2D, layers=TorchLayers).train()
+    hip = VSSM(**cfg, channel_first=False).train()
+    hip.load_state_dict(ref.state_dict())
+    hip = hip.to(DEV)
+    x = torch.randn(2, 3, 32, 32, generator=torch.Generator().manual_seed(12))
+    target = torch.tensor([1, 5])
+    loss_ref = torch.nn.functional.cross_entropy(ref(x), target)
+    loss_ref.backward()
+    loss_hip = torch.nn.functional.cross_entropy(hip(x.to(DEV)), target.to(DEV))
+    loss_hip.backward()
+    assert abs(loss_hip.item() - loss_ref.item()) < 1e-3
+    grads_ref = dict(ref.named_parameters())
+    n = 0
+    for name, p in hip.named_parameters():
+        g, w = p.grad, grads_ref[name].grad
+        assert g is not None and torch.isfinite(g).all(), name
+        w = w.view(g.shape)                   # 1x1-conv weights of the channel-first model are the same matrices
+        scale = w.abs().max().item()
+        assert (g.cpu() - w).abs().max().item() <= 5e-3 * scale + 1e-6, name
+        n += 1
+    assert n == len(grads_ref)

@@ -412,3 +412,29 @@ def test_dwconv_against_brute_force():
     # identity kernel (centre tap 1) without SiLU returns the input
     ident = torch.zeros(D, 1, 3, 3); ident[:, 0, 1, 1] = 1.0
     assert torch.equal(torch_ref.dwconv3x3_silu(x, ident, None, apply_silu=False), x)
+
+
+def test_selective_scan_gradient_oracle_against_finite_differences():
+    """The float64 restatement used as gradient oracle: equal to the fp32 one on the forward, and its autograd
+    gradients equal to central finite differences (torch.autograd.gradcheck) for every input."""
+    g = torch.Generator().manual_seed(77)
+    batch, dim, G, N, L = 1, 4, 2, 3, 6
+    u = torch.randn(batch, dim, L, generator=g, dtype=torch.float64)
+    delta = 0.5 * torch.rand(batch, 2, L, generator=g, dtype=torch.float64)          # two channels per delta row
+    A = -0.5 * torch.rand(dim, N, generator=g, dtype=torch.float64)
+    Bm = torch.randn(batch, G, N, L, generator=g, dtype=torch.float64)
+    Cm = torch.randn(batch, G, N, L, generator=g, dtype=torch.float64)
+    D = torch.randn(dim, generator=g, dtype=torch.float64)
+    bias = 0.5 * torch.rand(2, generator=g, dtype=torch.float64)
+    for softplus in (True, False):
+        y64 = torch_ref.selective_scan_f64(u, delta, A, Bm, Cm, D, bias, softplus)
+        y32 = torch_ref.selective_scan(u.float(), delta.float(), A.float(), Bm.float(), Cm.float(), D.float(), bias.float(), softplus)
+        assert torch.allclose(y64.float(), y32, rtol=1e-5, atol=1e-5)
+        leaves = [t.clone().requires_grad_(True) for t in (u, delta, A, Bm, Cm, D, bias)]
+        assert torch.autograd.gradcheck(lambda *a: torch_ref.selective_scan_f64(*a, delta_softplus=softplus), leaves,
+                                        eps=1e-6, atol=1e-6, rtol=1e-5)
+        dout = torch.randn(y64.shape, generator=g, dtype=torch.float64)
+        grads = torch_ref.selective_scan_grads(u, delta, A, Bm, Cm, D, bias, dout, softplus)
+        want = torch.autograd.grad((torch_ref.selective_scan_f64(*leaves, delta_softplus=softplus) * dout).sum(), leaves)
+        for a, b in zip(grads, want):
+            assert torch.equal(a, b)

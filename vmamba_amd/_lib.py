@@ -16,7 +16,8 @@ ABI_VERSION = 1
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
            "ss2d_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
-           "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_merge_flex")
+           "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_merge_flex",
+           "ss2d_selective_scan_bwd")
 
 
 class ScanParams(ctypes.Structure):
@@ -30,6 +31,21 @@ class ScanParams(ctypes.Structure):
                                          "B_batch_stride", "B_group_stride", "B_dstate_stride",
                                          "C_batch_stride", "C_group_stride", "C_dstate_stride",
                                          "out_batch_stride", "out_d_stride")]
+    )
+
+
+class ScanBwdParams(ctypes.Structure):
+    """struct ss2d_scan_bwd_params (include/ss2d_hip.h)."""
+    _fields_ = (
+        [(n, ctypes.c_int32) for n in ("batch", "dim", "seqlen", "dstate", "n_groups", "delta_dim",
+                                       "in_dtype", "dout_dtype", "delta_softplus", "reserved")]
+        + [(n, ctypes.c_void_p) for n in ("u", "delta", "A", "B", "C", "D", "delta_bias", "dout",
+                                          "du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias")]
+        + [(n, ctypes.c_int64) for n in ("u_batch_stride", "u_d_stride", "delta_batch_stride", "delta_d_stride",
+                                         "A_d_stride", "A_dstate_stride",
+                                         "B_batch_stride", "B_group_stride", "B_dstate_stride",
+                                         "C_batch_stride", "C_group_stride", "C_dstate_stride",
+                                         "dout_batch_stride", "dout_d_stride")]
     )
 
 
@@ -89,6 +105,8 @@ def lib():
         L.ss2d_cross_scan_flex.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 9 + [ctypes.c_void_p]
         L.ss2d_cross_merge_flex.restype = ctypes.c_int
         L.ss2d_cross_merge_flex.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 10 + [ctypes.c_void_p]
+        L.ss2d_selective_scan_bwd.restype = ctypes.c_int
+        L.ss2d_selective_scan_bwd.argtypes = [ctypes.POINTER(ScanBwdParams), ctypes.c_void_p]
         if L.ss2d_abi_version() != ABI_VERSION:
             raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L

@@ -80,7 +80,7 @@ __device__ __forceinline__ float dpp_move(float old, float v) {
                                                              kRowMask, 0xF, false));
 }
 constexpr int kDppRowShr1 = 0x111, kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
-constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143, kDppWaveShr1 = 0x138;
+constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143, kDppWaveShr1 = 0x138, kDppWaveShl1 = 0x130;
 
 __device__ __forceinline__ float read_lane(float v, int lane) {
     return bits_to_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_to_bits(v), lane));

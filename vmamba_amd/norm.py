@@ -6,6 +6,7 @@ torch modules, so state_dicts are interchangeable.  GPU tensors only: there is n
 """
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import _lib
 
@@ -60,11 +61,21 @@ def layer_norm_cf_hip(x, weight, bias, eps=1e-5, out_channel_last=False, out_dty
     return y
 
 
+def needs_grad(*tensors):
+    """True when autograd has to see this call: the HIP LayerNorm / conv kernels are inference kernels, so modules
+    route such calls to the differentiable torch operators the reference itself uses."""
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
 class LayerNorm(nn.LayerNorm):
     def forward(self, x):
+        if needs_grad(x, self.weight, self.bias):
+            return F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps)
         return layer_norm_hip(x, self.weight, self.bias, self.eps)
 
 
 class LayerNorm2d(nn.LayerNorm):
     def forward(self, x):
+        if needs_grad(x, self.weight, self.bias):          # vmamba.py:52-57
+            return F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight, self.bias, self.eps).permute(0, 3, 1, 2)
         return layer_norm_cf_hip(x, self.weight, self.bias, self.eps, out_channel_last=False)

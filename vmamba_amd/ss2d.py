@@ -24,7 +24,7 @@ from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
-from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip
+from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip, needs_grad
 
 
 class Linear2d(nn.Linear):
@@ -48,14 +48,19 @@ class HipLayers:
     @staticmethod
     def out_norm(norm, y, channel_first, dtype):
         """out_norm of forward_core on the merged channel-first map y (B, D, H, W), returned in the block's
-        layout and dtype: one kernel reads (B, D, L) and writes the normalised (B, D, L) or (B, L, D)."""
+        layout and dtype: one kernel reads (B, D, L) and writes the normalised (B, D, L) or (B, L, D).  Under
+        autograd: the reference's own torch operators (vmamba.py:641-646)."""
+        if needs_grad(y, norm.weight, norm.bias):
+            out = F.layer_norm(y.permute(0, 2, 3, 1), norm.normalized_shape, norm.weight, norm.bias, norm.eps)
+            return (out.permute(0, 3, 1, 2) if channel_first else out).to(dtype)
         return layer_norm_cf_hip(y, norm.weight, norm.bias, norm.eps, out_channel_last=not channel_first, out_dtype=dtype)
 
     @staticmethod
     def conv_act(conv2d, x, channel_first):
         """Depthwise conv + SiLU on the in_proj output x ((B,D,H,W) if channel_first else (B,H,W,D)); returns the
         channel-first (B,D,H,W) input of forward_core (vmamba.py:654-658).  ``conv2d`` None means no conv."""
-        if conv2d is not None and conv2d.kernel_size == (3, 3) and conv2d.padding == (1, 1) and conv2d.stride == (1, 1):
+        fusable = conv2d is not None and conv2d.kernel_size == (3, 3) and conv2d.padding == (1, 1) and conv2d.stride == (1, 1)
+        if fusable and not needs_grad(x, conv2d.weight, conv2d.bias):
             return dwconv3x3_silu_hip(x, conv2d.weight, conv2d.bias, in_channel_last=not channel_first, apply_silu=True)
         if not channel_first:
             x = x.permute(0, 3, 1, 2).contiguous()
@@ -168,7 +173,9 @@ class SS2D(nn.Module):
         B, D, H, W = x.shape
         K, L = self.k_group, H * W
         consts = self._inference_constants(B)
-        if self.d_state == 1 and self.fused_core and core_fits(H, W, x.dtype):
+        # the fused kernel is an inference kernel; under autograd the three operators (each with a backward) run
+        trains = needs_grad(x, self.x_proj_weight, self.dt_projs_weight, self.A_logs, self.Ds, self.dt_projs_bias)
+        if self.d_state == 1 and self.fused_core and not trains and core_fits(H, W, x.dtype):
             return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
         dts, Bs, Cs = self.project(xs, consts)
