@@ -116,6 +116,13 @@ def kernel_lines(reps):
                         core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
                         scan_bytes=b_sc, **fused))
         if name == "stage1":
+            # the scan's backward at the same shape (fp32 dout, as the oflex forward hands back): algorithmic bytes =
+            # u, delta, dout in; du, ddelta out; B, C in and fp32 dB, dC out once per (batch, direction)
+            dout = torch.randn(B, K * D, L, device=dev, generator=g)
+            t_b = time_op(lambda: va.selective_scan_bwd(u, delta, A, Bm, Cm, Dv, bias, dout, None, True, 1), max(reps // 4, 2), warm=2)
+            b_b = B * K * D * L * (2 + 2 + 4 + 2 + 2) + B * K * N * L * (2 * 2 + 2 * 4)
+            out[-1].update(scan_bwd_us=t_b * 1e6, scan_bwd_GBs=b_b / t_b / 1e9, scan_bwd_bytes=b_b)
+            del dout
             # the other layouts / modes of the two operators (generic kernels), same shape; bytes = 5 E s as above
             flex = {}
             x_cl = x.permute(0, 2, 3, 1).contiguous()
