@@ -52,6 +52,9 @@ CASES = [
     (1, 4, 1, 16, 300, None, True),        # 16 states
     (2, 4, 2, 2, 600, None, False),        # no softplus
     (1, 3, 1, 1, 9, None, True),           # shorter than a lane's 8 items + 1
+    (2, 32, 2, 1, 700, None, True),        # 16 channels per group: dB / dC summed per workgroup in LDS
+    (1, 60, 2, 2, 300, None, True),        # 30 channels per group in two chunks of 15, two states
+    (1, 27, 1, 1, 520, 9, True),           # 27 channels in chunks of 14 + 13, delta rows shared by three channels
 ]
 
 

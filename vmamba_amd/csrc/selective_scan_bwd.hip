@@ -32,18 +32,14 @@ struct ScanBwdArgs {
 
 __device__ __forceinline__ float lane_reverse(float v, int lane) { return __shfl(v, kWave - 1 - lane, kWave); }
 
-template <typename in_t, typename dy_t, bool kSoftplus>
-__global__ __launch_bounds__(kBlock) void scan_bwd_kernel(const ScanBwdArgs p) {
-    extern __shared__ __align__(16) float bwd_smem[];      // per wavefront: h_in [n_pass][N], g carry [N], a_next [N]
+// One (batch, channel) row by one wavefront.  `h_in` is the wavefront's LDS scratch ((n_pass + 2) * N floats).
+// kGroupAcc: dB / dC contributions go into the workgroup's LDS accumulators accB / accC ([N][L], shared by the
+// channels of one group that the workgroup walks) instead of straight to memory.
+template <typename in_t, typename dy_t, bool kSoftplus, bool kGroupAcc>
+__device__ __forceinline__ void scan_bwd_row(const ScanBwdArgs &p, int b, int d, float *h_in, float *accB, float *accC) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int row = (int)(blockIdx.x * kWavesPerWg) + wave;
-    if (row >= p.rows) return;           // whole wavefront leaves; no workgroup barrier in this kernel
     const int N = p.N, L = p.L, P = p.n_pass;
-    float *h_in = bwd_smem + (size_t)wave * (P + 2) * N;
     float *g_carry = h_in + (size_t)P * N, *a_next = g_carry + N;
-
-    const int b = row / p.dim, d = row - b * p.dim;
     const int grp = d / p.dim_per_group, dg = d / p.dim_per_delta;
     const in_t *u_row = reinterpret_cast<const in_t *>(p.u) + b * p.u_bs + d * p.u_ds;
     const in_t *dl_row = reinterpret_cast<const in_t *>(p.delta) + b * p.dl_bs + dg * p.dl_ds;
@@ -165,8 +161,13 @@ __global__ __launch_bounds__(kBlock) void scan_bwd_kernel(const ScanBwdArgs p) {
                 dA_acc = fmaf(da_a, dl[i], dA_acc);
                 du[i] = fmaf(g, dl[i] * Bv[i], du[i]);
                 if (pos + i < L) {
-                    unsafeAtomicAdd(dB_row + n * p.g_ns + pos + i, g * dl[i] * uv[i]);
-                    unsafeAtomicAdd(dC_row + n * p.g_ns + pos + i, dy[i] * h[i]);
+                    if constexpr (kGroupAcc) {
+                        __hip_atomic_fetch_add(accB + n * L + pos + i, g * dl[i] * uv[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        __hip_atomic_fetch_add(accC + n * L + pos + i, dy[i] * h[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    } else {
+                        unsafeAtomicAdd(dB_row + n * p.g_ns + pos + i, g * dl[i] * uv[i]);
+                        unsafeAtomicAdd(dC_row + n * p.g_ns + pos + i, dy[i] * h[i]);
+                    }
                 }
             }
 #pragma unroll
@@ -198,6 +199,44 @@ __global__ __launch_bounds__(kBlock) void scan_bwd_kernel(const ScanBwdArgs p) {
     if (lane == 0) {
         if (p.dD) unsafeAtomicAdd(p.dD + d, dD_acc);
         if (p.dbias) unsafeAtomicAdd(p.dbias + d, dbias_acc);
+    }
+}
+
+// One wavefront per row, 4 rows per workgroup; dB / dC straight to memory with atomics (any N, any L).
+template <typename in_t, typename dy_t, bool kSoftplus>
+__global__ __launch_bounds__(kBlock) void scan_bwd_kernel(const ScanBwdArgs p) {
+    extern __shared__ __align__(16) float bwd_smem[];      // per wavefront: h_in [n_pass][N], g carry [N], a_next [N]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int row = (int)(blockIdx.x * kWavesPerWg) + wave;
+    if (row >= p.rows) return;           // whole wavefront leaves; no workgroup barrier in this kernel
+    scan_bwd_row<in_t, dy_t, kSoftplus, false>(p, row / p.dim, row % p.dim, bwd_smem + (size_t)wave * (p.n_pass + 2) * p.N,
+                                               nullptr, nullptr);
+}
+
+// A workgroup walks `chunk` channels of ONE (batch, group): their dB / dC contributions -- the same N x L entries
+// for every channel -- are summed in LDS and reach memory once per workgroup (one atomic per entry per `chunk`
+// channels instead of one per channel).  Used when the N x L accumulators fit LDS.
+template <typename in_t, typename dy_t, bool kSoftplus>
+__global__ __launch_bounds__(kBlock) void scan_bwd_group_kernel(const ScanBwdArgs p, int chunk, int chunks_per_group, int n_groups) {
+    extern __shared__ __align__(16) float bwd_smem[];      // accB [N][L], accC [N][L], then the per-wavefront scratch
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int NL = p.N * p.L;
+    float *accB = bwd_smem, *accC = bwd_smem + NL;
+    float *scratch = accC + NL + (size_t)wave * (p.n_pass + 2) * p.N;
+    uint32_t wg = blockIdx.x;
+    const int ck = (int)(wg % chunks_per_group); wg /= chunks_per_group;
+    const int grp = (int)(wg % n_groups);
+    const int b = (int)(wg / n_groups);
+    for (int i = threadIdx.x; i < 2 * NL; i += kBlock) bwd_smem[i] = 0.0f;
+    __syncthreads();
+    const int d_end = min((ck + 1) * chunk, p.dim_per_group);
+    for (int c = ck * chunk + wave; c < d_end; c += kWavesPerWg)
+        scan_bwd_row<in_t, dy_t, kSoftplus, true>(p, b, grp * p.dim_per_group + c, scratch, accB, accC);
+    __syncthreads();
+    float *dB_row = p.dB + b * p.g_bs + grp * p.g_gs, *dC_row = p.dC + b * p.g_bs + grp * p.g_gs;
+    for (int i = threadIdx.x; i < NL; i += kBlock) {
+        unsafeAtomicAdd(dB_row + i, accB[i]);
+        unsafeAtomicAdd(dC_row + i, accC[i]);
     }
 }
 
@@ -248,8 +287,30 @@ extern "C" int ss2d_selective_scan_bwd(const ss2d_scan_bwd_params *q, void *stre
     vec = vec && a.do_bs % dy_vec == 0 && a.do_ds % dy_vec == 0;
     a.vec_ok = vec ? 1 : 0;
 
-    const uint32_t n_wg = (uint32_t)((a.rows + kWavesPerWg - 1) / kWavesPerWg);
     hipStream_t s = (hipStream_t)stream;
+    // group kernel: N x L accumulators for dB and dC in LDS
+    const size_t acc_bytes = 2 * (size_t)a.N * a.L * sizeof(float);
+    if (acc_bytes + smem <= 56 * 1024 && a.dim_per_group >= 2 * kWavesPerWg) {
+        int chunk = a.dim_per_group < 24 ? a.dim_per_group : 24;            // channels per workgroup
+        const int cpg = (a.dim_per_group + chunk - 1) / chunk;
+        chunk = (a.dim_per_group + cpg - 1) / cpg;                           // even split
+        const int64_t n = (int64_t)q->batch * q->n_groups * cpg;
+        if (n <= 0x7fffffff) {
+            const uint32_t n_wg_g = (uint32_t)n;
+            const size_t smem_g = acc_bytes + smem;
+#define SS2D_BWD_GROUP(IN, DY)                                                                                                  \
+    do {                                                                                                                        \
+        if (a.softplus) hipLaunchKernelGGL((scan_bwd_group_kernel<IN, DY, true>), dim3(n_wg_g), dim3(kBlock), smem_g, s, a, chunk, cpg, q->n_groups); \
+        else hipLaunchKernelGGL((scan_bwd_group_kernel<IN, DY, false>), dim3(n_wg_g), dim3(kBlock), smem_g, s, a, chunk, cpg, q->n_groups);          \
+    } while (0)
+            if (q->in_dtype == SS2D_F32) SS2D_BWD_GROUP(float, float);
+            else if (q->in_dtype == SS2D_BF16) { if (q->dout_dtype == SS2D_F32) SS2D_BWD_GROUP(bf16_t, float); else SS2D_BWD_GROUP(bf16_t, bf16_t); }
+            else { if (q->dout_dtype == SS2D_F32) SS2D_BWD_GROUP(f16_t, float); else SS2D_BWD_GROUP(f16_t, f16_t); }
+#undef SS2D_BWD_GROUP
+            return launch_status();
+        }
+    }
+    const uint32_t n_wg = (uint32_t)((a.rows + kWavesPerWg - 1) / kWavesPerWg);
 #define SS2D_BWD_LAUNCH(IN, DY)                                                                                         \
     do {                                                                                                                \
         if (a.softplus) hipLaunchKernelGGL((scan_bwd_kernel<IN, DY, true>), dim3(n_wg), dim3(kBlock), smem, s, a);      \
