@@ -243,6 +243,14 @@ int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H, int W, in
                           int y_channel_last, int one_by_one, int scans, int order, void *stream);
 
 /*
+ * Batched transpose (B, R, S) -> (B, S, R), any 1/2/4/8-byte element: the layout change between channel-first
+ * (B, C, L) and channel-last (B, L, C) activations -- the permute(...).contiguous() of cross_scan_fwd / cross_merge_fwd
+ * for mixed layouts (classification/models/csm_triton.py:48-51, 80-83).  The host serves the mixed-layout modes as
+ * this transpose of the small x-side tensor plus the same-layout kernel.
+ */
+int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, int elem_bytes, void *stream);
+
+/*
  * dt_proj of the SS2D core: the per-direction rank-R -> D projection between x_proj and the scan.
  * Replaces the grouped conv1d / einsum of SS2Dv2.forward_corev2 (classification/models/vmamba.py:608-609, 614-615):
  *   delta[k, d, n] = sum_r weight[k, d, r] * x[k*x_dir_stride + r*x_rank_stride + n]

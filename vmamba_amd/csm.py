@@ -44,11 +44,32 @@ def _flex_dims(t, channel_first, one_by_one, what):
     return t.shape[0], t.shape[-1], t.shape[1], t.shape[2]
 
 
+def transpose_bcl_hip(x):
+    """(B, R, S) -> (B, S, R) contiguous (ss2d_transpose_bcl)."""
+    x = x.contiguous()
+    B, R, S = x.shape
+    y = x.new_empty((B, S, R))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_transpose_bcl(x.data_ptr(), y.data_ptr(), B, R, S, x.element_size(), _stream(x))
+    _lib.check(rc, "ss2d_transpose_bcl")
+    return y
+
+
 def cross_scan_flex_hip(x, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0):
-    """Any layout / mode of CrossScan (ss2d_cross_scan_flex); bit-exact for any 1/2/4/8-byte dtype."""
+    """Any layout / mode of CrossScan; bit-exact for any 1/2/4/8-byte dtype.  Mixed layouts first bring x (the small
+    side) to the layout of y with one tiled transpose, then run the same-layout kernel."""
     _require_gpu(x, "cross_scan")
     B, C, H, W = _flex_dims(x, in_channel_first, one_by_one, "cross_scan")
     x = x.contiguous()
+    if in_channel_first != out_channel_first and x.numel():
+        K = 4 if one_by_one else 1
+        if in_channel_first:      # (B, K*C, L) -> (B, L, K*C)
+            x = transpose_bcl_hip(x.view(B, K * C, H * W)).view((B, H, W, 4, C) if one_by_one else (B, H, W, C))
+        else:                     # (B, L, K*C) -> (B, K*C, L)
+            x = transpose_bcl_hip(x.view(B, H * W, K * C)).view((B, 4, C, H, W) if one_by_one else (B, C, H, W))
+        in_channel_first = out_channel_first
+        if in_channel_first and scans == 0:
+            return cross_scan_1b1_hip(x) if one_by_one else cross_scan_hip(x)
     y = x.new_empty((B, 4, C, H * W) if out_channel_first else (B, H * W, 4, C))
     with torch.cuda.device(x.device):
         rc = _lib.lib().ss2d_cross_scan_flex(x.data_ptr(), y.data_ptr(), B, C, H, W, x.element_size(),
@@ -68,6 +89,15 @@ def cross_merge_flex_hip(y, in_channel_first=True, out_channel_first=True, one_b
         raise TypeError(f"cross_merge: unsupported dtype {y.dtype}")
     y = y.contiguous()
     L = H * W
+    if in_channel_first != out_channel_first and y.numel():
+        # mixed layouts: merge in the layout of y, then bring the (small) result to the other layout
+        x = cross_merge_flex_hip(y, out_channel_first, out_channel_first, one_by_one, scans, order)
+        K = 4 if one_by_one else 1
+        if out_channel_first:     # (B, K*C, L) -> (B, L, K*C)
+            return transpose_bcl_hip(x.view(B, K * C, L)).view((B, L, 4, C) if one_by_one else (B, L, C))
+        return transpose_bcl_hip(x.view(B, L, K * C)).view((B, 4, C, L) if one_by_one else (B, C, L))
+    if in_channel_first and out_channel_first and (not one_by_one) and scans == 0:
+        return cross_merge_hip(y, order)
     if one_by_one:
         x = y.new_empty((B, 4, C, L) if in_channel_first else (B, L, 4, C))
     else:

@@ -251,3 +251,57 @@ extern "C" int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H
 #undef SS2D_FLEX_MERGE
     return launch_status();
 }
+
+// ---- layout change (B, C, L) <-> (B, L, C) --------------------------------------------------------------------
+// The mixed-layout modes are served by the host as "bring the small x-side tensor to the other layout, then run the
+// same-layout kernel": this is that layout change, a batched matrix transpose through a 64 x 64 LDS tile (reads
+// and writes both run along the innermost axis of their side).
+namespace ss2d {
+
+template <typename U>
+__global__ __launch_bounds__(kBlock) void transpose_bcl_kernel(const U *__restrict__ src, U *__restrict__ dst, int R, int S,
+                                                               int r_tiles, int s_tiles) {
+    // src (B, R, S) -> dst (B, S, R)
+    constexpr int kT = 64;
+    __shared__ U tile[kT][kT + 1];
+    uint32_t wg = blockIdx.x;
+    const uint32_t st = wg % s_tiles; wg /= s_tiles;
+    const uint32_t rt = wg % r_tiles;
+    const uint32_t b = wg / r_tiles;
+    const int r0 = (int)rt * kT, s0 = (int)st * kT;
+    const int lx = threadIdx.x % kT, ly = threadIdx.x / kT;            // 64 x 4
+    const U *sb = src + (size_t)b * R * S;
+    U *db = dst + (size_t)b * R * S;
+#pragma unroll 4
+    for (int i = ly; i < kT; i += kBlock / kT) {
+        const int r = r0 + i, s = s0 + lx;
+        if (r < R && s < S) tile[i][lx] = sb[(size_t)r * S + s];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = ly; i < kT; i += kBlock / kT) {
+        const int s = s0 + i, r = r0 + lx;
+        if (r < R && s < S) db[(size_t)s * R + r] = tile[lx][i];
+    }
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, int elem_bytes, void *stream) {
+    using namespace ss2d;
+    if (B < 0 || R < 0 || S < 0) return SS2D_EINVAL;
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return SS2D_EINVAL;
+    if (B == 0 || R == 0 || S == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    const int r_tiles = (R + 63) / 64, s_tiles = (S + 63) / 64;
+    const int64_t n_wg = (int64_t)B * r_tiles * s_tiles;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    hipStream_t s = (hipStream_t)stream;
+    switch (elem_bytes) {
+        case 1: hipLaunchKernelGGL((transpose_bcl_kernel<uint8_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint8_t *)x, (uint8_t *)y, R, S, r_tiles, s_tiles); break;
+        case 2: hipLaunchKernelGGL((transpose_bcl_kernel<uint16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint16_t *)x, (uint16_t *)y, R, S, r_tiles, s_tiles); break;
+        case 4: hipLaunchKernelGGL((transpose_bcl_kernel<uint32_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint32_t *)x, (uint32_t *)y, R, S, r_tiles, s_tiles); break;
+        default: hipLaunchKernelGGL((transpose_bcl_kernel<uint64_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint64_t *)x, (uint64_t *)y, R, S, r_tiles, s_tiles); break;
+    }
+    return launch_status();
+}
