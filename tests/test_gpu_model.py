@@ -61,7 +61,7 @@ def test_forward_core_fp32(d_model, d_state, ratio, H, W):
 
 
 def test_forward_core_bf16_activations():
-    """BASELINE config 1 recipe at reduced batch: bf16 activations and weights, fp32 scan state.  The GEMMs run
+    """benchmark config 1 recipe at reduced batch: bf16 activations and weights, fp32 scan state.  The GEMMs run
     in bf16 on both sides but with different accumulation orders, so the bound is the bf16 one (2e-2)."""
     print("CASE core-bf16", flush=True)
     ref, hip = _pair(96, 1)

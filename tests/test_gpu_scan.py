@@ -28,7 +28,7 @@ def make_inputs(seed, batch, dim, G, N, L, dtype, delta_dim=None, ss2d_like=Fals
     g = torch.Generator().manual_seed(seed)
     delta_dim = dim if delta_dim is None else delta_dim
     if ss2d_like:
-        # BASELINE config 0 recipe: dt log-uniform in [1e-3, 0.1], bias = inverse softplus, A = -(1..N)
+        # benchmark config 0 recipe: dt log-uniform in [1e-3, 0.1], bias = inverse softplus, A = -(1..N)
         dt = torch.exp(torch.rand(delta_dim, generator=g) * (torch.log(torch.tensor(0.1)) - torch.log(torch.tensor(1e-3)))
                        + torch.log(torch.tensor(1e-3)))
         bias = dt + torch.log(-torch.expm1(-dt))
@@ -202,7 +202,7 @@ def test_scan_errors_from_host_api():
 
 @pytest.mark.parametrize("cfg", ["stage1", "stage3", "stage4", "n16"])
 def test_full_size_properties(cfg):
-    """BASELINE configs at full size: exact scaling linearity in u, exact skip path with B=0, and a
+    """the benchmark configurations at full size: exact scaling linearity in u, exact skip path with B=0, and a
     slice of rows against the oracle."""
     _announce("scan-full", cfg)
     batch, Dn, L, N = dict(stage1=(128, 96, 3136, 1), stage3=(128, 384, 196, 1), stage4=(128, 768, 49, 1),
