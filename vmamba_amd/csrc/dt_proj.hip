@@ -40,13 +40,6 @@ __device__ __forceinline__ floatx16_t mfma_32x32x8(f16_t, const uint32_t (&a)[2]
     return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(half4_t, aw), __builtin_bit_cast(half4_t, bw), c, 0, 0, 0);
 }
 
-// LDS traffic of one wavefront is ordered by program order; this keeps the compiler from moving it around.
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 struct DtArgs {
     const void *x, *W;
     void *out;

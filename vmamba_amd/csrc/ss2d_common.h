@@ -86,6 +86,14 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
     return bits_to_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_to_bits(v), lane));
 }
 
+// LDS traffic of one wavefront is ordered by program order; this keeps the compiler from moving it around when
+// lanes exchange data through a wavefront-private LDS region (no workgroup barrier needed).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? SS2D_OK : SS2D_ELAUNCH; }
 
 }  // namespace ss2d

@@ -440,6 +440,41 @@ __global__ __launch_bounds__(kBlock) void cross_scan_1b1_kernel(const T *__restr
     }
 }
 
+// Short maps (L <= 1024): one WAVEFRONT per map, four maps per workgroup, each with a private LDS tile -- a whole
+// workgroup per 49- or 196-element map leaves most of its lanes idle and the launch is then bound by workgroup count.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cross_scan_1b1_wave_kernel(const T *__restrict__ x, T *__restrict__ y, int H, int W,
+                                                                     int Wp, int64_t n_maps, int64_t y_bs, int64_t y_ks,
+                                                                     int64_t y_cs, FastDiv divC, FastDiv divW, FastDiv divH) {
+    extern __shared__ __align__(16) unsigned char map_smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int64_t map = (int64_t)blockIdx.x * (kBlock / kWave) + wave;
+    if (map >= n_maps) return;                 // whole wavefront leaves; no workgroup barrier in this kernel
+    T *tile = reinterpret_cast<T *>(map_smem) + (size_t)wave * H * Wp;
+    uint32_t bk, c;
+    divmod((uint32_t)map, divC, bk, c);
+    const uint32_t b = bk / 4, k = bk % 4;
+    const int L = H * W;
+    const T *src = x + (size_t)map * L;
+    T *dst = y + (int64_t)b * y_bs + (int64_t)k * y_ks + (int64_t)c * y_cs;
+    if ((k & 1u) == 0) {
+        for (int j = lane; j < L; j += kWave) dst[j] = src[k == 0 ? j : L - 1 - j];
+        return;
+    }
+    for (int r = lane; r < L; r += kWave) {
+        uint32_t h, w;
+        divmod((uint32_t)r, divW, h, w);
+        tile[h * Wp + w] = src[r];
+    }
+    wave_lds_sync();
+    for (int j = lane; j < L; j += kWave) {
+        uint32_t w, h;
+        divmod((uint32_t)(k == 1 ? j : L - 1 - j), divH, w, h);
+        dst[j] = tile[h * Wp + w];
+    }
+}
+
 template <typename T>
 static int launch_cross_scan_1b1(const void *x, void *y, int B, int C, int H, int W, int64_t y_bs, int64_t y_ks, int64_t y_cs,
                                  hipStream_t stream) {
@@ -447,6 +482,13 @@ static int launch_cross_scan_1b1(const void *x, void *y, int B, int C, int H, in
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     const int Wp = W | 1;
     size_t smem = (size_t)H * Wp * sizeof(T);
+    if ((int64_t)H * W <= 1024 && smem * (kBlock / kWave) <= 48 * 1024) {
+        const int64_t n = (n_wg + kBlock / kWave - 1) / (kBlock / kWave);
+        hipLaunchKernelGGL((cross_scan_1b1_wave_kernel<T>), dim3((uint32_t)n), dim3(kBlock), smem * (kBlock / kWave), stream, (const T *)x,
+                           (T *)y, H, W, Wp, n_wg, y_bs, y_ks, y_cs, make_fastdiv((uint32_t)C), make_fastdiv((uint32_t)W),
+                           make_fastdiv((uint32_t)H));
+        return launch_status();
+    }
     const int use_lds = smem <= 48 * 1024;
     if (!use_lds) smem = 0;
     hipLaunchKernelGGL((cross_scan_1b1_kernel<T>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x, (T *)y, H, W, Wp,
