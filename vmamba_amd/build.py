@@ -25,14 +25,26 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-def build_hip(verbose=True):
-    cmd = [
-        os.path.join(ROCM, "bin", "hipcc"), "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
-        # keep the compiler from forming packed-fp32 VALU ops
-        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wall", "-Wno-unused-function",
-    ] + [os.path.join(CSRC, s) for s in HIP_SOURCES] + ["-o", LIB]
-    _run(cmd)
+def build_hip(verbose=True, jobs=None):
+    """Every .hip source to an object (in parallel), then one shared library."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    flags = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
+             # keep the compiler from forming packed-fp32 VALU ops
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wall", "-Wno-unused-function"]
+    objdir = os.path.join(CSRC, "_build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.splitext(src)[0] + ".o") for src in HIP_SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        _run([hipcc] + flags + ["-c", os.path.join(CSRC, src), "-o", obj])
+
+    jobs = jobs or min(len(HIP_SOURCES), max(1, min(os.cpu_count() or 1, 16)))
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(compile_one, zip(HIP_SOURCES, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB])
     return LIB
 
 

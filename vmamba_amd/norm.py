@@ -67,8 +67,14 @@ def needs_grad(*tensors):
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
+def _gpu_only(x, what):
+    if not x.is_cuda:
+        raise NotImplementedError(f"{what}: vmamba_amd runs on the GPU only (got a {x.device.type} tensor)")
+
+
 class LayerNorm(nn.LayerNorm):
     def forward(self, x):
+        _gpu_only(x, "LayerNorm")
         if needs_grad(x, self.weight, self.bias):
             return F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps)
         return layer_norm_hip(x, self.weight, self.bias, self.eps)
@@ -76,6 +82,7 @@ class LayerNorm(nn.LayerNorm):
 
 class LayerNorm2d(nn.LayerNorm):
     def forward(self, x):
+        _gpu_only(x, "LayerNorm2d")
         if needs_grad(x, self.weight, self.bias):          # vmamba.py:52-57
             return F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight, self.bias, self.eps).permute(0, 3, 1, 2)
         return layer_norm_cf_hip(x, self.weight, self.bias, self.eps, out_channel_last=False)
