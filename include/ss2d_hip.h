@@ -261,6 +261,19 @@ int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, int elem_byt
 int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, int R, int64_t N, int64_t x_dir_stride,
                  int64_t x_rank_stride, int dtype, void *stream);
 
+/*
+ * Fused channel-last MLP of a VSS block: out = residual + fc2(GELU(fc1(x))) in one kernel, the hidden activations
+ * never leaving the registers.  Replaces Mlp.forward (classification/models/vmamba.py:1116-1131: fc1, GELU (erf form),
+ * fc2) and the residual add of VSSBlock (:1229) for the narrow stages.
+ *   x, residual (may be NULL), out: (M, C) contiguous;  w1 (4C, C), b1 (4C) or NULL;  w2 (C, 4C), b2 (C) or NULL;
+ *   all SS2D_BF16 or all SS2D_F16, 16-byte aligned.  fc1 output, GELU output, fc2 output and the sum are each
+ *   rounded to the tensor type, as the unfused operators would.
+ * C must be 96 or 192 (wider layers are compute-bound and stay library GEMMs): anything else, and SS2D_F32,
+ * returns SS2D_ENOTSUP.
+ */
+int ss2d_mlp_fused(const void *x, const void *w1, const void *b1, const void *w2, const void *b2, const void *residual,
+                   void *out, int64_t M, int C, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

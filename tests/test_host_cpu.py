@@ -85,3 +85,29 @@ def test_vssm_state_dict_uses_reference_key_names_and_loads_legacy_checkpoints()
     cf = VSSM(**small, channel_first=True, layers=src.layers[0].blocks[0].op.layers)
     cf.load_state_dict(src.state_dict(), strict=True)
     assert torch.equal(cf.layers[0].blocks[0].mlp.fc1.weight, src.layers[0].blocks[0].mlp.fc1.weight)
+
+
+def test_gelu_table_is_what_the_generator_writes_and_matches_erf():
+    """The fused MLP kernel's GELU table: the committed include equals a fresh render, and its entries are
+    0.5 erf(x / sqrt 2) at the bf16 grid (checked against scipy's erf, an independent implementation)."""
+    import importlib.util, os, re, struct
+    import numpy as np
+    from scipy.special import erf
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "vmamba_amd", "csrc")
+    spec = importlib.util.spec_from_file_location("gen_gelu_table", os.path.join(here, "gen_gelu_table.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    text = open(os.path.join(here, "gelu_table.inc")).read()
+    assert text == gen.render()
+    bits = np.array([int(h, 16) for h in re.findall(r"0x([0-9a-f]{8})u", text)], dtype=np.uint32)
+    assert bits.size == gen.HI_BITS - gen.LO_BITS == 2176
+    vals = bits.view(np.float32).astype(np.float64)
+    x = (np.arange(gen.LO_BITS, gen.HI_BITS, dtype=np.uint32) << 16).view(np.float32).astype(np.float64)
+    assert x[0] == 2.0 ** -14 and x[-1] < 8.0 and x[-1] > 7.9
+    want = 0.5 * erf(x / np.sqrt(2.0))
+    assert np.all(np.abs(vals - want) <= 2.0 ** -24 * np.maximum(want, 1e-30) * 1.01)      # fp32 rounding of the exact value
+    assert vals[-1] == 0.5 and np.all(np.diff(vals) >= 0)
+    # the identity the kernel uses: gelu(x) = 0.5 x + |x| E(|x|), both signs
+    for s in (1.0, -1.0):
+        g = 0.5 * s * x + x * vals
+        assert np.allclose(g, 0.5 * s * x * (1.0 + erf(s * x / np.sqrt(2.0))), rtol=0, atol=1e-6)

@@ -18,27 +18,12 @@
 
 namespace ss2d {
 
-typedef short short4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef float floatx16_t __attribute__((ext_vector_type(16)));
-
 constexpr int kDtTile = 32;          // positions (and channels) per MFMA tile
 constexpr int kDtBlock = 128;        // positions per block: four tiles
 constexpr int kDtPitch = kDtBlock + 8;   // LDS row pitch in elements (272 bytes: 16-byte aligned, banks spread)
 constexpr int kDtGroups = 3;         // channel groups of 32 per wavefront
 constexpr int kDtMaxRank = 48;
 constexpr uint32_t kDtOutOfRange = 0x7ffffff0u;   // byte offset beyond any buffer here (spans are checked < 2^31 - 16)
-
-__device__ __forceinline__ floatx16_t mfma_32x32x8(bf16_t, const uint32_t (&a)[2], const uint32_t (&b)[2], floatx16_t c) {
-    const short4_t av = {(short)(a[0] & 0xffffu), (short)(a[0] >> 16), (short)(a[1] & 0xffffu), (short)(a[1] >> 16)};
-    const short4_t bv = {(short)(b[0] & 0xffffu), (short)(b[0] >> 16), (short)(b[1] & 0xffffu), (short)(b[1] >> 16)};
-    return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(av, bv, c, 0, 0, 0);
-}
-__device__ __forceinline__ floatx16_t mfma_32x32x8(f16_t, const uint32_t (&a)[2], const uint32_t (&b)[2], floatx16_t c) {
-    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-    const u32x2 aw = {a[0], a[1]}, bw = {b[0], b[1]};
-    return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(half4_t, aw), __builtin_bit_cast(half4_t, bw), c, 0, 0, 0);
-}
 
 struct DtArgs {
     const void *x, *W;

@@ -1,0 +1,287 @@
+// Fused channel-last MLP of a VSS block (classification/models/vmamba.py:1116-1131 Mlp, :1229 the residual add):
+//     out = residual + fc2(GELU(fc1(x)))          x (M, C), fc1 (4C x C) + bias, fc2 (C x 4C) + bias, 16-bit tensors
+// in ONE kernel for the narrow stages (C = 96, 192), where the two library GEMMs, the GELU pass and the add are all
+// bound by the (M, 4C) hidden tensor going to HBM and back three times.  Here the hidden activations never leave the
+// registers:
+//   * a wavefront owns 32 (C = 192) or 64 (C = 96) positions and walks the hidden units in chunks of 32;
+//   * GEMM 1 computes the chunk transposed, D1[hidden][position] = W1 chunk * x^T (v_mfma_f32_32x32x16, fp32
+//     accumulate).  In the MFMA output layout a lane holds, for its position, hidden units 8g + 4*(lane/32) + t
+//     (g, t = 0..3), accumulator 4g + t.  GEMM 2, D2[channel][position] += W2 chunk * h, contracts 16 hidden units per
+//     instruction and a lane supplies 8 of them; the order of the contraction index is free as long as both operands
+//     agree, so k-slot e of lane half kh in step s is DEFINED as hidden unit 16s + 8(e/4) + 4kh + e%4 -- which makes
+//     accumulators 8s .. 8s+7 (after bias, GELU and rounding to 16 bits) the B fragment of step s with no data
+//     movement between the two GEMMs.  The W2 chunk is written to LDS with its columns in that order;
+//   * the W1 / W2 chunks (2 x 6..12 KB) are staged through LDS by the whole workgroup, double-buffered, one barrier
+//     per chunk; x tiles come in and results go out through a wavefront-private LDS tile so that global loads and
+//     stores are 16 bytes per lane along the channel axis; the residual is added on the way out.
+// Rounding follows the unfused reference: fc1 output, GELU output and fc2 output are each rounded to the 16-bit type,
+// then the residual add is rounded once more.  GELU is the exact (erf) form:
+//   * bf16: the pre-activation is a bf16 value, so gelu(x) = 0.5 x + |x| E(|x|), E(x) = 0.5 erf(x / sqrt 2), with E read
+//     from a 2176-entry fp32 table in LDS indexed by the bf16 bit pattern clamped to [2^-14, 8) (below, |x| E is under
+//     1e-4 of 0.5 |x|; above, E is 0.5 to fp32 precision).  The table is generated in double precision at build time;
+//   * fp16: erf from Abramowitz-Stegun 7.1.26 (absolute error 1.5e-7, far below 16-bit rounding).
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+#include "gelu_table.inc"
+
+constexpr int kMlpChunk = 32;      // hidden units per chunk = one MFMA tile
+constexpr int kGeluEntries = kGeluHiBits - kGeluLoBits;
+
+__device__ __forceinline__ float gelu_erf(float x) {
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float poly = fmaf(1.061405429f, t, -1.453152027f);
+    poly = fmaf(poly, t, 1.421413741f);
+    poly = fmaf(poly, t, -0.284496736f);
+    poly = fmaf(poly, t, 0.254829592f);
+    const float e = __builtin_amdgcn_exp2f(z * z * -1.4426950408889634f);
+    const float erf_abs = fmaf(-poly * t, e, 1.0f);                   // erf(|x| / sqrt 2)
+    const float erf_x = __builtin_copysignf(erf_abs, x);
+    return 0.5f * x * (1.0f + erf_x);
+}
+
+// GELU of two packed 16-bit values, result packed and rounded again
+__device__ __forceinline__ uint32_t gelu_pair(bf16_t, uint32_t w, const float *tbl) {
+    const uint32_t a0 = w & 0x7fffu, a1 = (w >> 16) & 0x7fffu;
+    const uint32_t m0 = min(max(a0, (uint32_t)kGeluLoBits), (uint32_t)kGeluHiBits - 1u) - kGeluLoBits;
+    const uint32_t m1 = min(max(a1, (uint32_t)kGeluLoBits), (uint32_t)kGeluHiBits - 1u) - kGeluLoBits;
+    const float e0 = tbl[m0], e1 = tbl[m1];
+    const float x0 = bits_to_f32(w << 16), x1 = bits_to_f32(w & 0xffff0000u);
+    return pack2_from_f32<bf16_t>(fmaf(fabsf(x0), e0, 0.5f * x0), fmaf(fabsf(x1), e1, 0.5f * x1));
+}
+__device__ __forceinline__ uint32_t gelu_pair(f16_t, uint32_t w, const float *) {
+    return pack2_from_f32<f16_t>(gelu_erf(unpack_lo<f16_t>(w)), gelu_erf(unpack_hi<f16_t>(w)));
+}
+
+struct MlpArgs {
+    const void *x, *w1, *b1, *w2, *b2, *residual;
+    void *out;
+    int64_t M;
+};
+
+template <typename T, int C> struct MlpLayout {
+    static constexpr bool kTable = ElemTraits<T>::dtype == SS2D_BF16;
+    static constexpr int P1 = C + 8, P2 = kMlpChunk + 8, PS = C + 8;   // LDS row pitches (elements): rows stay 16-byte
+                                                                       // aligned and 16 rows x 16 bytes cover all banks
+    static constexpr int kW1Elems = kMlpChunk * P1, kW2Elems = C * P2, kBufElems = kW1Elems + kW2Elems;
+    static constexpr int kStageElems = kMlpChunk * PS;                 // one 32-position tile per wavefront
+    static constexpr size_t kBytes = (size_t)(2 * kBufElems + 5 * C) * sizeof(uint16_t) + (kTable ? kGeluEntries * sizeof(float) : 0);
+};
+
+template <typename T, int C, int kCT>
+__global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
+    using Lay = MlpLayout<T, C>;
+    constexpr int kHidden = 4 * C;
+    constexpr int kChunks = kHidden / kMlpChunk;
+    constexpr int kSteps1 = C / 16;                 // k-steps of GEMM 1
+    constexpr int kOG = C / 32;                     // output-channel groups of GEMM 2
+    constexpr int P1 = Lay::P1, P2 = Lay::P2, PS = Lay::PS;
+    constexpr int kW1Elems = Lay::kW1Elems, kBufElems = Lay::kBufElems, kStageElems = Lay::kStageElems;
+    constexpr int kWaves = kBlock / kWave;
+    static_assert(2 * kBufElems >= kWaves * kStageElems, "the staging tiles alias the weight buffers");
+    static_assert((2 * kBufElems + 5 * C) % 8 == 0, "the table starts 16-byte aligned");
+    extern __shared__ __align__(16) uint16_t mlp_smem[];
+    uint16_t *wbuf = mlp_smem;                                      // [2][W1 chunk | W2 chunk]
+    uint16_t *bias1 = mlp_smem + 2 * kBufElems;                     // [4C]
+    uint16_t *bias2 = bias1 + kHidden;                              // [C]
+    float *tbl = reinterpret_cast<float *>(bias2 + C);              // [kGeluEntries], bf16 only
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int j = lane & 31, kh = lane >> 5;
+    uint16_t *stage = mlp_smem + wave * kStageElems;                // aliases wbuf: used before and after the chunk loop
+    const T *x = reinterpret_cast<const T *>(p.x);
+    const T *w1 = reinterpret_cast<const T *>(p.w1), *w2 = reinterpret_cast<const T *>(p.w2);
+    const int64_t pos0 = ((int64_t)blockIdx.x * kWaves + wave) * (kCT * 32);   // first position of this wavefront
+
+    // ---- weight chunks: global -> registers -> LDS, one chunk ahead ---------------------------------------------------
+    constexpr int kN1 = kMlpChunk * C / 8, kN2 = C * kMlpChunk / 8;   // 16-byte pieces per chunk of W1, W2
+    constexpr int kL1 = (kN1 + kBlock - 1) / kBlock, kL2 = (kN2 + kBlock - 1) / kBlock;
+    uint4 r1[kL1], r2[kL2];
+    auto fetch = [&](int chunk) {
+#pragma unroll
+        for (int it = 0; it < kL1; ++it) {
+            const int idx = min((int)threadIdx.x + it * kBlock, kN1 - 1);
+            const int i = idx / (C / 8), q = idx % (C / 8);
+            r1[it] = *reinterpret_cast<const uint4 *>(w1 + (size_t)(chunk * kMlpChunk + i) * C + 8 * q);
+        }
+#pragma unroll
+        for (int it = 0; it < kL2; ++it) {
+            const int idx = min((int)threadIdx.x + it * kBlock, kN2 - 1);
+            const int o = idx / (kMlpChunk / 8), q = idx % (kMlpChunk / 8);
+            r2[it] = *reinterpret_cast<const uint4 *>(w2 + (size_t)o * kHidden + chunk * kMlpChunk + 8 * q);
+        }
+    };
+    auto park = [&](int buf) {
+        uint16_t *b1w = wbuf + buf * kBufElems, *b2w = b1w + kW1Elems;
+#pragma unroll
+        for (int it = 0; it < kL1; ++it) {
+            const int idx = (int)threadIdx.x + it * kBlock;
+            if (idx < kN1) {
+                const int i = idx / (C / 8), q = idx % (C / 8);
+                *reinterpret_cast<uint4 *>(b1w + i * P1 + 8 * q) = r1[it];
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < kL2; ++it) {
+            const int idx = (int)threadIdx.x + it * kBlock;
+            if (idx < kN2) {
+                // hidden units 8q .. 8q+7 of row o: the first four are k-slots of lane half 0, the last four of half 1
+                const int o = idx / (kMlpChunk / 8), q = idx % (kMlpChunk / 8);
+                uint16_t *d = b2w + o * P2 + 16 * (q >> 1) + 4 * (q & 1);
+                *reinterpret_cast<uint2 *>(d) = make_uint2(r2[it].x, r2[it].y);
+                *reinterpret_cast<uint2 *>(d + 8) = make_uint2(r2[it].z, r2[it].w);
+            }
+        }
+    };
+    fetch(0);
+
+    // ---- biases and the GELU table to LDS; x tiles -> fragments -------------------------------------------------------
+    for (int i = threadIdx.x; i < kHidden; i += kBlock) bias1[i] = p.b1 ? reinterpret_cast<const uint16_t *>(p.b1)[i] : (uint16_t)0;
+    for (int i = threadIdx.x; i < C; i += kBlock) bias2[i] = p.b2 ? reinterpret_cast<const uint16_t *>(p.b2)[i] : (uint16_t)0;
+    if constexpr (Lay::kTable)
+        for (int i = threadIdx.x; i < kGeluEntries / 4; i += kBlock)
+            reinterpret_cast<uint4 *>(tbl)[i] = reinterpret_cast<const uint4 *>(kGeluHalfErfBits)[i];
+    u32x4_t xf[kCT][kSteps1];
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct) {
+        constexpr int kPieces = 32 * C / 8;                          // 16-byte pieces of a 32 x C tile
+#pragma unroll
+        for (int it = 0; it < kPieces / kWave; ++it) {
+            const int idx = lane + it * kWave;
+            const int r = idx / (C / 8), q = idx % (C / 8);
+            int64_t pos = pos0 + ct * 32 + r;
+            pos = pos < p.M ? pos : p.M - 1;                         // rows past the end: any valid row, never stored
+            *reinterpret_cast<uint4 *>(stage + r * PS + 8 * q) = *reinterpret_cast<const uint4 *>(x + pos * C + 8 * q);
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int s = 0; s < kSteps1; ++s) xf[ct][s] = *reinterpret_cast<const u32x4_t *>(stage + j * PS + 16 * s + 8 * kh);
+        wave_lds_sync();
+    }
+    __syncthreads();                                                 // staging aliases the weight buffers
+    park(0);
+    __syncthreads();
+
+    floatx16_t acc2[kCT][kOG];
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct)
+#pragma unroll
+        for (int og = 0; og < kOG; ++og)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc2[ct][og][v] = 0.0f;
+
+    for (int chunk = 0; chunk < kChunks; ++chunk) {
+        if (chunk + 1 < kChunks) fetch(chunk + 1);
+        const uint16_t *w1c = wbuf + (chunk & 1) * kBufElems, *w2c = w1c + kW1Elems;
+        // GEMM 1: D1[hidden][position], one 32 x 32 tile per column tile
+        floatx16_t acc1[kCT];
+#pragma unroll
+        for (int ct = 0; ct < kCT; ++ct)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc1[ct][v] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kSteps1; ++s) {
+            const u32x4_t a = *reinterpret_cast<const u32x4_t *>(w1c + j * P1 + 16 * s + 8 * kh);
+#pragma unroll
+            for (int ct = 0; ct < kCT; ++ct) acc1[ct] = mfma_32x32x16(T{}, a, xf[ct][s], acc1[ct]);
+        }
+        // bias, rounding, GELU, rounding: accumulators 8s .. 8s+7 become the B fragment of GEMM 2's step s
+        u32x4_t hf[kCT][2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint2 bb = *reinterpret_cast<const uint2 *>(bias1 + chunk * kMlpChunk + 8 * g + 4 * kh);
+            const float bv[4] = {unpack_lo<T>(bb.x), unpack_hi<T>(bb.x), unpack_lo<T>(bb.y), unpack_hi<T>(bb.y)};
+#pragma unroll
+            for (int ct = 0; ct < kCT; ++ct) {
+                // fc1 output as a GEMM stores it (rounded), then GELU
+                const uint32_t pre01 = pack2_from_f32<T>(acc1[ct][4 * g + 0] + bv[0], acc1[ct][4 * g + 1] + bv[1]);
+                const uint32_t pre23 = pack2_from_f32<T>(acc1[ct][4 * g + 2] + bv[2], acc1[ct][4 * g + 3] + bv[3]);
+                hf[ct][g >> 1][2 * (g & 1) + 0] = gelu_pair(T{}, pre01, tbl);
+                hf[ct][g >> 1][2 * (g & 1) + 1] = gelu_pair(T{}, pre23, tbl);
+            }
+        }
+        // GEMM 2: D2[channel][position] += W2[:, chunk] * h
+#pragma unroll
+        for (int og = 0; og < kOG; ++og)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(w2c + (og * 32 + j) * P2 + 16 * s + 8 * kh);
+#pragma unroll
+                for (int ct = 0; ct < kCT; ++ct) acc2[ct][og] = mfma_32x32x16(T{}, a, hf[ct][s], acc2[ct][og]);
+            }
+        if (chunk + 1 < kChunks) park((chunk + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- out = residual + (acc2 + b2), through the wavefront's staging tile ------------------------------------------
+    T *out = reinterpret_cast<T *>(p.out);
+    const T *res = reinterpret_cast<const T *>(p.residual);
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct) {
+#pragma unroll
+        for (int og = 0; og < kOG; ++og)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int c0 = og * 32 + 8 * g + 4 * kh;             // accumulators 4g .. 4g+3: channels c0 .. c0+3
+                const uint2 bb = *reinterpret_cast<const uint2 *>(bias2 + c0);
+                *reinterpret_cast<uint2 *>(stage + j * PS + c0) =
+                    make_uint2(pack2_from_f32<T>(acc2[ct][og][4 * g + 0] + unpack_lo<T>(bb.x), acc2[ct][og][4 * g + 1] + unpack_hi<T>(bb.x)),
+                               pack2_from_f32<T>(acc2[ct][og][4 * g + 2] + unpack_lo<T>(bb.y), acc2[ct][og][4 * g + 3] + unpack_hi<T>(bb.y)));
+            }
+        wave_lds_sync();
+        constexpr int kPieces = 32 * C / 8;
+#pragma unroll
+        for (int it = 0; it < kPieces / kWave; ++it) {
+            const int idx = lane + it * kWave;
+            const int r = idx / (C / 8), q = idx % (C / 8);
+            const int64_t pos = pos0 + ct * 32 + r;
+            if (pos < p.M) {
+                uint4 v = *reinterpret_cast<const uint4 *>(stage + r * PS + 8 * q);
+                if (res) {
+                    const uint4 rv = *reinterpret_cast<const uint4 *>(res + pos * C + 8 * q);
+                    uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+                    const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        vw[e] = pack2_from_f32<T>(unpack_lo<T>(vw[e]) + unpack_lo<T>(rw[e]), unpack_hi<T>(vw[e]) + unpack_hi<T>(rw[e]));
+                    v = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                }
+                *reinterpret_cast<uint4 *>(out + pos * C + 8 * q) = v;
+            }
+        }
+        wave_lds_sync();
+    }
+}
+
+template <typename T, int C, int kCT>
+static int launch_mlp(const MlpArgs &a, hipStream_t stream) {
+    const size_t smem = MlpLayout<T, C>::kBytes;
+    const int64_t per_wg = (int64_t)(kBlock / kWave) * kCT * 32;
+    const int64_t n_wg = (a.M + per_wg - 1) / per_wg;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    hipLaunchKernelGGL((mlp_fused_kernel<T, C, kCT>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    return launch_status();
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_mlp_fused(const void *x, const void *w1, const void *b1, const void *w2, const void *b2,
+                              const void *residual, void *out, int64_t M, int C, int dtype, void *stream) {
+    using namespace ss2d;
+    if (M < 0 || C <= 0) return SS2D_EINVAL;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (M == 0) return SS2D_OK;
+    if (!x || !w1 || !w2 || !out) return SS2D_EINVAL;
+    if (dtype == SS2D_F32 || (C != 96 && C != 192)) return SS2D_ENOTSUP;       // wider stages, fp32: the library GEMMs
+    const void *ptrs[] = {x, w1, b1, w2, b2, residual, out};
+    for (const void *q : ptrs)
+        if (q && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return SS2D_ENOTSUP;
+    MlpArgs a;
+    a.x = x; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.residual = residual; a.out = out; a.M = M;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == SS2D_BF16) return C == 96 ? launch_mlp<bf16_t, 96, 2>(a, s) : launch_mlp<bf16_t, 192, 1>(a, s);
+    return C == 96 ? launch_mlp<f16_t, 96, 2>(a, s) : launch_mlp<f16_t, 192, 1>(a, s);
+}

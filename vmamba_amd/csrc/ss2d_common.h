@@ -43,6 +43,24 @@ template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) {
     return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
 }
 
+// two fp32 -> one dword of packed 16-bit values (low half first), round-to-nearest-even: v_cvt_pk_bf16_f32 /
+// v_cvt_pk_f16_f32, the same results as from_f32 in one instruction per pair
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+template <typename T> __device__ __forceinline__ uint32_t pack2_from_f32(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2_from_f32<bf16_t>(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const floatx2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+template <> __device__ __forceinline__ uint32_t pack2_from_f32<f16_t>(float lo, float hi) {
+    typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
+    const floatx2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, halfx2_t));
+}
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w) { return to_f32(T{(uint16_t)(w & 0xffffu)}); }
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w) { return to_f32(T{(uint16_t)(w >> 16)}); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return bits_to_f32(w & 0xffff0000u); }
+
 // ---- division by a runtime constant -------------------------------------------
 // q = n / d for n < 2^32 using one mulhi and one correction; m = floor(2^32 / d) (d >= 2) or
 // the divisor 1 flagged by m == 0.
@@ -84,6 +102,37 @@ constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143, kDppWaveShr1 = 0x1
 
 __device__ __forceinline__ float read_lane(float v, int lane) {
     return bits_to_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_to_bits(v), lane));
+}
+
+// ---- matrix cores -------------------------------------------------------------------------------------------
+// v_mfma_f32_32x32x8 (bf16 / f16 operands, fp32 accumulate): D (32 x 32) += A (32 x 8) * B (8 x 32).  Lane l supplies
+// A[l % 32][4*(l/32) .. +3] and B[4*(l/32) .. +3][l % 32] as two dwords of packed 16-bit values, and holds
+// D[8*(v/4) + 4*(l/32) + v%4][l % 32] in accumulator v = 0..15.
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ floatx16_t mfma_32x32x8(bf16_t, const uint32_t (&a)[2], const uint32_t (&b)[2], floatx16_t c) {
+    const short4_t av = {(short)(a[0] & 0xffffu), (short)(a[0] >> 16), (short)(a[1] & 0xffffu), (short)(a[1] >> 16)};
+    const short4_t bv = {(short)(b[0] & 0xffffu), (short)(b[0] >> 16), (short)(b[1] & 0xffffu), (short)(b[1] >> 16)};
+    return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(av, bv, c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16_t mfma_32x32x8(f16_t, const uint32_t (&a)[2], const uint32_t (&b)[2], floatx16_t c) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 aw = {a[0], a[1]}, bw = {b[0], b[1]};
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(half4_t, aw), __builtin_bit_cast(half4_t, bw), c, 0, 0, 0);
+}
+
+// v_mfma_f32_32x32x16 (gfx950): D (32 x 32) += A (32 x 16) * B (16 x 32).  Lane l supplies A[l % 32][8*(l/32) .. +7] and
+// B[8*(l/32) .. +7][l % 32] as four dwords; the accumulator layout is that of 32x32x8.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ floatx16_t mfma_32x32x16(bf16_t, u32x4_t a, u32x4_t b, floatx16_t c) {
+    typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16_t mfma_32x32x16(f16_t, u32x4_t a, u32x4_t b, floatx16_t c) {
+    typedef _Float16 halfx8_t __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
 }
 
 // LDS traffic of one wavefront is ordered by program order; this keeps the compiler from moving it around when
