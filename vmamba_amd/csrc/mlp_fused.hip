@@ -10,9 +10,9 @@
 //     instruction and a lane supplies 8 of them; the order of the contraction index is free as long as both operands
 //     agree, so k-slot e of lane half kh in step s is DEFINED as hidden unit 16s + 8(e/4) + 4kh + e%4 -- which makes
 //     accumulators 8s .. 8s+7 (after bias, GELU and rounding to 16 bits) the B fragment of step s with no data
-//     movement between the two GEMMs.  The W2 chunk is written to LDS with its columns in that order;
-//   * the W1 / W2 chunks (2 x 6..12 KB) are staged through LDS by the whole workgroup, double-buffered, one barrier
-//     per chunk; x tiles come in and results go out through a wavefront-private LDS tile so that global loads and
+//     movement between the two GEMMs.  The matching W2 fragment is two 8-byte runs of a row (one ds_read2_b64);
+//   * the W1 / W2 chunks (2 x 6..12 KB) go from global memory straight into LDS (global_load_lds_dwordx4, no
+//     registers in between), double-buffered, one barrier per chunk; x tiles come in and results go out through a wavefront-private LDS tile so that global loads and
 //     stores are 16 bytes per lane along the channel axis; the residual is added on the way out.
 // Rounding follows the unfused reference: fc1 output, GELU output and fc2 output are each rounded to the 16-bit type,
 // then the residual add is rounded once more.  GELU is the exact (erf) form:
@@ -96,47 +96,39 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
     const T *w1 = reinterpret_cast<const T *>(p.w1), *w2 = reinterpret_cast<const T *>(p.w2);
     const int64_t pos0 = ((int64_t)blockIdx.x * kWaves + wave) * (kCT * 32);   // first position of this wavefront
 
-    // ---- weight chunks: global -> registers -> LDS, one chunk ahead ---------------------------------------------------
-    constexpr int kN1 = kMlpChunk * C / 8, kN2 = C * kMlpChunk / 8;   // 16-byte pieces per chunk of W1, W2
-    constexpr int kL1 = (kN1 + kBlock - 1) / kBlock, kL2 = (kN2 + kBlock - 1) / kBlock;
-    uint4 r1[kL1], r2[kL2];
-    auto fetch = [&](int chunk) {
+    // ---- weight chunks: global -> LDS directly (global_load_lds_dwordx4), one chunk ahead --------------------------------
+    // A wavefront's load instruction writes 64 consecutive 16-byte pieces of LDS (piece = lane), each lane fetching from
+    // its own global address; the buffer [W1 chunk | W2 chunk] is one run of pieces, the pad piece that ends every row
+    // is filled from a valid address and never read.
+    constexpr int kRow1 = P1 / 8, kRow2 = P2 / 8;                     // pieces per LDS row, pad included
+    constexpr int kPieces1 = kMlpChunk * kRow1, kPiecesW = kPieces1 + C * kRow2;
+    constexpr int kDmaIters = (kPiecesW + kBlock - 1) / kBlock;
+    static_assert(kPiecesW % 32 == 0 && kBufElems == 8 * kPiecesW, "whole or half wavefronts of pieces");
+    uint32_t w_off[kDmaIters];                                        // element offset of this lane's piece in chunk 0
+    bool w_second[kDmaIters];                                         // the piece belongs to W2
 #pragma unroll
-        for (int it = 0; it < kL1; ++it) {
-            const int idx = min((int)threadIdx.x + it * kBlock, kN1 - 1);
-            const int i = idx / (C / 8), q = idx % (C / 8);
-            r1[it] = *reinterpret_cast<const uint4 *>(w1 + (size_t)(chunk * kMlpChunk + i) * C + 8 * q);
+    for (int it = 0; it < kDmaIters; ++it) {
+        const int piece = (it * kWaves + wave) * kWave + lane;
+        if (piece < kPieces1) {
+            const int i = piece / kRow1, q = min(piece % kRow1, kRow1 - 2);
+            w_off[it] = (uint32_t)(i * C + 8 * q); w_second[it] = false;
+        } else {
+            const int pp = min(piece, kPiecesW - 1) - kPieces1;
+            const int o = pp / kRow2, q = min(pp % kRow2, kRow2 - 2);
+            w_off[it] = (uint32_t)(o * kHidden + 8 * q); w_second[it] = true;
         }
+    }
+    auto fetch = [&](int chunk, int buf) {
 #pragma unroll
-        for (int it = 0; it < kL2; ++it) {
-            const int idx = min((int)threadIdx.x + it * kBlock, kN2 - 1);
-            const int o = idx / (kMlpChunk / 8), q = idx % (kMlpChunk / 8);
-            r2[it] = *reinterpret_cast<const uint4 *>(w2 + (size_t)o * kHidden + chunk * kMlpChunk + 8 * q);
-        }
-    };
-    auto park = [&](int buf) {
-        uint16_t *b1w = wbuf + buf * kBufElems, *b2w = b1w + kW1Elems;
-#pragma unroll
-        for (int it = 0; it < kL1; ++it) {
-            const int idx = (int)threadIdx.x + it * kBlock;
-            if (idx < kN1) {
-                const int i = idx / (C / 8), q = idx % (C / 8);
-                *reinterpret_cast<uint4 *>(b1w + i * P1 + 8 * q) = r1[it];
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < kL2; ++it) {
-            const int idx = (int)threadIdx.x + it * kBlock;
-            if (idx < kN2) {
-                // hidden units 8q .. 8q+7 of row o: the first four are k-slots of lane half 0, the last four of half 1
-                const int o = idx / (kMlpChunk / 8), q = idx % (kMlpChunk / 8);
-                uint16_t *d = b2w + o * P2 + 16 * (q >> 1) + 4 * (q & 1);
-                *reinterpret_cast<uint2 *>(d) = make_uint2(r2[it].x, r2[it].y);
-                *reinterpret_cast<uint2 *>(d + 8) = make_uint2(r2[it].z, r2[it].w);
+        for (int it = 0; it < kDmaIters; ++it) {
+            const int first = (it * kWaves + wave) * kWave;           // wave-uniform
+            if (first + lane < kPiecesW) {
+                const T *src = w_second[it] ? w2 + w_off[it] + chunk * kMlpChunk : w1 + w_off[it] + (size_t)chunk * kMlpChunk * C;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                                 (__attribute__((address_space(3))) void *)(wbuf + buf * kBufElems + first * 8), 16, 0, 0);
             }
         }
     };
-    fetch(0);
 
     // ---- biases and the GELU table to LDS; x tiles -> fragments -------------------------------------------------------
     for (int i = threadIdx.x; i < kHidden; i += kBlock) bias1[i] = p.b1 ? reinterpret_cast<const uint16_t *>(p.b1)[i] : (uint16_t)0;
@@ -162,7 +154,7 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
         wave_lds_sync();
     }
     __syncthreads();                                                 // staging aliases the weight buffers
-    park(0);
+    fetch(0, 0);
     __syncthreads();
 
     floatx16_t acc2[kCT][kOG];
@@ -174,7 +166,7 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
             for (int v = 0; v < 16; ++v) acc2[ct][og][v] = 0.0f;
 
     for (int chunk = 0; chunk < kChunks; ++chunk) {
-        if (chunk + 1 < kChunks) fetch(chunk + 1);
+        if (chunk + 1 < kChunks) fetch(chunk + 1, (chunk + 1) & 1);
         const uint16_t *w1c = wbuf + (chunk & 1) * kBufElems, *w2c = w1c + kW1Elems;
         // GEMM 1: D1[hidden][position], one 32 x 32 tile per column tile
         floatx16_t acc1[kCT];
@@ -208,11 +200,12 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
         for (int og = 0; og < kOG; ++og)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(w2c + (og * 32 + j) * P2 + 16 * s + 8 * kh);
+                const uint16_t *row = w2c + (og * 32 + j) * P2 + 16 * s + 4 * kh;     // units 16s+4kh.., 16s+8+4kh..
+                const uint2 lo = *reinterpret_cast<const uint2 *>(row), hi = *reinterpret_cast<const uint2 *>(row + 8);
+                const u32x4_t a = {lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
                 for (int ct = 0; ct < kCT; ++ct) acc2[ct][og] = mfma_32x32x16(T{}, a, hf[ct][s], acc2[ct][og]);
             }
-        if (chunk + 1 < kChunks) park((chunk + 1) & 1);
         __syncthreads();
     }
 
