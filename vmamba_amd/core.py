@@ -15,16 +15,21 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
+def _lds_extent(n, es):
+    """Elements an LDS array of n logical elements takes: one spare 4-byte word per 32 words, rounded to 8 elements."""
+    idx = n + (n >> 5) if es == 4 else n + ((n >> 6) << 1)
+    return (idx + 8) & ~7
+
+
 def core_fits(H, W, dtype):
     """True when ss2d_core_fwd takes an H x W image of this dtype: at least 8 positions, and the LDS arrays of one
-    image (two fp32 merge planes and two copies of the x map, each with one spare word per 32) within 64 KiB."""
+    image (two fp32 merge planes, two copies of the x map plus a block of 8 zeros each) within 64 KiB."""
     if dtype not in _DTYPE_CODE:
         return False
     L = H * W
     es = 4 if dtype == torch.float32 else 2
-    plane = L + (L >> 5) + 2
-    xmap = plane if es == 4 else L + 2 * (L >> 6) + 2
-    return L >= 8 and 2 * plane * 4 + 2 * xmap * es <= 64 * 1024
+    maps = _lds_extent(((L + 7) & ~7) + 8, es)
+    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024
 
 
 def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True):

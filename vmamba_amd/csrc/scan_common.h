@@ -123,35 +123,26 @@ __device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32
 }
 
 // delta -> dl for the 8 items of a lane.
-//   kSoftplus: dl = softplus(raw + bias) = ln2 * log2(1 + 2^((raw + bias) * log2e)) with the two hardware
-//   transcendentals.  w = 1 + t loses the low bits of a small t; c = t - (w - 1) is exactly that loss (t < 1), and
-//   log(1 + t) = log(w) + c/w with c/w ~ c.  Arguments above 20 return the argument itself (the reference's
-//   threshold); that select sits behind a wave-uniform vote because it is almost never taken.
+//   kSoftplus: dl = softplus(x), x = raw + bias, as  max(x, 0) + log(1 + exp(-|x|))  with the two hardware
+//   transcendentals in base 2: z = x * log2e, t = 2^-|z| <= 1, w = 1 + t, dl = ln2 * (max(z, 0) + log2 w) + c.
+//   w = 1 + t loses the low bits of a small t; c = t - (w - 1) is exactly that loss (1 <= w <= 2), and
+//   log(1 + t) = log(w) + c/w with c/w ~ c.  For x above the reference's threshold of 20 (where it returns x itself)
+//   the log term is below 2.1e-9 = 1e-10 x, invisible in fp32, so no special case is needed.
 //   A raw value of -inf (the fill for positions past the end of a row) gives t = 0, dl = 0: the identity pair.
 //   !kSoftplus: dl = raw + bias; the caller zeroes positions past the end.
-constexpr float kSoftplusThreshold = 20.0f;
+constexpr float kSoftplusThreshold = 20.0f;     // the backward's d softplus / dx is 1 above it, as in the reference
 
 template <bool kSoftplus>
 __device__ __forceinline__ void delta_transform(const float (&raw)[kItems], const float (&bias)[kItems],
                                                 float (&dl)[kItems]) {
     if constexpr (kSoftplus) {
-        float zmax = -__builtin_inff();
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
             const float z = fmaf(raw[i], kLog2e, bias[i] * kLog2e);
-            zmax = __builtin_fmaxf(zmax, z);
-            const float t = __builtin_amdgcn_exp2f(z);
+            const float t = __builtin_amdgcn_exp2f(-__builtin_fabsf(z));
             const float w = 1.0f + t;
-            float c = t - (w - 1.0f);
-            c = t < 1.0f ? c : 0.0f;
-            dl[i] = fmaf(kLn2, __builtin_amdgcn_logf(w), c);
-        }
-        if (__builtin_amdgcn_ballot_w64(zmax > kSoftplusThreshold * kLog2e) != 0) {
-#pragma unroll
-            for (int i = 0; i < kItems; ++i) {
-                const float x = raw[i] + bias[i];
-                dl[i] = x > kSoftplusThreshold ? x : dl[i];
-            }
+            const float c = t - (w - 1.0f);
+            dl[i] = fmaf(__builtin_fmaxf(z, 0.0f), kLn2, fmaf(kLn2, __builtin_amdgcn_logf(w), c));
         }
     } else {
 #pragma unroll
@@ -160,25 +151,34 @@ __device__ __forceinline__ void delta_transform(const float (&raw)[kItems], cons
 }
 
 // Inclusive scan of (a,h) over the 64 lanes; returns this lane's EXCLUSIVE prefix in
-// (a_ex,h_ex) and the wave total, uniform, in (a_tot,h_tot).
+// (a_ex,h_ex) and the wave total, uniform, in (a_tot,h_tot).  Call with all 64 lanes active.
+// Each step combines a lane with the lane `shift` below it:  h += a * h_below;  a *= a_below.  The DPP operand does
+// the lane movement inside the arithmetic instruction, and a lane without a source (row start, masked row) is left
+// untouched by the hardware -- which is the identity (a_below = 1, h_below = 0) -- so a step is two instructions.
+// The compiler does not fold its own DPP moves into these operations, hence the assembly; the s_nop are the two wait
+// states a DPP read needs after a VALU write of the same register.
 __device__ __forceinline__ void wave_scan_pairs(float a, float h, float &a_ex, float &h_ex, float &a_tot,
                                                 float &h_tot) {
-#define SS2D_SCAN_STEP(CTRL, MASK)                        \
-    {                                                     \
-        const float ap = dpp_move<CTRL, MASK>(1.0f, a);   \
-        const float hp = dpp_move<CTRL, MASK>(0.0f, h);   \
-        h = fmaf(a, hp, h);                               \
-        a = a * ap;                                       \
-    }
-    SS2D_SCAN_STEP(kDppRowShr1, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr2, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr4, 0xF)
-    SS2D_SCAN_STEP(kDppRowShr8, 0xF)
-    SS2D_SCAN_STEP(kDppRowBcast15, 0xA)
-    SS2D_SCAN_STEP(kDppRowBcast31, 0xC)
+    float ax = 1.0f, hx = 0.0f;
+#define SS2D_SCAN_STEP(CTRL)                                   \
+    "v_fmac_f32_dpp %1, %1, %0 " CTRL " bank_mask:0xf\n\t" \
+    "v_mul_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"  \
+    "s_nop 0\n\t"
+    asm("s_nop 1\n\t"
+                 SS2D_SCAN_STEP("row_shr:1 row_mask:0xf")
+                 SS2D_SCAN_STEP("row_shr:2 row_mask:0xf")
+                 SS2D_SCAN_STEP("row_shr:4 row_mask:0xf")
+                 SS2D_SCAN_STEP("row_shr:8 row_mask:0xf")
+                 SS2D_SCAN_STEP("row_bcast:15 row_mask:0xa")
+                 SS2D_SCAN_STEP("row_bcast:31 row_mask:0xc")
+                 "s_nop 0\n\t"
+                 "v_mov_b32_dpp %2, %0 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "v_mov_b32_dpp %3, %1 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1"
+                 : "+v"(a), "+v"(h), "+v"(ax), "+v"(hx));
 #undef SS2D_SCAN_STEP
-    a_ex = dpp_move<kDppWaveShr1>(1.0f, a);
-    h_ex = dpp_move<kDppWaveShr1>(0.0f, h);
+    a_ex = ax;
+    h_ex = hx;
     a_tot = read_lane(a, kWave - 1);
     h_tot = read_lane(h, kWave - 1);
 }

@@ -11,13 +11,12 @@
 //     kernels: 8 positions per lane, DPP wavefront scan, state carried in a register, softplus fused;
 //   * each wavefront puts its outputs into an fp32 LDS plane at the position the merge wants them: plane A
 //     (row-major index) collects directions 0 and 2, plane B (column-major index) directions 1 and 3.  Every
-//     plane entry has exactly two writers, one forward and one backward direction; whichever comes first
-//     stores, the other adds, giving fl(y0 + y2) resp. fl(y1 + y3) -- the association order of cross_merge_fwd
+//     plane entry has exactly two writers, one forward and one backward direction; the planes start at zero and
+//     both add, giving fl(y0 + y2) resp. fl(y1 + y3) -- the association order of cross_merge_fwd
 //     (classification/models/csm_triton.py:61-62) -- and ys never exists.  LDS float atomics are an order of
-//     magnitude slower than plain LDS traffic on this chip, so the order is fixed by construction instead: the
-//     four wavefronts advance pass by pass, in each pass the forward directions update the planes, a barrier,
-//     then the backward directions, a barrier; "who is first" follows from the pass in which the other
-//     direction reaches the same entry;
+//     magnitude slower than plain LDS traffic on this chip, so the updates are plain read-add-write sequences kept
+//     apart by construction: the four wavefronts advance pass by pass, in each pass the forward directions update
+//     the planes, a barrier, then the backward directions, a barrier;
 //   * finally out[r] = A[r] + B[t(r)] is written once.
 // HBM traffic per element: x (s_in) + 4 delta (4 s_in) + out (s_out) = 14 bytes instead of 62.
 //
@@ -29,6 +28,8 @@
 // in the flat scan kernel), which needs their delta rows adjacent in memory: delta is therefore taken with
 // explicit (direction, channel, batch) strides and CB > 1 requires batch stride == L, i.e. the batch-innermost
 // layout (K, D, B, L) that a single large dt_proj GEMM per direction produces.
+#include <type_traits>
+
 #include "scan_common.h"
 
 namespace ss2d {
@@ -53,7 +54,14 @@ template <int kBytes> __host__ __device__ __forceinline__ constexpr int lds_exte
     return (lds_index<kBytes>(n) + 8) & ~7;
 }
 
-constexpr int kCoreBurst = 4;     // passes whose delta / B / C loads are in flight per wavefront
+// The x maps carry one extra aligned block of kItems zeros behind the last image: groups past the end of the stream
+// read their u there, so that u = 0 (and with it the drive term) needs no select.
+__host__ __device__ __forceinline__ constexpr int core_zero_block(int n) { return (n + kItems - 1) & ~(kItems - 1); }
+template <int kBytes> __host__ __device__ __forceinline__ constexpr int core_map_extent(int n) {
+    return lds_extent<kBytes>(core_zero_block(n) + kItems);
+}
+
+constexpr int kCoreBurst = 2;     // passes whose delta / B / C loads are in flight per wavefront
 
 // What one pass of one lane loads from memory, as it arrives.
 template <typename in_t, int kGran>
@@ -65,7 +73,7 @@ struct CorePassLoads {
     uint32_t i0, j0;      // image and position of the lane's first item
 };
 
-template <typename in_t, bool kSoftplus, int kGran>
+template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta>
 __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD) {
     extern __shared__ __align__(16) float core_smem[];
     constexpr int kEs = (int)sizeof(in_t);
@@ -73,7 +81,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     using Loads = CorePassLoads<in_t, kGran>;
     const int L = p.L, H = p.H;
     const int n_max = p.CB * L;
-    const int plane_ext = lds_extent<4>(n_max), map_ext = lds_extent<kEs>(n_max);
+    const int plane_ext = lds_extent<4>(n_max), map_ext = core_map_extent<kEs>(n_max);
     float *planeA = core_smem;                           // fl(y0 + y2), row-major index
     float *planeB = planeA + plane_ext;                  // fl(y1 + y3), column-major index
     in_t *xR = reinterpret_cast<in_t *>(planeB + plane_ext);
@@ -88,11 +96,12 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     // ---- this wavefront's direction ---------------------------------------------------------------------------
     const int lane = threadIdx.x & (kWave - 1);
     const int dir = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const bool reverse = dir >= 2;
+    const int zero_block = core_zero_block(n_max);
     const in_t *xs = (dir & 1) ? xT : xR;
     float *plane = (dir & 1) ? planeB : planeA;
     const int kd = dir * p.D + (int)d;
     const in_t *dl_base = reinterpret_cast<const in_t *>(p.delta) + dir * p.dl_ks + (int64_t)d * p.dl_ds + b0 * p.dl_bs;
+    const __amdgpu_buffer_rsrc_t dl_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<in_t *>(dl_base), 0, (n_el * kEs + 3) & ~3, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bm), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Cm), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     const uint32_t B_soff = (uint32_t)(dir * p.B_ks + b0 * p.B_bs), C_soff = (uint32_t)(dir * p.C_ks + b0 * p.C_bs);
@@ -108,8 +117,20 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     divmod((uint32_t)kPass, divL, step_i, step_j);
     auto issue = [&](int pass, Loads &r) {
         const int e0 = pass * kPass + lane * kItems;
-        if (e0 + kItems <= n_el && p.vec_ok) r.dl = load_raw<in_t, true>(dl_base, e0, n_el, delta_fill<kSoftplus>());
-        else r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
+        if constexpr (kVecDelta) {
+            // the stream starts 16-byte aligned (host-checked); the descriptor's range check returns 0 for the dwords
+            // past its end.  What those items hold is immaterial: they follow every valid item of the stream, their u
+            // is 0 and their outputs are never stored.
+            const int byte_off = e0 * kEs;
+            const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off, 0, 0);
+            r.dl.w[0] = t0[0]; r.dl.w[1] = t0[1]; r.dl.w[2] = t0[2]; r.dl.w[3] = t0[3];
+            if constexpr (kEs == 4) {
+                const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off + 16, 0, 0);
+                r.dl.w[4] = t1[0]; r.dl.w[5] = t1[1]; r.dl.w[6] = t1[2]; r.dl.w[7] = t1[3];
+            }
+        } else {
+            r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
+        }
         r.i0 = next_i; r.j0 = next_j;
         next_i += step_i; next_j += step_j;
         if (next_j >= (uint32_t)L) { next_j -= (uint32_t)L; next_i += 1; }
@@ -189,17 +210,27 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             }
         }
     }
+    // the merge planes start at zero (every entry is then updated by plain read-add-write, 0 + y being exact), and so
+    // does the block behind the maps
+    {
+        float4 *planes4 = reinterpret_cast<float4 *>(planeA);
+        for (int i = threadIdx.x; i < 2 * plane_ext / 4; i += kBlock) planes4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (threadIdx.x < 2 * kItems) {
+            in_t *m = threadIdx.x < kItems ? xR : xT;
+            m[lds_index<kEs>(core_zero_block(n_max) + (int)(threadIdx.x % kItems))] = in_t{};
+        }
+    }
     __syncthreads();
 
     // ---- scan: 8 positions per lane per pass, loads kCoreBurst passes ahead ---------------------------------------
     // Where one group of kGran consecutive positions (never split between images) sits in the LDS arrays.
     struct GroupSlot {
         int plane_idx;     // index into the plane of the group's lowest logical index
-        bool valid, add;   // inside the stream; add to the plane entry (the other direction was there first) or store
+        bool valid;        // inside the stream
     };
 
     // One pass: the outputs in yv (scan order) and the plane slots of its groups.
-    auto compute = [&](int pass, const Loads &r, float &h_carry, float (&yv)[kItems], GroupSlot (&slot)[kGroups]) {
+    auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kItems], GroupSlot (&slot)[kGroups]) {
         const int e0 = pass * kPass + lane * kItems;
         const int j0 = (int)r.j0, i0 = (int)r.i0;
         const int k = kGran == kItems ? kItems : min(kItems, L - j0);
@@ -223,22 +254,15 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             // backwards img*L + L-1 - (jg + t), i.e. the block starting at img*L + L - jg - kGran read downwards.
             const bool valid = e0 + gi * kGran < n_el;
             int base = reverse ? img_off + L - jg - kGran : e0 + gi * kGran;
-            base = valid ? base : 0;
-            // the other direction reaches this block at the mirrored stream position of the same image
-            const int other_pos = reverse ? base : 2 * img_off + L - 1 - base;
-            const int other_pass = (int)((uint32_t)other_pos / (uint32_t)kPass);
+            base = valid ? base : zero_block;                                // past the end: u = 0
             slot[gi].valid = valid;
-            slot[gi].add = reverse ? other_pass <= pass : other_pass < pass;
             slot[gi].plane_idx = lds_index<4>(base);
             const in_t *src = xs + lds_index<kEs>(base);                     // no pad word inside an aligned block
             float um[kGran];
 #pragma unroll
             for (int c = 0; c < kGran; ++c) um[c] = to_f32(src[c]);
 #pragma unroll
-            for (int t = 0; t < kGran; ++t) {
-                const float v = reverse ? um[kGran - 1 - t] : um[t];
-                uv[gi * kGran + t] = valid ? v : 0.0f;
-            }
+            for (int t = 0; t < kGran; ++t) uv[gi * kGran + t] = reverse ? um[kGran - 1 - t] : um[t];
         }
         float dl[kItems], bias_items[kItems];
 #pragma unroll
@@ -247,11 +271,12 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         float ac[kItems], hh[kItems];
 #pragma unroll
         for (int i = 0; i < kItems; ++i) {
-            // past the end of the stream delta was filled so that dl = 0 (softplus) or is zeroed here; u is 0 there
+            // past the end of the stream delta was filled so that dl = 0 (softplus) or is zeroed here; u is 0 there and
+            // B finite (the buffer load returns 0 out of range), so the pair is the identity (1, 0)
             if constexpr (!kSoftplus) dl[i] = slot[i / kGran].valid ? dl[i] : 0.0f;
             float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
             if (i % kGran == 0) a = first[i / kGran] ? 0.0f : a;
-            const float bb = slot[i / kGran].valid ? Bv[i] * (dl[i] * uv[i]) : 0.0f;
+            const float bb = Bv[i] * (dl[i] * uv[i]);
             ac[i] = i == 0 ? a : ac[i - 1] * a;
             hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
         }
@@ -263,42 +288,46 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         for (int i = 0; i < kItems; ++i) yv[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), Dv * uv[i]);
     };
 
-    // Plane update of one pass.  An entry at logical index a of image img is written by the forward direction in
-    // pass a / 512 and by the backward direction in pass (2*img*L + L-1 - a) / 512 (its stream position there is
-    // the mirror image of a within the image).  The earlier pass stores, the later one adds; in the same pass the
-    // forward direction goes first (the barrier between the two halves of a pass orders them).
-    auto update_plane = [&](const float (&yv)[kItems], const GroupSlot (&slot)[kGroups]) {
+    // Plane update of one pass: every entry is reached once by the forward and once by the backward direction of its
+    // plane; both add to the zero-initialised entry, so it ends as fl(y_fwd + y_bwd) whatever the order.  Only when the
+    // two meet in the same pass could the read-add-write sequences overlap: the barrier between the two halves of a
+    // pass keeps them apart.
+    auto update_plane = [&](bool reverse, const float (&yv)[kItems], const GroupSlot (&slot)[kGroups]) {
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             if (slot[gi].valid) {
                 float *dst = plane + slot[gi].plane_idx;
+                float old[kGran];
 #pragma unroll
-                for (int c = 0; c < kGran; ++c) {
-                    const float y = reverse ? yv[gi * kGran + kGran - 1 - c] : yv[gi * kGran + c];
-                    const float old = dst[c];
-                    dst[c] = slot[gi].add ? old + y : y;
-                }
+                for (int c = 0; c < kGran; ++c) old[c] = dst[c];
+#pragma unroll
+                for (int c = 0; c < kGran; ++c) dst[c] = old[c] + (reverse ? yv[gi * kGran + kGran - 1 - c] : yv[gi * kGran + c]);
             }
         }
     };
 
-    float h_carry = 0.0f;
-    for (int pass0 = 0; pass0 < n_pass; pass0 += kCoreBurst) {
+    auto run_passes = [&](bool rev) {
+        const bool reverse = rev;
+        float h_carry = 0.0f;
+        for (int pass0 = 0; pass0 < n_pass; pass0 += kCoreBurst) {
 #pragma unroll
-        for (int q = 0; q < kCoreBurst; ++q) {
-            const int pass = pass0 + q;
-            if (pass < n_pass) {                     // uniform over the workgroup: every wavefront meets every barrier
-                float yv[kItems];
-                GroupSlot slot[kGroups];
-                compute(pass, regs[q], h_carry, yv, slot);
-                if (!reverse) update_plane(yv, slot);
-                __syncthreads();
-                if (reverse) update_plane(yv, slot);
-                __syncthreads();
-                if (pass + kCoreBurst < n_pass) issue(pass + kCoreBurst, regs[q]);
+            for (int q = 0; q < kCoreBurst; ++q) {
+                const int pass = pass0 + q;
+                if (pass < n_pass) {                 // uniform over the workgroup: every wavefront meets every barrier
+                    float yv[kItems];
+                    GroupSlot slot[kGroups];
+                    compute(rev, pass, regs[q], h_carry, yv, slot);
+                    if (!reverse) update_plane(false, yv, slot);
+                    __syncthreads();
+                    if (reverse) update_plane(true, yv, slot);
+                    __syncthreads();
+                    if (pass + kCoreBurst < n_pass) issue(pass + kCoreBurst, regs[q]);
+                }
             }
         }
-    }
+    };
+    // the direction is uniform per wavefront; both branches meet the same barriers
+    run_passes(dir >= 2);
 
     // ---- merge: out[r] = A[r] + B[t(r)] ---------------------------------------------------------------------------
     float *yo = reinterpret_cast<float *>(p.y);
@@ -321,25 +350,32 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
 }
 
 constexpr size_t kCoreMaxLds = 64 * 1024;
+constexpr size_t kCoreFourPerCu = 40 * 1024;    // a quarter of the 160 KB of LDS of a CU
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
 
 template <typename in_t>
 static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t L = a.L;
-    // images per workgroup: ~3072 positions per direction; a workgroup's first delta row sits on a 16-byte
-    // boundary when CB*L is a multiple of 8 elements
-    const int64_t align_rows = 8 / core_gcd(L, 8);
-    int64_t CB = (3072 + L / 2) / L;
-    CB = CB < 1 ? 1 : CB;
-    CB = (CB + align_rows - 1) / align_rows * align_rows;
-    if (CB >= a.B) CB = a.B;                                  // a single tile starts at image 0
-    if (CB > 1 && a.dl_bs != L) CB = 1;                       // adjacent delta rows need the batch-innermost layout
+    // Images per workgroup.  A workgroup walks its CB images as one stream in passes of 512 positions, so the last
+    // pass of a tile is partly empty; CB is chosen to minimise the passes of the whole batch among the tile sizes whose
+    // LDS arrays still let four workgroups share a CU (~3400 positions).  A workgroup's first delta row sits on a
+    // 16-byte boundary when CB*L is a multiple of 8 elements.
     auto lds_bytes = [&](int64_t cb) {
         const int n = (int)(cb * L);
-        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)lds_extent<(int)sizeof(in_t)>(n) * sizeof(in_t);
+        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)core_map_extent<(int)sizeof(in_t)>(n) * sizeof(in_t);
     };
-    while (CB > 1 && lds_bytes(CB) > kCoreMaxLds) CB = CB > align_rows ? CB - align_rows : 1;
+    const int64_t align_rows = 8 / core_gcd(L, 8);
+    auto passes = [&](int64_t images) { return (images * L + kPass - 1) / kPass; };
+    int64_t CB = 1;
+    if (a.dl_bs == L) {                                       // adjacent delta rows need the batch-innermost layout
+        int64_t best = -1;
+        for (int64_t cb = align_rows; cb < a.B && lds_bytes(cb) <= kCoreFourPerCu; cb += align_rows) {
+            const int64_t cost = (a.B / cb) * passes(cb) + passes(a.B % cb);
+            if (best < 0 || cost <= best) { best = cost; CB = cb; }
+        }
+        if (lds_bytes(a.B) <= kCoreFourPerCu && (best < 0 || passes(a.B) <= best)) CB = a.B;   // a single tile starts at image 0
+    }
     const size_t smem = lds_bytes(CB);
     if (smem > kCoreMaxLds) return SS2D_ENOTSUP;
     a.CB = (int)CB;
@@ -358,8 +394,11 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t n_wg = tiles * a.D;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dD = make_fastdiv((uint32_t)a.D);
-#define SS2D_CORE_LAUNCH(SP, G) \
-    hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD)
+#define SS2D_CORE_LAUNCH(SP, G)                                                                                                     \
+    do {                                                                                                                            \
+        if (a.vec_ok) hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD); \
+        else hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD);       \
+    } while (0)
     if (a.softplus) {
         if (g == 8) SS2D_CORE_LAUNCH(true, 8); else if (g == 4) SS2D_CORE_LAUNCH(true, 4); else SS2D_CORE_LAUNCH(true, 1);
     } else {
