@@ -59,9 +59,14 @@ def run_core(x, delta, Bs, Cs, A, Dv, bias, softplus=True):
 
 CORE_SHAPES = [
     (2, 3, 56, 56),      # one image per workgroup, 8-wide B/C groups
-    (5, 4, 28, 28),      # four images per workgroup + a one-image tail
-    (18, 2, 14, 14),     # L % 8 == 4: 16 images per workgroup, tail of two
-    (70, 2, 7, 7),       # odd L: 64 images per workgroup, element-wise B/C gathers
+    (5, 4, 28, 28),      # several images per workgroup + a shorter last tile
+    (18, 2, 14, 14),     # L % 8 == 4: an even number of images per workgroup
+    (19, 1, 14, 14),     # ... and a last tile of odd length: its final 16-byte delta load runs past the tensor's end
+    (5, 2, 14, 14),      # one tile whose length is not a multiple of 8
+    (70, 2, 7, 7),       # odd L: many images per workgroup, element-wise B/C gathers
+    (3, 2, 4, 4),        # rows shorter than a block of 8 (element-wise staging), 16-byte merge stores
+    (2, 2, 8, 2),        # rows shorter than 4
+    (2, 2, 2, 8),
     (3, 2, 7, 9),        # H != W, odd L
     (2, 2, 10, 12),      # H != W
     (9, 1, 6, 5),        # L = 30: two-element granularity handled element-wise
@@ -94,6 +99,22 @@ def test_core_optional_arguments(softplus):
         want = oracle_core(x, delta, Bs, Cs, A, dv, bi, softplus)
         got = run_core(x, delta, Bs, Cs, A, dv, bi, softplus)
         assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
+
+
+def test_core_into_caller_buffer_not_16_byte_aligned():
+    """The result may land anywhere a float can: the kernel then stores element by element."""
+    _announce("core unaligned out")
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(5, 3, 2, 28, 28, torch.bfloat16)
+    want = oracle_core(x, delta, Bs, Cs, A, Dv, bias)
+    dev = lambda t: t.to(DEV)
+    buf = torch.full((want.numel() + 5,), 7.0, device=DEV)
+    out = buf[1:1 + want.numel()].view(want.shape)
+    assert out.data_ptr() % 16 == 4
+    got = ss2d_core_hip(dev(x), dev(delta), dev(Bs), dev(Cs), dev(A), dev(Dv), dev(bias), True, out=out)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == out.data_ptr()
+    assert torch.allclose(got.cpu(), want, **TOL)
+    assert buf[0].item() == 7.0 and torch.all(buf[1 + want.numel():] == 7.0)
 
 
 def test_core_reference_layout_strides():

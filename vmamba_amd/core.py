@@ -32,9 +32,10 @@ def core_fits(H, W, dtype):
     return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024
 
 
-def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True):
+def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True, out=None):
     """x (B,D,H,W); delta (4,D,B,L) view; Bs, Cs (4,B,L) views (last stride 1), all of x.dtype and already in the
-    scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32.
+    scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32 (written into
+    ``out`` when given: a contiguous fp32 tensor of that shape).
 
     Raises Ss2dError with status SS2D_ENOTSUP when the shape has no fused kernel (image too large for the LDS
     planes, unaligned delta rows): callers fall back to the three separate operators.
@@ -59,7 +60,12 @@ def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus
                "delta_bias must be (4*dim) float32")
         delta_bias = delta_bias.contiguous()
     x = x.contiguous()
-    y = torch.empty((B, D, L), device=x.device, dtype=torch.float32)
+    if out is None:
+        y = torch.empty((B, D, L), device=x.device, dtype=torch.float32)
+    else:
+        _check(out.is_cuda and out.dtype == torch.float32 and tuple(out.shape) == (B, D, L) and out.is_contiguous(),
+               "out must be a contiguous float32 GPU tensor of shape (batch, dim, L)")
+        y = out
     p = _lib.CoreParams()
     p.batch, p.dim, p.height, p.width = B, D, H, W
     p.in_dtype = _DTYPE_CODE[x.dtype]

@@ -38,7 +38,7 @@ struct CoreArgs {
     const void *x, *delta, *Bm, *Cm;
     const float *A, *Dv, *bias;
     void *y;
-    int32_t B, D, H, W, L, CB, softplus, vec_ok;
+    int32_t B, D, H, W, L, CB, softplus, vec_ok, vec_out;
     int64_t dl_ks, dl_ds, dl_bs;        // delta strides over direction, channel, batch (elements)
     int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
     uint32_t B_span_bytes, C_span_bytes;
@@ -154,40 +154,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
 
     // ---- stage: copy the maps into xR / xT ------------------------------------------------------------------------
     const in_t *xin = reinterpret_cast<const in_t *>(p.x);
-    if constexpr (kGran == kItems && sizeof(in_t) == 2) {
-        // rows are multiples of 8 elements (and 16-byte aligned, host-checked through kGran): 16-byte loads
-        const int n_vec = n_el / kItems;
-        for (int base = 0; base < n_vec; base += 2 * kBlock) {
-            uint4 v[2];
-            uint32_t ii[2], rr[2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int vi = base + u * kBlock + (int)threadIdx.x;
-                divmod((uint32_t)min(vi, n_vec - 1) * kItems, divL, ii[u], rr[u]);
-                v[u] = *reinterpret_cast<const uint4 *>(xin + ((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]);
-            }
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int vi = base + u * kBlock + (int)threadIdx.x;
-                if (vi < n_vec) {
-                    const uint32_t w32[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
-                    uint32_t h, w;
-                    divmod(rr[u], divW, h, w);
-                    const int at_r = vi * kItems;
-                    int at_t = (int)(ii[u] * L + w * H + h);
-#pragma unroll
-                    for (int i = 0; i < kItems; ++i) {
-                        const in_t e = in_t{(uint16_t)(w32[i / 2] >> (16 * (i % 2)))};
-                        xR[lds_index<kEs>(at_r + i)] = e;
-                        xT[lds_index<kEs>(at_t)] = e;
-                        ++w;                                   // next column, wrapping to the next row
-                        at_t += H;
-                        if ((int)w == p.W) { w = 0; ++h; at_t = (int)(ii[u] * L + h); }
-                    }
-                }
-            }
-        }
-    } else {
+    auto stage_elements = [&]() {
         constexpr int kChunk = 8;
         for (int base = 0; base < n_el; base += kChunk * kBlock) {
             in_t v[kChunk];
@@ -209,6 +176,46 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
                 }
             }
         }
+    };
+    if constexpr (kGran == kItems && sizeof(in_t) == 2) {
+        if (p.W >= kItems) {
+            // rows are multiples of 8 elements (and 16-byte aligned, host-checked through kGran): 16-byte loads.  A block
+            // of 8 lies in one image and, with W >= 8, in at most two rows of it.
+            const int n_vec = n_el / kItems;
+            for (int base = 0; base < n_vec; base += 2 * kBlock) {
+                uint4 v[2];
+                uint32_t ii[2], rr[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int vi = base + u * kBlock + (int)threadIdx.x;
+                    divmod((uint32_t)min(vi, n_vec - 1) * kItems, divL, ii[u], rr[u]);
+                    v[u] = *reinterpret_cast<const uint4 *>(xin + ((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int vi = base + u * kBlock + (int)threadIdx.x;
+                    if (vi < n_vec) {
+                        const uint32_t w32[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+                        uint32_t h, w;
+                        divmod(rr[u], divW, h, w);
+                        *reinterpret_cast<uint4 *>(xR + lds_index<kEs>(vi * kItems)) = v[u];   // no pad word inside the block
+                        // column-major index of element i: row h, column w + i while that is < W, then row h + 1
+                        const int n_first = p.W - (int)w;
+                        const int t0 = (int)(ii[u] * L + w * H + h);
+                        const int t1 = (int)(ii[u] * L + h + 1) - n_first * H;
+#pragma unroll
+                        for (int i = 0; i < kItems; ++i) {
+                            const int at_t = (i < n_first ? t0 : t1) + i * H;
+                            xT[lds_index<kEs>(at_t)] = in_t{(uint16_t)(w32[i / 2] >> (16 * (i % 2)))};
+                        }
+                    }
+                }
+            }
+        } else {
+            stage_elements();
+        }
+    } else {
+        stage_elements();
     }
     // the merge planes start at zero (every entry is then updated by plain read-add-write, 0 + y being exact), and so
     // does the block behind the maps
@@ -331,6 +338,34 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
 
     // ---- merge: out[r] = A[r] + B[t(r)] ---------------------------------------------------------------------------
     float *yo = reinterpret_cast<float *>(p.y);
+    if (kGran >= 4 && p.vec_out && p.W >= 4) {
+        // four consecutive positions per lane (L is a multiple of kGran, so they share an image and, with W >= 4, span
+        // at most two rows): one 16-byte store
+        const int n_quad = n_el / 4;
+        for (int base = 0; base < n_quad; base += 2 * kBlock) {
+            float4 v[2];
+            size_t off[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int idx = 4 * min(base + u * kBlock + (int)threadIdx.x, n_quad - 1);
+                uint32_t i, r, h, w;
+                divmod((uint32_t)idx, divL, i, r);
+                divmod(r, divW, h, w);
+                const float *pa = planeA + lds_index<4>(idx);               // no pad word inside an aligned group of 4
+                const int n_first = p.W - (int)w;
+                const int t0 = (int)(i * L + w * H + h), t1 = (int)(i * L + h + 1) - n_first * H;
+                float o[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) o[c] = pa[c] + planeB[lds_index<4>((c < n_first ? t0 : t1) + c * H)];
+                v[u] = make_float4(o[0], o[1], o[2], o[3]);
+                off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (base + u * kBlock + (int)threadIdx.x < n_quad) *reinterpret_cast<float4 *>(yo + off[u]) = v[u];
+        }
+        return;
+    }
     for (int base = 0; base < n_el; base += 4 * kBlock) {
         float v[4];
         size_t off[4];
@@ -384,6 +419,7 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t vec = 16 / (int64_t)sizeof(in_t);
     a.vec_ok = (reinterpret_cast<uintptr_t>(a.delta) % 16 == 0) && a.dl_ks % vec == 0 && a.dl_ds % vec == 0 &&
                (CB >= a.B || (CB * a.dl_bs) % vec == 0);
+    a.vec_out = reinterpret_cast<uintptr_t>(a.y) % 16 == 0;   // 16-byte stores of the result (rows are multiples of 4 then)
     int64_t g = core_gcd(L, kItems);
     const int64_t strides[] = {a.B_ks, a.B_bs, a.C_ks, a.C_bs};
     for (int64_t s : strides) g = core_gcd(g, s == 0 ? g : s);
@@ -434,7 +470,7 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     const int64_t B_span = (3 * a.B_ks + (int64_t)(a.B - 1) * a.B_bs + L) * eb, C_span = (3 * a.C_ks + (int64_t)(a.B - 1) * a.C_bs + L) * eb;
     if (B_span >= 0x7fffffffll || C_span >= 0x7fffffffll) return SS2D_ENOTSUP;
     a.B_span_bytes = (uint32_t)B_span; a.C_span_bytes = (uint32_t)C_span;
-    a.CB = 1; a.vec_ok = 0;
+    a.CB = 1; a.vec_ok = 0; a.vec_out = 0;
 
     hipStream_t s = (hipStream_t)stream;
     if (q->in_dtype == SS2D_F32) return launch_core<float>(a, s);
