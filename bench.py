@@ -210,6 +210,10 @@ def main():
     torch.backends.cudnn.benchmark = True
     torch.manual_seed(0)
     model = vmamba_tiny_s1l8(channel_first=(args.layout == "channel_first")).to(dev).bfloat16().eval()
+    if args.layout != "channel_first":
+        # conv weights in channels-last memory format (same values, same state_dict): the stem / downsample convs then
+        # run NHWC kernels and the permutes around them are views instead of copies
+        model = model.to(memory_format=torch.channels_last)
     x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
 
     def capture_forward():

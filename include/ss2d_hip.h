@@ -274,6 +274,19 @@ int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, i
 int ss2d_mlp_fused(const void *x, const void *w1, const void *b1, const void *w2, const void *b2, const void *residual,
                    void *out, int64_t M, int C, int dtype, void *stream);
 
+/*
+ * Narrow channel-last projection with its neighbours folded in:  out = [LayerNorm](x) W^T + bias + residual.
+ * Replaces, in a VSS block, norm + in_proj (classification/models/vmamba.py:1225-1227 ln_1, :648-650 in_proj) and
+ * out_proj + the residual add (:662, :1228) where the layer is too narrow for a library GEMM to reach the HBM bound.
+ *   x (M, K), residual (M, N) or NULL, out (M, N) contiguous;  weight (N, K);  bias (N) or NULL;
+ *   ln_weight (K) or NULL = no LayerNorm, ln_bias (K) or NULL, eps;  all SS2D_BF16 or all SS2D_F16, 16-byte aligned.
+ *   LayerNorm output, projection output and the sum are each rounded to the tensor type, as the separate operators
+ *   would; statistics are fp32.
+ * K = N = 96 only: anything else, and SS2D_F32, returns SS2D_ENOTSUP.
+ */
+int ss2d_linear_cl(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
+                   const void *bias, const void *residual, void *out, int64_t M, int K, int N, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

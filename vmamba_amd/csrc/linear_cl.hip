@@ -1,0 +1,213 @@
+// Narrow channel-last projection with its neighbours folded in:
+//     out = [LayerNorm](x) W^T + bias + residual        x (M, K), W (N, K), 16-bit tensors, K = N = 96
+// -- the in_proj of a VSS block with the block's first LayerNorm in front (classification/models/vmamba.py:1225-1227,
+// :648-650) and its out_proj with the residual add behind (:662, :1228).  At K = N = 96 these GEMMs move 154 MB for
+// 7.4 GFLOP: they are bound by HBM, and the library kernels picked for them reach 1.5 TB/s.  Here the whole weight
+// matrix (18 KB) sits in LDS, a wavefront owns 64 positions at a time, reads them with 16-byte loads into a private
+// LDS tile (normalising the rows in place when asked to), takes matrix-core fragments from there
+// (D[n][position] = W x^T, v_mfma_f32_32x32x16, fp32 accumulate) and sends the result back through the tile so that
+// the stores and the residual loads are 16 bytes per lane as well.
+// Rounding follows the separate operators: LayerNorm output, projection output (+ bias), and the sum with the
+// residual are each rounded to the tensor type.  LayerNorm statistics are fp32 with the centred variance.
+#include "ss2d_common.h"
+
+namespace ss2d {
+
+struct LinArgs {
+    const void *x, *ln_w, *ln_b, *w, *bias, *residual;
+    void *out;
+    int64_t M;
+    float eps;
+    int tiles_per_wg;
+};
+
+template <typename T, int K, int N, int kCT, bool kLN>
+__global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
+    constexpr int kSteps = K / 16;                  // k-steps of the contraction
+    constexpr int kOG = N / 32;                     // output-channel groups
+    constexpr int PK = K + 8;                       // weight row pitch (elements): 16-byte rows, banks spread
+    constexpr int kMaxKN = K > N ? K : N;
+    constexpr int PS = kMaxKN + 8;                  // staging pitch
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int kRowPieces = PK / 8, kPiecesW = N * kRowPieces;     // 16-byte pieces of the padded weight array
+    static_assert(kPiecesW % 32 == 0, "whole or half wavefronts of pieces");
+    extern __shared__ __align__(16) uint16_t lin_smem[];
+    uint16_t *wl = lin_smem;                                        // [N][PK]
+    uint16_t *stage_all = wl + N * PK;                              // [kWaves][32][PS]
+    uint16_t *bias_l = stage_all + kWaves * 32 * PS;                // [N]
+    uint16_t *gamma_l = bias_l + N;                                 // [K]
+    uint16_t *beta_l = gamma_l + K;                                 // [K]
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int j = lane & 31, kh = lane >> 5;
+    uint16_t *stage = stage_all + wave * 32 * PS;
+    const T *x = reinterpret_cast<const T *>(p.x);
+    const T *w = reinterpret_cast<const T *>(p.w);
+
+    // ---- weights: global -> LDS directly; the pad piece that ends every row is filled from a valid address ---------
+    constexpr int kDmaIters = (kPiecesW + kBlock - 1) / kBlock;
+#pragma unroll
+    for (int it = 0; it < kDmaIters; ++it) {
+        const int first = (it * kWaves + wave) * kWave;              // wave-uniform
+        if (first + lane < kPiecesW) {
+            const int piece = first + lane;
+            const int n = piece / kRowPieces, q = min(piece % kRowPieces, kRowPieces - 2);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(w + n * K + 8 * q),
+                                             (__attribute__((address_space(3))) void *)(wl + first * 8), 16, 0, 0);
+        }
+    }
+    for (int i = threadIdx.x; i < N; i += kBlock) bias_l[i] = p.bias ? reinterpret_cast<const uint16_t *>(p.bias)[i] : (uint16_t)0;
+    if constexpr (kLN)
+        for (int i = threadIdx.x; i < K; i += kBlock) {
+            gamma_l[i] = reinterpret_cast<const uint16_t *>(p.ln_w)[i];
+            beta_l[i] = p.ln_b ? reinterpret_cast<const uint16_t *>(p.ln_b)[i] : (uint16_t)0;
+        }
+    __syncthreads();
+
+    T *out = reinterpret_cast<T *>(p.out);
+    const T *res = reinterpret_cast<const T *>(p.residual);
+    constexpr int kPiecesIn = 32 * K / 8, kPiecesOut = 32 * N / 8;     // 16-byte pieces of a 32-position tile
+    for (int t = 0; t < p.tiles_per_wg; ++t) {
+        const int64_t pos0 = (((int64_t)blockIdx.x * p.tiles_per_wg + t) * kWaves + wave) * (kCT * 32);
+        if (pos0 >= p.M) break;                                      // wave-uniform; no workgroup barrier below
+        u32x4_t xf[kCT][kSteps];
+#pragma unroll
+        for (int ct = 0; ct < kCT; ++ct) {
+#pragma unroll
+            for (int it = 0; it < kPiecesIn / kWave; ++it) {
+                const int idx = lane + it * kWave;
+                const int r = idx / (K / 8), q = idx % (K / 8);
+                int64_t pos = pos0 + ct * 32 + r;
+                pos = pos < p.M ? pos : p.M - 1;                     // rows past the end: any valid row, never stored
+                *reinterpret_cast<uint4 *>(stage + r * PS + 8 * q) = *reinterpret_cast<const uint4 *>(x + pos * K + 8 * q);
+            }
+            wave_lds_sync();
+            if constexpr (kLN) {
+                // two lanes per row, each half of the channels; statistics meet through one lane exchange
+                constexpr int kHalf = K / 2, kVec = kHalf / 8;
+                static_assert(kHalf % 8 == 0, "whole 16-byte pieces per half row");
+                uint16_t *row = stage + j * PS + kh * kHalf;
+                float v[kHalf];
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) {
+                    const uint4 q4 = *reinterpret_cast<const uint4 *>(row + 8 * i);
+                    const uint32_t ww[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[8 * i + 2 * e] = unpack_lo<T>(ww[e]);
+                        v[8 * i + 2 * e + 1] = unpack_hi<T>(ww[e]);
+                        sum += v[8 * i + 2 * e] + v[8 * i + 2 * e + 1];
+                    }
+                }
+                sum += __shfl_xor(sum, 32);
+                const float mean = sum * (1.0f / K);
+                float sq = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kHalf; ++i) { const float c = v[i] - mean; sq = fmaf(c, c, sq); }
+                sq += __shfl_xor(sq, 32);
+                const float rstd = __builtin_amdgcn_rsqf(sq * (1.0f / K) + p.eps);
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) {
+                    const uint4 g4 = *reinterpret_cast<const uint4 *>(gamma_l + kh * kHalf + 8 * i);
+                    const uint4 b4 = *reinterpret_cast<const uint4 *>(beta_l + kh * kHalf + 8 * i);
+                    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
+                    uint32_t ow[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float lo = fmaf((v[8 * i + 2 * e] - mean) * rstd, unpack_lo<T>(gw[e]), unpack_lo<T>(bw[e]));
+                        const float hi = fmaf((v[8 * i + 2 * e + 1] - mean) * rstd, unpack_hi<T>(gw[e]), unpack_hi<T>(bw[e]));
+                        ow[e] = pack2_from_f32<T>(lo, hi);
+                    }
+                    *reinterpret_cast<uint4 *>(row + 8 * i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+                }
+                wave_lds_sync();
+            }
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) xf[ct][s] = *reinterpret_cast<const u32x4_t *>(stage + j * PS + 16 * s + 8 * kh);
+            wave_lds_sync();
+        }
+#pragma unroll
+        for (int ct = 0; ct < kCT; ++ct) {
+#pragma unroll
+            for (int og = 0; og < kOG; ++og) {
+                floatx16_t acc;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < kSteps; ++s) {
+                    const u32x4_t a = *reinterpret_cast<const u32x4_t *>(wl + (og * 32 + j) * PK + 16 * s + 8 * kh);
+                    acc = mfma_32x32x16(T{}, a, xf[ct][s], acc);
+                }
+                // lane (position j, half kh) holds channels og*32 + 8g + 4kh + t in accumulator 4g + t
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int c0 = og * 32 + 8 * g + 4 * kh;
+                    const uint2 bb = *reinterpret_cast<const uint2 *>(bias_l + c0);
+                    *reinterpret_cast<uint2 *>(stage + j * PS + c0) =
+                        make_uint2(pack2_from_f32<T>(acc[4 * g + 0] + unpack_lo<T>(bb.x), acc[4 * g + 1] + unpack_hi<T>(bb.x)),
+                                   pack2_from_f32<T>(acc[4 * g + 2] + unpack_lo<T>(bb.y), acc[4 * g + 3] + unpack_hi<T>(bb.y)));
+                }
+            }
+            wave_lds_sync();
+#pragma unroll
+            for (int it = 0; it < kPiecesOut / kWave; ++it) {
+                const int idx = lane + it * kWave;
+                const int r = idx / (N / 8), q = idx % (N / 8);
+                const int64_t pos = pos0 + ct * 32 + r;
+                if (pos < p.M) {
+                    uint4 v = *reinterpret_cast<const uint4 *>(stage + r * PS + 8 * q);
+                    if (res) {
+                        const uint4 rv = *reinterpret_cast<const uint4 *>(res + pos * N + 8 * q);
+                        uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+                        const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            vw[e] = pack2_from_f32<T>(unpack_lo<T>(vw[e]) + unpack_lo<T>(rw[e]), unpack_hi<T>(vw[e]) + unpack_hi<T>(rw[e]));
+                        v = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                    }
+                    *reinterpret_cast<uint4 *>(out + pos * N + 8 * q) = v;
+                }
+            }
+            wave_lds_sync();
+        }
+    }
+}
+
+template <typename T, int K, int N, int kCT>
+static int launch_linear(LinArgs a, hipStream_t stream) {
+    constexpr int kMaxKN = K > N ? K : N;
+    const size_t smem = (size_t)(N * (K + 8) + (kBlock / kWave) * 32 * (kMaxKN + 8) + N + 2 * K) * sizeof(uint16_t);
+    const int64_t per_tile = (int64_t)(kBlock / kWave) * kCT * 32;
+    const int64_t tiles = (a.M + per_tile - 1) / per_tile;
+    a.tiles_per_wg = tiles >= 2048 ? 2 : 1;                          // the weight load is shared by two tiles when there are plenty
+    const int64_t n_wg = (tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    if (a.ln_w) hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    else hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    return launch_status();
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_linear_cl(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
+                              const void *bias, const void *residual, void *out, int64_t M, int K, int N, int dtype,
+                              void *stream) {
+    using namespace ss2d;
+    if (M < 0 || K <= 0 || N <= 0) return SS2D_EINVAL;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (M == 0) return SS2D_OK;
+    if (!x || !weight || !out) return SS2D_EINVAL;
+    if (ln_bias && !ln_weight) return SS2D_EINVAL;
+    if (dtype == SS2D_F32 || K != 96 || N != 96) return SS2D_ENOTSUP;          // other widths, fp32: the library GEMMs
+    const void *ptrs[] = {x, ln_weight, ln_bias, weight, bias, residual, out};
+    for (const void *q : ptrs)
+        if (q && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return SS2D_ENOTSUP;
+    LinArgs a;
+    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.w = weight; a.bias = bias; a.residual = residual; a.out = out;
+    a.M = M; a.eps = eps; a.tiles_per_wg = 1;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == SS2D_BF16) return launch_linear<bf16_t, 96, 96, 2>(a, s);
+    return launch_linear<f16_t, 96, 96, 2>(a, s);
+}

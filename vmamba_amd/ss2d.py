@@ -24,6 +24,7 @@ from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
+from .linear import linear_cl_hip, linear_fusable
 from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip, needs_grad
 
 
@@ -188,11 +189,21 @@ class SS2D(nn.Module):
         """out_norm on the merged (B, D, L) map, in the block's layout (vmamba.py:641-646)."""
         return self.layers.out_norm(self.out_norm, y.view(B, D, H, W), self.channel_first, dtype)
 
-    def forward(self, x, residual=None):
-        """``residual`` (same layout as x) is added to the result; channel-last blocks without an out_proj bias fold
-        the addition into the out_proj GEMM (one pass over the activation fewer than the block's separate add,
-        vmamba.py:1228, and one rounding instead of two)."""
-        x = self.in_proj(x)
+    def _narrow(self, x, linear, *extra):
+        """True when ss2d_linear_cl serves this projection: channel-last, 16-bit, width 96, no autograd."""
+        return (not self.channel_first and isinstance(linear, nn.Linear) and not isinstance(linear, Linear2d)
+                and linear_fusable(x, linear.weight) and not needs_grad(x, linear.weight, linear.bias, *extra))
+
+    def forward(self, x, residual=None, pre_norm=None):
+        """``pre_norm``: the block's LayerNorm, applied to x first (vmamba.py:1227); ``residual`` (same layout as x) is
+        added to the result (:1228).  A channel-last block of width 96 runs norm + in_proj and out_proj + add as one
+        HIP kernel each (ss2d_linear_cl); otherwise channel-last blocks without an out_proj bias fold the addition
+        into the out_proj GEMM (one pass over the activation fewer than the block's separate add)."""
+        if (pre_norm is not None and isinstance(pre_norm, nn.LayerNorm) and pre_norm.elementwise_affine
+                and self._narrow(x, self.in_proj, pre_norm.weight, pre_norm.bias)):
+            x = linear_cl_hip(x, self.in_proj.weight, self.in_proj.bias, None, pre_norm.weight, pre_norm.bias, pre_norm.eps)
+        else:
+            x = self.in_proj(x if pre_norm is None else pre_norm(x))
         z = None
         if not self.disable_z:
             x, z = x.chunk(2, dim=(1 if self.channel_first else -1))
@@ -201,6 +212,8 @@ class SS2D(nn.Module):
         y = self.forward_core(x)
         if z is not None:
             y = y * z
+        if self._narrow(y, self.out_proj, residual):
+            return linear_cl_hip(y, self.out_proj.weight, self.out_proj.bias, residual)
         if residual is None:
             return self.out_proj(y)
         if self.channel_first or self.out_proj.bias is not None:

@@ -71,7 +71,7 @@ class VSSBlock(nn.Module):
         self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
     def forward(self, x):
-        x = self.op(self.norm(x), residual=x)
+        x = self.op(x, residual=x, pre_norm=self.norm)
         return self.mlp(self.norm2(x), residual=x)
 
 
