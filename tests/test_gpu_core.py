@@ -64,6 +64,8 @@ CORE_SHAPES = [
     (19, 1, 14, 14),     # ... and a last tile of odd length: its final 16-byte delta load runs past the tensor's end
     (5, 2, 14, 14),      # one tile whose length is not a multiple of 8
     (70, 2, 7, 7),       # odd L: many images per workgroup, element-wise B/C gathers
+    (8, 2, 14, 14),      # 3 full passes + 32 positions walked one per lane
+    (21, 1, 7, 7),       # 2 full passes + 5 positions
     (3, 2, 4, 4),        # rows shorter than a block of 8 (element-wise staging), 16-byte merge stores
     (2, 2, 8, 2),        # rows shorter than 4
     (2, 2, 2, 8),

@@ -132,18 +132,20 @@ __device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32
 //   !kSoftplus: dl = raw + bias; the caller zeroes positions past the end.
 constexpr float kSoftplusThreshold = 20.0f;     // the backward's d softplus / dx is 1 above it, as in the reference
 
+// softplus(x) for z = x * log2e
+__device__ __forceinline__ float softplus_log2(float z) {
+    const float t = __builtin_amdgcn_exp2f(-__builtin_fabsf(z));
+    const float w = 1.0f + t;
+    const float c = t - (w - 1.0f);
+    return fmaf(__builtin_fmaxf(z, 0.0f), kLn2, fmaf(kLn2, __builtin_amdgcn_logf(w), c));
+}
+
 template <bool kSoftplus>
 __device__ __forceinline__ void delta_transform(const float (&raw)[kItems], const float (&bias)[kItems],
                                                 float (&dl)[kItems]) {
     if constexpr (kSoftplus) {
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) {
-            const float z = fmaf(raw[i], kLog2e, bias[i] * kLog2e);
-            const float t = __builtin_amdgcn_exp2f(-__builtin_fabsf(z));
-            const float w = 1.0f + t;
-            const float c = t - (w - 1.0f);
-            dl[i] = fmaf(__builtin_fmaxf(z, 0.0f), kLn2, fmaf(kLn2, __builtin_amdgcn_logf(w), c));
-        }
+        for (int i = 0; i < kItems; ++i) dl[i] = softplus_log2(fmaf(raw[i], kLog2e, bias[i] * kLog2e));
     } else {
 #pragma unroll
         for (int i = 0; i < kItems; ++i) dl[i] = raw[i] + bias[i];

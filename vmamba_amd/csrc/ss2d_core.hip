@@ -108,7 +108,10 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     const float A_log2e = p.A[kd] * kLog2e;
     const float Dv = p.Dv ? p.Dv[kd] : 0.0f;
     const float bias = p.bias ? p.bias[kd] : 0.0f;
-    const int n_pass = (n_el + kPass - 1) / kPass;
+    // passes of 512 positions; a remainder of at most 64 positions is walked one position per lane instead
+    const int tail_len = n_el % kPass;
+    const bool short_tail = tail_len > 0 && tail_len <= kWave;
+    const int n_pass = short_tail ? n_el / kPass : (n_el + kPass - 1) / kPass;
 
     // Image and position of this lane's first item in the pass issued next: passes are issued strictly in order, so
     // the pair just advances by 512 positions each time (no division in the loop).
@@ -313,6 +316,37 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         }
     };
 
+    // The short last pass: lane l holds stream position 512 * n_pass + l.  Same arithmetic and the same two-barrier
+    // plane update as a full pass, one item per lane.
+    auto short_pass = [&](bool reverse, float h_carry) {
+        const int e = n_pass * kPass + lane;
+        const bool valid = e < n_el;
+        uint32_t i, jj;
+        divmod((uint32_t)min(e, n_el - 1), divL, i, jj);
+        const int base = reverse ? (int)(i * L) + L - 1 - (int)jj : e;      // this direction's index of the position
+        float raw = 0.0f, Bv = 0.0f, Cv = 0.0f, u = 0.0f;
+        if (valid) {
+            raw = to_f32(dl_base[e]);
+            Bv = gather_elem<in_t>(B_rsrc, B_soff + i * (uint32_t)p.B_bs + jj);
+            Cv = gather_elem<in_t>(C_rsrc, C_soff + i * (uint32_t)p.C_bs + jj);
+            u = to_f32(xs[lds_index<kEs>(base)]);
+        }
+        float dl = kSoftplus ? softplus_log2(fmaf(raw, kLog2e, bias * kLog2e)) : raw + bias;
+        dl = valid ? dl : 0.0f;
+        float a = __builtin_amdgcn_exp2f(dl * A_log2e);
+        a = (valid && jj == 0) ? 0.0f : a;                                   // an image starts: the state restarts
+        const float b = Bv * (dl * u);
+        float a_ex, h_ex, a_tot, h_tot;
+        wave_scan_pairs(a, b, a_ex, h_ex, a_tot, h_tot);
+        const float h = fmaf(a, fmaf(a_ex, h_carry, h_ex), b);
+        const float y = fmaf(Cv, h, Dv * u);
+        float *dst = plane + lds_index<4>(base);
+        if (!reverse && valid) *dst += y;
+        __syncthreads();
+        if (reverse && valid) *dst += y;
+        __syncthreads();
+    };
+
     auto run_passes = [&](bool rev) {
         const bool reverse = rev;
         float h_carry = 0.0f;
@@ -332,6 +366,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
                 }
             }
         }
+        if (short_tail) short_pass(reverse, h_carry);
     };
     // the direction is uniform per wavefront; both branches meet the same barriers
     run_passes(dir >= 2);
@@ -385,7 +420,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
 }
 
 constexpr size_t kCoreMaxLds = 64 * 1024;
-constexpr size_t kCoreFourPerCu = 40 * 1024;    // a quarter of the 160 KB of LDS of a CU
+constexpr size_t kCoreSixPerCu = 26 * 1024;     // a sixth of the 160 KB of LDS of a CU: the kernel's registers allow six wavefronts per SIMD
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
 
@@ -393,23 +428,27 @@ template <typename in_t>
 static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t L = a.L;
     // Images per workgroup.  A workgroup walks its CB images as one stream in passes of 512 positions, so the last
-    // pass of a tile is partly empty; CB is chosen to minimise the passes of the whole batch among the tile sizes whose
-    // LDS arrays still let four workgroups share a CU (~3400 positions).  A workgroup's first delta row sits on a
-    // 16-byte boundary when CB*L is a multiple of 8 elements.
+    // pass of a tile is partly empty (a remainder of up to 64 positions costs little, see short_pass); CB is chosen to
+    // minimise the passes of the whole batch among the tile sizes whose LDS arrays still let six workgroups share a
+    // CU (~2200 positions; measured: more resident workgroups beat longer tiles).  A workgroup's first delta row sits
+    // on a 16-byte boundary when CB*L is a multiple of 8 elements.
     auto lds_bytes = [&](int64_t cb) {
         const int n = (int)(cb * L);
         return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)core_map_extent<(int)sizeof(in_t)>(n) * sizeof(in_t);
     };
     const int64_t align_rows = 8 / core_gcd(L, 8);
-    auto passes = [&](int64_t images) { return (images * L + kPass - 1) / kPass; };
+    auto passes = [&](int64_t images) {                       // cost of a tile in tenths of a full pass
+        const int64_t n = images * L, rem = n % kPass;
+        return 10 * (n / kPass) + (rem == 0 ? 0 : rem <= kWave ? 3 : 10);
+    };
     int64_t CB = 1;
     if (a.dl_bs == L) {                                       // adjacent delta rows need the batch-innermost layout
         int64_t best = -1;
-        for (int64_t cb = align_rows; cb < a.B && lds_bytes(cb) <= kCoreFourPerCu; cb += align_rows) {
+        for (int64_t cb = align_rows; cb < a.B && lds_bytes(cb) <= kCoreSixPerCu; cb += align_rows) {
             const int64_t cost = (a.B / cb) * passes(cb) + passes(a.B % cb);
             if (best < 0 || cost <= best) { best = cost; CB = cb; }
         }
-        if (lds_bytes(a.B) <= kCoreFourPerCu && (best < 0 || passes(a.B) <= best)) CB = a.B;   // a single tile starts at image 0
+        if (lds_bytes(a.B) <= kCoreSixPerCu && (best < 0 || passes(a.B) <= best)) CB = a.B;   // a single tile starts at image 0
     }
     const size_t smem = lds_bytes(CB);
     if (smem > kCoreMaxLds) return SS2D_ENOTSUP;
