@@ -262,17 +262,20 @@ int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, i
                  int64_t x_rank_stride, int dtype, void *stream);
 
 /*
- * Fused channel-last MLP of a VSS block: out = residual + fc2(GELU(fc1(x))) in one kernel, the hidden activations
- * never leaving the registers.  Replaces Mlp.forward (classification/models/vmamba.py:1116-1131: fc1, GELU (erf form),
- * fc2) and the residual add of VSSBlock (:1229) for the narrow stages.
+ * Fused channel-last MLP of a VSS block: out = residual + fc2(GELU(fc1([LayerNorm](x)))) in one kernel, the hidden
+ * activations never leaving the registers.  Replaces Mlp.forward (classification/models/vmamba.py:1116-1131: fc1, GELU
+ * (erf form), fc2), the residual add of VSSBlock (:1229) and, when ln_weight is given, the block's second LayerNorm
+ * (:1229 norm2) for the narrow stages.
  *   x, residual (may be NULL), out: (M, C) contiguous;  w1 (4C, C), b1 (4C) or NULL;  w2 (C, 4C), b2 (C) or NULL;
- *   all SS2D_BF16 or all SS2D_F16, 16-byte aligned.  fc1 output, GELU output, fc2 output and the sum are each
- *   rounded to the tensor type, as the unfused operators would.
+ *   ln_weight (C) or NULL = no LayerNorm, ln_bias (C) or NULL, eps;  all SS2D_BF16 or all SS2D_F16, 16-byte aligned.
+ *   LayerNorm output, fc1 output, GELU output, fc2 output and the sum are each rounded to the tensor type, as the
+ *   unfused operators would; LayerNorm statistics are fp32.
  * C must be 96 or 192 (wider layers are compute-bound and stay library GEMMs): anything else, and SS2D_F32,
  * returns SS2D_ENOTSUP.
  */
-int ss2d_mlp_fused(const void *x, const void *w1, const void *b1, const void *w2, const void *b2, const void *residual,
-                   void *out, int64_t M, int C, int dtype, void *stream);
+int ss2d_mlp_fused(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *w1, const void *b1,
+                   const void *w2, const void *b2, const void *residual, void *out, int64_t M, int C, int dtype,
+                   void *stream);
 
 /*
  * Narrow channel-last projection with its neighbours folded in:  out = [LayerNorm](x) W^T + bias + residual.

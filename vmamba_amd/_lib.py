@@ -110,7 +110,8 @@ def lib():
         L.ss2d_transpose_bcl.restype = ctypes.c_int
         L.ss2d_transpose_bcl.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
         L.ss2d_mlp_fused.restype = ctypes.c_int
-        L.ss2d_mlp_fused.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        L.ss2d_mlp_fused.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_float] + [ctypes.c_void_p] * 6 +
+                                     [ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
         L.ss2d_linear_cl.restype = ctypes.c_int
         L.ss2d_linear_cl.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_float] + [ctypes.c_void_p] * 4 +
                                      [ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])

@@ -56,9 +56,10 @@ __device__ __forceinline__ uint32_t gelu_pair(f16_t, uint32_t w, const float *) 
 }
 
 struct MlpArgs {
-    const void *x, *w1, *b1, *w2, *b2, *residual;
+    const void *x, *ln_w, *ln_b, *w1, *b1, *w2, *b2, *residual;
     void *out;
     int64_t M;
+    float eps;
 };
 
 template <typename T, int C> struct MlpLayout {
@@ -67,10 +68,10 @@ template <typename T, int C> struct MlpLayout {
                                                                        // aligned and 16 rows x 16 bytes cover all banks
     static constexpr int kW1Elems = kMlpChunk * P1, kW2Elems = C * P2, kBufElems = kW1Elems + kW2Elems;
     static constexpr int kStageElems = kMlpChunk * PS;                 // one 32-position tile per wavefront
-    static constexpr size_t kBytes = (size_t)(2 * kBufElems + 5 * C) * sizeof(uint16_t) + (kTable ? kGeluEntries * sizeof(float) : 0);
+    static constexpr size_t kBytes = (size_t)(2 * kBufElems + 5 * C + 2 * C) * sizeof(uint16_t) + (kTable ? kGeluEntries * sizeof(float) : 0);
 };
 
-template <typename T, int C, int kCT>
+template <typename T, int C, int kCT, bool kLN>
 __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
     using Lay = MlpLayout<T, C>;
     constexpr int kHidden = 4 * C;
@@ -81,12 +82,14 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
     constexpr int kW1Elems = Lay::kW1Elems, kBufElems = Lay::kBufElems, kStageElems = Lay::kStageElems;
     constexpr int kWaves = kBlock / kWave;
     static_assert(2 * kBufElems >= kWaves * kStageElems, "the staging tiles alias the weight buffers");
-    static_assert((2 * kBufElems + 5 * C) % 8 == 0, "the table starts 16-byte aligned");
+    static_assert((2 * kBufElems + 5 * C) % 8 == 0 && C % 8 == 0, "LayerNorm vectors and the table start 16-byte aligned");
     extern __shared__ __align__(16) uint16_t mlp_smem[];
     uint16_t *wbuf = mlp_smem;                                      // [2][W1 chunk | W2 chunk]
     uint16_t *bias1 = mlp_smem + 2 * kBufElems;                     // [4C]
     uint16_t *bias2 = bias1 + kHidden;                              // [C]
-    float *tbl = reinterpret_cast<float *>(bias2 + C);              // [kGeluEntries], bf16 only
+    uint16_t *gamma_l = bias2 + C;                                  // [C] LayerNorm weight
+    uint16_t *beta_l = gamma_l + C;                                 // [C] LayerNorm bias
+    float *tbl = reinterpret_cast<float *>(beta_l + C);             // [kGeluEntries], bf16 only
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -133,6 +136,13 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
     // ---- biases and the GELU table to LDS; x tiles -> fragments -------------------------------------------------------
     for (int i = threadIdx.x; i < kHidden; i += kBlock) bias1[i] = p.b1 ? reinterpret_cast<const uint16_t *>(p.b1)[i] : (uint16_t)0;
     for (int i = threadIdx.x; i < C; i += kBlock) bias2[i] = p.b2 ? reinterpret_cast<const uint16_t *>(p.b2)[i] : (uint16_t)0;
+    if constexpr (kLN) {
+        for (int i = threadIdx.x; i < C; i += kBlock) {
+            gamma_l[i] = reinterpret_cast<const uint16_t *>(p.ln_w)[i];
+            beta_l[i] = p.ln_b ? reinterpret_cast<const uint16_t *>(p.ln_b)[i] : (uint16_t)0;
+        }
+        __syncthreads();                                             // the tiles below read them
+    }
     if constexpr (Lay::kTable)
         for (int i = threadIdx.x; i < kGeluEntries / 4; i += kBlock)
             reinterpret_cast<uint4 *>(tbl)[i] = reinterpret_cast<const uint4 *>(kGeluHalfErfBits)[i];
@@ -149,6 +159,47 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
             *reinterpret_cast<uint4 *>(stage + r * PS + 8 * q) = *reinterpret_cast<const uint4 *>(x + pos * C + 8 * q);
         }
         wave_lds_sync();
+        if constexpr (kLN) {
+            // LayerNorm of the rows in place (fp32 statistics, centred variance, result rounded to the tensor type):
+            // two lanes per row, each half of the channels; the halves meet through one lane exchange
+            constexpr int kHalf = C / 2, kVec = kHalf / 8;
+            uint16_t *row = stage + j * PS + kh * kHalf;
+            float v[kHalf];
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                const uint4 q4 = *reinterpret_cast<const uint4 *>(row + 8 * i);
+                const uint32_t ww[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[8 * i + 2 * e] = unpack_lo<T>(ww[e]);
+                    v[8 * i + 2 * e + 1] = unpack_hi<T>(ww[e]);
+                    sum += v[8 * i + 2 * e] + v[8 * i + 2 * e + 1];
+                }
+            }
+            sum += __shfl_xor(sum, 32);
+            const float mean = sum * (1.0f / C);
+            float sq = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) { const float c = v[i] - mean; sq = fmaf(c, c, sq); }
+            sq += __shfl_xor(sq, 32);
+            const float rstd = __builtin_amdgcn_rsqf(sq * (1.0f / C) + p.eps);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                const uint4 g4 = *reinterpret_cast<const uint4 *>(gamma_l + kh * kHalf + 8 * i);
+                const uint4 b4 = *reinterpret_cast<const uint4 *>(beta_l + kh * kHalf + 8 * i);
+                const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
+                uint32_t ow[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float lo = fmaf((v[8 * i + 2 * e] - mean) * rstd, unpack_lo<T>(gw[e]), unpack_lo<T>(bw[e]));
+                    const float hi = fmaf((v[8 * i + 2 * e + 1] - mean) * rstd, unpack_hi<T>(gw[e]), unpack_hi<T>(bw[e]));
+                    ow[e] = pack2_from_f32<T>(lo, hi);
+                }
+                *reinterpret_cast<uint4 *>(row + 8 * i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+            }
+            wave_lds_sync();
+        }
 #pragma unroll
         for (int s = 0; s < kSteps1; ++s) xf[ct][s] = *reinterpret_cast<const u32x4_t *>(stage + j * PS + 16 * s + 8 * kh);
         wave_lds_sync();
@@ -255,25 +306,28 @@ static int launch_mlp(const MlpArgs &a, hipStream_t stream) {
     const int64_t per_wg = (int64_t)(kBlock / kWave) * kCT * 32;
     const int64_t n_wg = (a.M + per_wg - 1) / per_wg;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-    hipLaunchKernelGGL((mlp_fused_kernel<T, C, kCT>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    if (a.ln_w) hipLaunchKernelGGL((mlp_fused_kernel<T, C, kCT, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    else hipLaunchKernelGGL((mlp_fused_kernel<T, C, kCT, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
     return launch_status();
 }
 
 }  // namespace ss2d
 
-extern "C" int ss2d_mlp_fused(const void *x, const void *w1, const void *b1, const void *w2, const void *b2,
-                              const void *residual, void *out, int64_t M, int C, int dtype, void *stream) {
+extern "C" int ss2d_mlp_fused(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *w1,
+                              const void *b1, const void *w2, const void *b2, const void *residual, void *out, int64_t M,
+                              int C, int dtype, void *stream) {
     using namespace ss2d;
     if (M < 0 || C <= 0) return SS2D_EINVAL;
     if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
     if (M == 0) return SS2D_OK;
     if (!x || !w1 || !w2 || !out) return SS2D_EINVAL;
+    if (ln_bias && !ln_weight) return SS2D_EINVAL;
     if (dtype == SS2D_F32 || (C != 96 && C != 192)) return SS2D_ENOTSUP;       // wider stages, fp32: the library GEMMs
-    const void *ptrs[] = {x, w1, b1, w2, b2, residual, out};
+    const void *ptrs[] = {x, ln_weight, ln_bias, w1, b1, w2, b2, residual, out};
     for (const void *q : ptrs)
         if (q && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return SS2D_ENOTSUP;
     MlpArgs a;
-    a.x = x; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.residual = residual; a.out = out; a.M = M;
+    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.eps = eps; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.residual = residual; a.out = out; a.M = M;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == SS2D_BF16) return C == 96 ? launch_mlp<bf16_t, 96, 2>(a, s) : launch_mlp<bf16_t, 192, 1>(a, s);
     return C == 96 ? launch_mlp<f16_t, 96, 2>(a, s) : launch_mlp<f16_t, 192, 1>(a, s);

@@ -19,8 +19,9 @@ def mlp_fusable(x, fc1, fc2):
             and tuple(fc2.weight.shape) == (C, 4 * C) and fc1.weight.dtype == x.dtype and fc2.weight.dtype == x.dtype)
 
 
-def mlp_fused_hip(x, w1, b1, w2, b2, residual=None):
-    """x (..., C) channel-last; returns residual + fc2(gelu(fc1(x))) with the shape of x."""
+def mlp_fused_hip(x, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, eps=1e-5):
+    """x (..., C) channel-last; returns residual + fc2(gelu(fc1(h))) with the shape of x, where h = x or, when ln_weight
+    is given, layer_norm(x) over the channels."""
     if not x.is_cuda:
         raise NotImplementedError("mlp_fused_hip: vmamba_amd runs on the GPU only")
     if x.dtype not in _DTYPE_CODE:
@@ -36,9 +37,10 @@ def mlp_fused_hip(x, w1, b1, w2, b2, residual=None):
         residual = residual.contiguous()
     out = torch.empty_like(x)
     ptr = lambda t: None if t is None else t.contiguous().data_ptr()
-    keep = [None if t is None else t.contiguous() for t in (b1, b2)]
+    keep = [None if t is None else t.to(x.dtype).contiguous() for t in (b1, b2, ln_weight, ln_bias)]
     with torch.cuda.device(x.device):
-        rc = _lib.lib().ss2d_mlp_fused(x.data_ptr(), w1.data_ptr(), ptr(keep[0]), w2.data_ptr(), ptr(keep[1]), ptr(residual),
+        rc = _lib.lib().ss2d_mlp_fused(x.data_ptr(), ptr(keep[2]), ptr(keep[3]), float(eps), w1.data_ptr(), ptr(keep[0]),
+                                       w2.data_ptr(), ptr(keep[1]), ptr(residual),
                                        out.data_ptr(), x.numel() // C, C, _DTYPE_CODE[x.dtype],
                                        torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "ss2d_mlp_fused")

@@ -49,12 +49,20 @@ class Mlp(nn.Module):
         self.act = nn.GELU()
         self.fc2 = Linear(hidden, dim)
 
-    def forward(self, x, residual=None):
-        """fc2(GELU(fc1(x))) (+ residual).  Channel-last 16-bit inference at widths 96 / 192 runs as one HIP kernel
-        that keeps the hidden activations in registers; everything else on the torch operators."""
+    def forward(self, x, residual=None, pre_norm=None):
+        """fc2(GELU(fc1(h))) (+ residual), h = x or pre_norm(x) (the block's second LayerNorm, vmamba.py:1229).
+        Channel-last 16-bit inference at widths 96 / 192 runs as one HIP kernel that normalises the rows on the way
+        in and keeps the hidden activations in registers; everything else on the torch operators."""
         if (self.fused and not self.channel_first and mlp_fusable(x, self.fc1, self.fc2)
                 and not needs_grad(x, self.fc1.weight, self.fc2.weight, self.fc1.bias, self.fc2.bias)):
-            return mlp_fused_hip(x, self.fc1.weight, self.fc1.bias, self.fc2.weight, self.fc2.bias, residual)
+            if pre_norm is None:
+                return mlp_fused_hip(x, self.fc1.weight, self.fc1.bias, self.fc2.weight, self.fc2.bias, residual)
+            if (isinstance(pre_norm, nn.LayerNorm) and pre_norm.elementwise_affine
+                    and not needs_grad(pre_norm.weight, pre_norm.bias)):
+                return mlp_fused_hip(x, self.fc1.weight, self.fc1.bias, self.fc2.weight, self.fc2.bias, residual,
+                                     pre_norm.weight, pre_norm.bias, pre_norm.eps)
+        if pre_norm is not None:
+            x = pre_norm(x)
         y = self.fc2(self.act(self.fc1(x)))
         return y if residual is None else residual + y
 
@@ -72,7 +80,7 @@ class VSSBlock(nn.Module):
 
     def forward(self, x):
         x = self.op(x, residual=x, pre_norm=self.norm)
-        return self.mlp(self.norm2(x), residual=x)
+        return self.mlp(x, residual=x, pre_norm=self.norm2)
 
 
 class VSSM(nn.Module):
