@@ -25,10 +25,10 @@ def make(seed, M, K, N, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("M", [1, 77, 256, 1000, 16 * 3136, 128 * 3136])
-def test_linear_cl_matches_separate_operators(M, dtype):
-    print("CASE linear_cl", M, dtype, flush=True)
-    K = N = 96
+@pytest.mark.parametrize("M,K", [(1, 96), (77, 96), (256, 96), (1000, 96), (16 * 3136, 96), (128 * 3136, 96)])
+def test_linear_cl_matches_separate_operators(M, K, dtype):
+    print("CASE linear_cl", M, K, dtype, flush=True)
+    N = K
     x, res, w, b, gamma, beta = [t.to(DEV) for t in make(M, M, K, N, dtype)]
     tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
     d = lambda t: t.double()
@@ -72,6 +72,7 @@ def test_linear_cl_rejections():
     L = _lib.lib()
     args = lambda K, N, dt: (x.data_ptr(), None, None, 1e-5, w.data_ptr(), None, None, x.data_ptr(), 8, K, N, dt, None)
     assert L.ss2d_linear_cl(*args(192, 192, _lib.SS2D_BF16)) == _lib.SS2D_ENOTSUP
+    assert L.ss2d_linear_cl(*args(96, 192, _lib.SS2D_BF16)) == _lib.SS2D_ENOTSUP
     assert L.ss2d_linear_cl(*args(96, 96, _lib.SS2D_F32)) == _lib.SS2D_ENOTSUP
     assert L.ss2d_linear_cl(None, None, None, 1e-5, None, None, None, None, 8, 96, 96, _lib.SS2D_BF16, None) == _lib.SS2D_EINVAL
     assert L.ss2d_linear_cl(x.data_ptr(), None, gamma.data_ptr(), 1e-5, w.data_ptr(), None, None, x.data_ptr(), 8, 96, 96,
