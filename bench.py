@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE x1.0); the summary is profiles/ss2d_core_kernels_vmamba_t_bs128.txt.  Counters cannot be read from
 # inside the timed process, so this is the last profiled value, refreshed whenever the kernel changes.
 SCAN_STAGE1_MEASURED_TRAFFIC_BYTES = 668.4e6 + 617.1e6
-CORE_STAGE1_MEASURED_TRAFFIC_BYTES = 437.5e6 + 154.1e6    # same profile: FETCH_SIZE 213622 KiB x 2.0, WRITE_SIZE 150528 KiB
+CORE_STAGE1_MEASURED_TRAFFIC_BYTES = 437.0e6 + 154.1e6    # same profile: FETCH_SIZE 213382 KiB x 2.0, WRITE_SIZE 150528 KiB
 
 
 def log(*a):
@@ -109,6 +109,26 @@ def kernel_lines(reps):
             b_dt = 2 * K * (D + R) * B * L + 2 * K * D * R
             fused.update(dt_proj_us=t_dt * 1e6, dt_proj_GBs=b_dt / t_dt / 1e9)
             del delta_k, B_k, C_k, dts, Wdt
+        if name in ("stage1", "stage2"):
+            # block-level kernels of the narrow stages (harness side): fused LayerNorm + MLP + residual, and at width 96
+            # the two projections with their LayerNorm / residual.  Bytes: activations in and out once (+ residual).
+            from vmamba_amd.mlp import mlp_fused_hip
+            from vmamba_amd.linear import linear_cl_hip, linear_fusable
+            M = B * L
+            xa = torch.randn(M, D, device=dev, generator=g).bfloat16()
+            w1 = (torch.randn(4 * D, D, device=dev, generator=g) * D ** -0.5).bfloat16()
+            w2 = (torch.randn(D, 4 * D, device=dev, generator=g) * (4 * D) ** -0.5).bfloat16()
+            b1, b2 = torch.zeros(4 * D, device=dev).bfloat16(), torch.zeros(D, device=dev).bfloat16()
+            gam, bet = torch.ones(D, device=dev).bfloat16(), torch.zeros(D, device=dev).bfloat16()
+            t_m = time_op(lambda: mlp_fused_hip(xa, w1, b1, w2, b2, xa, gam, bet, 1e-5), reps)
+            fused.update(mlp_fused_us=t_m * 1e6, mlp_fused_TFLOPs=16.0 * M * D * D / t_m / 1e12, mlp_fused_GBs=3 * M * D * 2 / t_m / 1e9)
+            wp = (torch.randn(D, D, device=dev, generator=g) * D ** -0.5).bfloat16()
+            if linear_fusable(xa, wp):
+                t_i = time_op(lambda: linear_cl_hip(xa, wp, None, None, gam, bet, 1e-5), reps)
+                t_o = time_op(lambda: linear_cl_hip(xa, wp, None, xa), reps)
+                fused.update(ln_in_proj_us=t_i * 1e6, ln_in_proj_GBs=2 * M * D * 2 / t_i / 1e9,
+                             out_proj_add_us=t_o * 1e6, out_proj_add_GBs=3 * M * D * 2 / t_o / 1e9)
+            del xa, w1, w2, wp
         out.append(dict(shape=name, B=B, D=D, H=H, W=W, N=N,
                         cross_scan_us=t_cs * 1e6, cross_scan_GBs=b_cs / t_cs / 1e9,
                         scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9,
