@@ -55,6 +55,8 @@ CASES = [
     (2, 32, 2, 1, 700, None, True),        # 16 channels per group: dB / dC summed per workgroup in LDS
     (1, 60, 2, 2, 300, None, True),        # 30 channels per group in two chunks of 15, two states
     (1, 27, 1, 1, 520, 9, True),           # 27 channels in chunks of 14 + 13, delta rows shared by three channels
+    (1, 24, 1, 1, 3136, None, True),       # one state, 7 passes, 6 channels per wavefront (pass-major kernel)
+    (2, 10, 1, 1, 100, None, False),       # the same kernel without softplus, wavefronts with 3 and 2 channels
 ]
 
 
@@ -74,10 +76,11 @@ def test_scan_bwd_fp32_against_float64_autograd(case):
     compare(got2, want2, 2e-3, "no D / bias")
 
 
+@pytest.mark.parametrize("dim,G", [(8, 4), (16, 1)], ids=["rows", "grouped"])
 @pytest.mark.parametrize("dtype,dout_float", [(torch.bfloat16, True), (torch.bfloat16, False), (torch.float16, True)])
-def test_scan_bwd_16bit_inputs(dtype, dout_float):
-    print("CASE scan-bwd-16", dtype, dout_float, flush=True)
-    u, delta, A, B, C, D, bias, dout = make(5, 2, 8, 4, 1, 1200, dtype)
+def test_scan_bwd_16bit_inputs(dtype, dout_float, dim, G):
+    print("CASE scan-bwd-16", dtype, dout_float, dim, G, flush=True)
+    u, delta, A, B, C, D, bias, dout = make(5, 2, dim, G, 1, 1200, dtype)
     dout = dout if dout_float else dout.to(dtype)
     want = torch_ref.selective_scan_grads(u.float(), delta.float(), A, B.float(), C.float(), D, bias, dout.float(), True)
     got = va.selective_scan_bwd(*[t.to(DEV) for t in (u, delta, A, B, C, D, bias, dout)], None, True, 1)

@@ -240,6 +240,196 @@ __global__ __launch_bounds__(kBlock) void scan_bwd_group_kernel(const ScanBwdArg
     }
 }
 
+// The same for ONE state per channel (the VMamba setting), pass-major: a wavefront walks its channels of the group
+// inside every pass, so the B / C items of the pass are loaded once for all of them and the channels' dB / dC
+// contributions are summed in registers first -- one LDS atomic per entry per wavefront and pass instead of one per
+// channel (LDS float atomics cost about ten plain LDS accesses here).  Per-channel state between passes (the state
+// entering each pass, the adjoint carry, the next pass's first a, the row sums) lives in a few floats of LDS per channel.
+template <typename in_t, typename dy_t, bool kSoftplus>
+__global__ __launch_bounds__(kBlock) void scan_bwd_group1_kernel(const ScanBwdArgs p, int chunk, int chunks_per_group, int n_groups) {
+    extern __shared__ __align__(16) float bwd_smem[];      // accB [L], accC [L], then the per-wavefront scratch
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int L = p.L, P = p.n_pass;
+    float *accB = bwd_smem, *accC = bwd_smem + L;
+    const int nc_max = (chunk + kWavesPerWg - 1) / kWavesPerWg;
+    float *h_in = accC + L + (size_t)wave * nc_max * (P + 5);        // [nc_max][P]: state entering each pass
+    float *g_carry = h_in + nc_max * P, *a_next = g_carry + nc_max;  // [nc_max] each
+    float *dA_s = a_next + nc_max, *dD_s = dA_s + nc_max, *db_s = dD_s + nc_max;
+    uint32_t wg = blockIdx.x;
+    const int ck = (int)(wg % chunks_per_group); wg /= chunks_per_group;
+    const int grp = (int)(wg % n_groups);
+    const int b = (int)(wg / n_groups);
+    for (int i = threadIdx.x; i < 2 * L; i += kBlock) bwd_smem[i] = 0.0f;
+    for (int i = lane; i < nc_max; i += kWave) {
+        h_in[i * P] = 0.0f; g_carry[i] = 0.0f; a_next[i] = 1.0f; dA_s[i] = 0.0f; dD_s[i] = 0.0f; db_s[i] = 0.0f;
+    }
+    __syncthreads();
+
+    const int c_first = ck * chunk + wave, c_end = min((ck + 1) * chunk, p.dim_per_group);
+    const int nc = c_first < c_end ? (c_end - c_first + kWavesPerWg - 1) / kWavesPerWg : 0;
+    const in_t *B_row = reinterpret_cast<const in_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
+    const in_t *C_row = reinterpret_cast<const in_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+    const bool vec = p.vec_ok != 0;
+    auto load8 = [&](const auto *rowp, int pos, float (&v)[kItems], float fill) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(rowp)>>;
+        if (vec) load_items<T, true>(rowp, pos, L, v, fill);
+        else load_items<T, false>(rowp, pos, L, v, fill);
+    };
+    struct Row {
+        const in_t *u, *dl;
+        const dy_t *dy;
+        in_t *du, *dd;
+        float A_log2e, An, Dv, bias;
+        int d;
+    };
+    auto row_of = [&](int i) {
+        Row r;
+        r.d = grp * p.dim_per_group + c_first + i * kWavesPerWg;
+        const int dg = r.d / p.dim_per_delta;
+        r.u = reinterpret_cast<const in_t *>(p.u) + b * p.u_bs + r.d * p.u_ds;
+        r.dl = reinterpret_cast<const in_t *>(p.delta) + b * p.dl_bs + dg * p.dl_ds;
+        r.dy = reinterpret_cast<const dy_t *>(p.dout) + b * p.do_bs + r.d * p.do_ds;
+        r.du = reinterpret_cast<in_t *>(p.du) + ((size_t)b * p.dim + r.d) * L;
+        r.dd = reinterpret_cast<in_t *>(p.ddelta) + ((size_t)b * p.dim + r.d) * L;
+        r.An = p.A[r.d * p.A_ds];
+        r.A_log2e = r.An * kLog2e;
+        r.Dv = p.D ? p.D[r.d] : 0.0f;
+        r.bias = p.bias ? p.bias[dg] : 0.0f;
+        return r;
+    };
+    auto load_dl_u = [&](const Row &r, int pos, float (&dl)[kItems], float (&uv)[kItems], float (&z)[kItems]) {
+        float raw[kItems], bias_items[kItems];
+        load8(r.dl, pos, raw, delta_fill<kSoftplus>());
+        load8(r.u, pos, uv, 0.0f);
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) { bias_items[i] = r.bias; z[i] = raw[i] + r.bias; }
+        delta_transform<kSoftplus>(raw, bias_items, dl);
+        if constexpr (!kSoftplus) {
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) dl[i] = pos + i < L ? dl[i] : 0.0f;
+        }
+    };
+
+    // ---- sweep 1: the state entering every pass, for every channel of this wavefront -------------------------------
+    for (int pass = 0; pass + 1 < P; ++pass) {
+        const int pos = pass * kPass + lane * kItems;
+        float Bv[kItems];
+        load8(B_row, pos, Bv, 0.0f);
+        for (int ci = 0; ci < nc; ++ci) {
+            const Row r = row_of(ci);
+            float dl[kItems], uv[kItems], z[kItems];
+            load_dl_u(r, pos, dl, uv, z);
+            float ac = 1.0f, hh = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const float a = __builtin_amdgcn_exp2f(dl[i] * r.A_log2e);
+                ac *= a;
+                hh = fmaf(a, hh, Bv[i] * (dl[i] * uv[i]));
+            }
+            float a_ex, h_ex, a_tot, h_tot;
+            wave_scan_pairs(ac, hh, a_ex, h_ex, a_tot, h_tot);
+            const float carry = h_in[ci * P + pass];
+            if (lane == 0) h_in[ci * P + pass + 1] = fmaf(a_tot, carry, h_tot);
+        }
+    }
+
+    // ---- sweep 2: passes in reverse, channels inside ------------------------------------------------------------------
+    for (int pass = P - 1; pass >= 0; --pass) {
+        const int pos = pass * kPass + lane * kItems;
+        float Bv[kItems], Cv[kItems], sumB[kItems], sumC[kItems];
+        load8(B_row, pos, Bv, 0.0f);
+        load8(C_row, pos, Cv, 0.0f);
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) { sumB[i] = 0.0f; sumC[i] = 0.0f; }
+        for (int ci = 0; ci < nc; ++ci) {
+            const Row r = row_of(ci);
+            float dl[kItems], uv[kItems], z[kItems], dy[kItems];
+            load_dl_u(r, pos, dl, uv, z);
+            load8(r.dy, pos, dy, 0.0f);
+            // forward inside the pass: a, and h at every position from the state entering the pass
+            float a[kItems], ac[kItems], hh[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                a[i] = __builtin_amdgcn_exp2f(dl[i] * r.A_log2e);
+                const float bb = Bv[i] * (dl[i] * uv[i]);
+                ac[i] = i == 0 ? a[i] : ac[i - 1] * a[i];
+                hh[i] = i == 0 ? bb : fmaf(a[i], hh[i - 1], bb);
+            }
+            float a_ex, h_ex, a_tot, h_tot;
+            wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+            const float s_in = fmaf(a_ex, h_in[ci * P + pass], h_ex);       // h just before this lane's first item
+            // reverse scan: g_t = C_t dy_t + a_t+1 g_t+1 (see scan_bwd_row)
+            float a_up = dpp_move<kDppWaveShl1>(0.0f, a[0]);
+            const float a_after = a_next[ci];
+            a_up = lane == kWave - 1 ? a_after : a_up;
+            float m[kItems], gl[kItems];
+#pragma unroll
+            for (int i = kItems - 1; i >= 0; --i) {
+                const float sh = i == kItems - 1 ? a_up : a[i + 1];
+                const float c = Cv[i] * dy[i];
+                m[i] = i == kItems - 1 ? sh : sh * m[i + 1];
+                gl[i] = i == kItems - 1 ? c : fmaf(sh, gl[i + 1], c);
+            }
+            float me, ge, mt, gt;
+            wave_scan_pairs(lane_reverse(m[0], lane), lane_reverse(gl[0], lane), me, ge, mt, gt);
+            const float gc = g_carry[ci];
+            const float G = lane_reverse(fmaf(me, gc, ge), lane);
+            if (lane == 0) { g_carry[ci] = fmaf(mt, gc, gt); a_next[ci] = a[0]; }
+
+            float dA_acc = 0.0f, dD_acc = 0.0f, db_acc = 0.0f, du[kItems], dd[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const float g = fmaf(m[i], G, gl[i]);
+                const float h = fmaf(ac[i], s_in, hh[i]);
+                const float h_prev = i == 0 ? s_in : fmaf(ac[i - 1], s_in, hh[i - 1]);
+                const float da_a = g * h_prev * a[i];                       // dL/da_t * a_t
+                const float d_dl = fmaf(da_a, r.An, g * (Bv[i] * uv[i]));
+                dA_acc = fmaf(da_a, dl[i], dA_acc);
+                dD_acc = fmaf(dy[i], uv[i], dD_acc);
+                du[i] = fmaf(g, dl[i] * Bv[i], dy[i] * r.Dv);
+                sumB[i] = fmaf(g, dl[i] * uv[i], sumB[i]);
+                sumC[i] = fmaf(dy[i], h, sumC[i]);
+                if constexpr (kSoftplus) {
+                    const float sg = z[i] > kSoftplusThreshold ? 1.0f : 1.0f / (1.0f + __expf(-z[i]));
+                    dd[i] = d_dl * sg;
+                } else {
+                    dd[i] = d_dl;
+                }
+                dd[i] = pos + i < L ? dd[i] : 0.0f;
+                db_acc += dd[i];
+            }
+            if (vec) { store_items<in_t, true>(r.du, pos, L, du); store_items<in_t, true>(r.dd, pos, L, dd); }
+            else { store_items<in_t, false>(r.du, pos, L, du); store_items<in_t, false>(r.dd, pos, L, dd); }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                dA_acc += __shfl_xor(dA_acc, off, kWave);
+                dD_acc += __shfl_xor(dD_acc, off, kWave);
+                db_acc += __shfl_xor(db_acc, off, kWave);
+            }
+            if (lane == 0) { dA_s[ci] += dA_acc; dD_s[ci] += dD_acc; db_s[ci] += db_acc; }
+        }
+#pragma unroll
+        for (int i = 0; i < kItems; ++i)
+            if (pos + i < L && nc > 0) {
+                __hip_atomic_fetch_add(accB + pos + i, sumB[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(accC + pos + i, sumC[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+    }
+    for (int ci = lane; ci < nc; ci += kWave) {
+        const int d = grp * p.dim_per_group + c_first + ci * kWavesPerWg;
+        unsafeAtomicAdd(p.dA + d, dA_s[ci]);
+        if (p.dD) unsafeAtomicAdd(p.dD + d, dD_s[ci]);
+        if (p.dbias) unsafeAtomicAdd(p.dbias + d, db_s[ci]);
+    }
+    __syncthreads();
+    float *dB_row = p.dB + b * p.g_bs + grp * p.g_gs, *dC_row = p.dC + b * p.g_bs + grp * p.g_gs;
+    for (int i = threadIdx.x; i < L; i += kBlock) {
+        unsafeAtomicAdd(dB_row + i, accB[i]);
+        unsafeAtomicAdd(dC_row + i, accC[i]);
+    }
+}
+
 }  // namespace ss2d
 
 extern "C" int ss2d_selective_scan_bwd(const ss2d_scan_bwd_params *q, void *stream) {
@@ -298,6 +488,21 @@ extern "C" int ss2d_selective_scan_bwd(const ss2d_scan_bwd_params *q, void *stre
         if (n <= 0x7fffffff) {
             const uint32_t n_wg_g = (uint32_t)n;
             const size_t smem_g = acc_bytes + smem;
+            if (a.N == 1) {
+                // one state: the pass-major kernel (channels inside the pass, dB / dC summed in registers first)
+                const int nc_max = (chunk + kWavesPerWg - 1) / kWavesPerWg;
+                const size_t smem_1 = acc_bytes + (size_t)kWavesPerWg * nc_max * (a.n_pass + 5) * sizeof(float);
+#define SS2D_BWD_GROUP1(IN, DY)                                                                                                 \
+    do {                                                                                                                        \
+        if (a.softplus) hipLaunchKernelGGL((scan_bwd_group1_kernel<IN, DY, true>), dim3(n_wg_g), dim3(kBlock), smem_1, s, a, chunk, cpg, q->n_groups); \
+        else hipLaunchKernelGGL((scan_bwd_group1_kernel<IN, DY, false>), dim3(n_wg_g), dim3(kBlock), smem_1, s, a, chunk, cpg, q->n_groups);          \
+    } while (0)
+                if (q->in_dtype == SS2D_F32) SS2D_BWD_GROUP1(float, float);
+                else if (q->in_dtype == SS2D_BF16) { if (q->dout_dtype == SS2D_F32) SS2D_BWD_GROUP1(bf16_t, float); else SS2D_BWD_GROUP1(bf16_t, bf16_t); }
+                else { if (q->dout_dtype == SS2D_F32) SS2D_BWD_GROUP1(f16_t, float); else SS2D_BWD_GROUP1(f16_t, f16_t); }
+#undef SS2D_BWD_GROUP1
+                return launch_status();
+            }
 #define SS2D_BWD_GROUP(IN, DY)                                                                                                  \
     do {                                                                                                                        \
         if (a.softplus) hipLaunchKernelGGL((scan_bwd_group_kernel<IN, DY, true>), dim3(n_wg_g), dim3(kBlock), smem_g, s, a, chunk, cpg, q->n_groups); \
