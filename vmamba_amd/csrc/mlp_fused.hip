@@ -3,7 +3,8 @@
 // in ONE kernel for the narrow stages (C = 96, 192), where the two library GEMMs, the GELU pass and the add are all
 // bound by the (M, 4C) hidden tensor going to HBM and back three times.  Here the hidden activations never leave the
 // registers:
-//   * a wavefront owns 32 (C = 192) or 64 (C = 96) positions and walks the hidden units in chunks of 32;
+//   * a wavefront owns 32 positions (kCT tiles of 32; measured at C = 96: one tile and three workgroups per CU beat
+//     two tiles and two workgroups) and walks the hidden units in chunks of 32;
 //   * GEMM 1 computes the chunk transposed, D1[hidden][position] = W1 chunk * x^T (v_mfma_f32_32x32x16, fp32
 //     accumulate).  In the MFMA output layout a lane holds, for its position, hidden units 8g + 4*(lane/32) + t
 //     (g, t = 0..3), accumulator 4g + t.  GEMM 2, D2[channel][position] += W2 chunk * h, contracts 16 hidden units per
@@ -12,7 +13,8 @@
 //     accumulators 8s .. 8s+7 (after bias, GELU and rounding to 16 bits) the B fragment of step s with no data
 //     movement between the two GEMMs.  The matching W2 fragment is two 8-byte runs of a row (one ds_read2_b64);
 //   * the W1 / W2 chunks (2 x 6..12 KB) go from global memory straight into LDS (global_load_lds_dwordx4, no
-//     registers in between), double-buffered, one barrier per chunk; x tiles come in and results go out through a wavefront-private LDS tile so that global loads and
+//     registers in between), double-buffered, one barrier per chunk, the next chunk in flight during the whole of
+//     the current one; x tiles come in and results go out through a wavefront-private LDS tile so that global loads and
 //     stores are 16 bytes per lane along the channel axis; the residual is added on the way out.
 // Rounding follows the unfused reference: fc1 output, GELU output and fc2 output are each rounded to the 16-bit type,
 // then the residual add is rounded once more.  GELU is the exact (erf) form:
@@ -55,6 +57,17 @@ __device__ __forceinline__ uint32_t gelu_pair(f16_t, uint32_t w, const float *) 
     return pack2_from_f32<f16_t>(gelu_erf(unpack_lo<f16_t>(w)), gelu_erf(unpack_hi<f16_t>(w)));
 }
 
+// One global_load_lds_dwordx4: every lane fetches 16 bytes from its own address, the wavefront's 1 KB lands at
+// lds_base + 16 * lane (lds_base wave-uniform).  Written as assembly so that the compiler does not order every later
+// LDS read behind the outstanding load (it cannot tell the double buffers apart and waits for vmcnt(0) at the first
+// LDS access after the issue, which puts the whole L2 latency on the critical path of every chunk); the waits are
+// placed by hand instead: wait_loads_to_lds() before the barrier that publishes a buffer.
+__device__ __forceinline__ void load_to_lds_16(const void *src, const void *lds_base) {
+    const uint32_t base = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void wait_loads_to_lds() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
+
 struct MlpArgs {
     const void *x, *ln_w, *ln_b, *w1, *b1, *w2, *b2, *residual;
     void *out;
@@ -72,7 +85,7 @@ template <typename T, int C> struct MlpLayout {
 };
 
 template <typename T, int C, int kCT, bool kLN>
-__global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
+__global__ __launch_bounds__(kBlock, (kCT == 1 && C == 96 ? 3 : 2)) void mlp_fused_kernel(const MlpArgs p) {
     using Lay = MlpLayout<T, C>;
     constexpr int kHidden = 4 * C;
     constexpr int kChunks = kHidden / kMlpChunk;
@@ -127,8 +140,7 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
             const int first = (it * kWaves + wave) * kWave;           // wave-uniform
             if (first + lane < kPiecesW) {
                 const T *src = w_second[it] ? w2 + w_off[it] + chunk * kMlpChunk : w1 + w_off[it] + (size_t)chunk * kMlpChunk * C;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                                 (__attribute__((address_space(3))) void *)(wbuf + buf * kBufElems + first * 8), 16, 0, 0);
+                load_to_lds_16(src, wbuf + buf * kBufElems + first * 8);
             }
         }
     };
@@ -206,6 +218,7 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
     }
     __syncthreads();                                                 // staging aliases the weight buffers
     fetch(0, 0);
+    wait_loads_to_lds();
     __syncthreads();
 
     floatx16_t acc2[kCT][kOG];
@@ -257,6 +270,7 @@ __global__ __launch_bounds__(kBlock, 2) void mlp_fused_kernel(const MlpArgs p) {
 #pragma unroll
                 for (int ct = 0; ct < kCT; ++ct) acc2[ct][og] = mfma_32x32x16(T{}, a, hf[ct][s], acc2[ct][og]);
             }
+        wait_loads_to_lds();                                         // the next chunk, in flight since the top of this one
         __syncthreads();
     }
 
@@ -329,6 +343,6 @@ extern "C" int ss2d_mlp_fused(const void *x, const void *ln_weight, const void *
     MlpArgs a;
     a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.eps = eps; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.residual = residual; a.out = out; a.M = M;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == SS2D_BF16) return C == 96 ? launch_mlp<bf16_t, 96, 2>(a, s) : launch_mlp<bf16_t, 192, 1>(a, s);
-    return C == 96 ? launch_mlp<f16_t, 96, 2>(a, s) : launch_mlp<f16_t, 192, 1>(a, s);
+    if (dtype == SS2D_BF16) return C == 96 ? launch_mlp<bf16_t, 96, 1>(a, s) : launch_mlp<bf16_t, 192, 1>(a, s);
+    return C == 96 ? launch_mlp<f16_t, 96, 1>(a, s) : launch_mlp<f16_t, 192, 1>(a, s);
 }
