@@ -164,6 +164,13 @@ int ss2d_selective_scan_bwd(const ss2d_scan_bwd_params *params, void *stream);
  */
 int ss2d_layer_norm(const void *x, const void *weight, const void *bias, void *y, int64_t rows, int C, float eps,
                     int in_dtype, int w_dtype, int out_dtype, void *stream);
+/*
+ * Residual add and LayerNorm in one pass: sum_out = x + residual (rounded to the input type, as the separate add of
+ * classification/models/vmamba.py:1228 would leave it), y = LayerNorm(sum_out) (:1229 norm2).  Same dtype triples as
+ * ss2d_layer_norm; rows must be vectorisable (C % 8 == 0, C <= 1024, 16-byte aligned pointers), else SS2D_ENOTSUP.
+ */
+int ss2d_add_layer_norm(const void *x, const void *residual, const void *weight, const void *bias, void *sum_out, void *y,
+                        int64_t rows, int C, float eps, int in_dtype, int w_dtype, int out_dtype, void *stream);
 int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void *y, int B, int C, int L, float eps,
                        int in_dtype, int w_dtype, int out_dtype, int out_channel_last, void *stream);
 

@@ -5,7 +5,9 @@ import pytest
 import torch
 
 from oracle import torch_ref
-from vmamba_amd.norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip, layer_norm_hip
+from vmamba_amd import _lib
+from vmamba_amd.norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip,
+                             layer_norm_hip)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -37,6 +39,35 @@ def test_layer_norm_rows(rows, C, in_dt, w_dt, out_dt):
     got = layer_norm_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_dtype=out_dt).cpu()
     assert got.dtype == want.dtype and got.shape == want.shape
     assert torch.allclose(got.float(), want.float(), **_tol(out_dt))
+
+
+@pytest.mark.parametrize("rows,C", [(1, 8), (401, 96), (77, 192), (128 * 196, 384), (33, 768), (9, 1024)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+def test_add_layer_norm_is_the_add_then_the_norm(rows, C, dt):
+    """sum bit-identical to the separate add (one rounding to the tensor type); the norm as the rows kernel's."""
+    print("CASE add-ln", rows, C, dt, flush=True)
+    g = torch.Generator().manual_seed(rows + C)
+    x = (torch.randn(rows, C, generator=g) * 2 + 0.5).to(dt)
+    r = torch.randn(rows, C, generator=g).to(dt)
+    w, b = (torch.randn(C, generator=g) + 1).to(dt), torch.randn(C, generator=g).to(dt)
+    total, normed = add_layer_norm_hip(_dev(x), _dev(r), _dev(w), _dev(b), 1e-6)
+    want_total = x + r
+    assert torch.equal(total.cpu(), want_total)
+    want = torch_ref.layer_norm_rows(want_total, w, b, 1e-6, dt)
+    assert torch.allclose(normed.cpu().float(), want.float(), **_tol(dt))
+    assert torch.equal(normed, layer_norm_hip(total, _dev(w), _dev(b), 1e-6))
+
+
+def test_add_layer_norm_rejections():
+    x = torch.randn(4, 100, device=DEV).bfloat16()          # C % 8 != 0: no fused kernel
+    assert not add_layer_norm_fusable(x, x)
+    with pytest.raises(_lib.Ss2dError):
+        add_layer_norm_hip(x, x, None, None)
+    with pytest.raises(ValueError):
+        add_layer_norm_hip(x, x[:2], None, None)
+    with pytest.raises(NotImplementedError):
+        add_layer_norm_hip(x.cpu(), x.cpu(), None, None)
+    assert _lib.lib().ss2d_add_layer_norm(x.data_ptr(), None, None, None, x.data_ptr(), x.data_ptr(), 4, 96, 1e-5, 1, 1, 1, None) == _lib.SS2D_EINVAL
 
 
 def test_layer_norm_rows_without_affine_and_known_answers():

@@ -37,6 +37,33 @@ def layer_norm_hip(x, weight, bias, eps=1e-5, out_dtype=None):
     return y
 
 
+def add_layer_norm_fusable(x, residual):
+    """True when ss2d_add_layer_norm takes these rows (vectorisable: C % 8 == 0, C <= 1024)."""
+    C = x.shape[-1]
+    return (x.is_cuda and x.dtype in _DTYPE_CODE and residual.dtype == x.dtype and residual.shape == x.shape
+            and C % 8 == 0 and C <= 1024)
+
+
+def add_layer_norm_hip(x, residual, weight, bias, eps=1e-5):
+    """(x + residual, LayerNorm(x + residual)) over the last axis in one pass; the sum is rounded to x.dtype first, as
+    the separate add would leave it."""
+    if not x.is_cuda:
+        raise NotImplementedError("add_layer_norm_hip: vmamba_amd runs on the GPU only")
+    if residual.shape != x.shape or residual.dtype != x.dtype:
+        raise ValueError("add_layer_norm_hip: residual must have the shape and dtype of x")
+    x, residual = x.contiguous(), residual.contiguous()
+    C = x.shape[-1]
+    weight, bias, wdt = _params(weight, bias)
+    total, y = torch.empty_like(x), torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_add_layer_norm(x.data_ptr(), residual.data_ptr(), weight.data_ptr() if weight is not None else None,
+                                            bias.data_ptr() if bias is not None else None, total.data_ptr(), y.data_ptr(),
+                                            x.numel() // max(C, 1), C, eps, _DTYPE_CODE[x.dtype], _DTYPE_CODE[wdt],
+                                            _DTYPE_CODE[y.dtype], torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_add_layer_norm")
+    return total, y
+
+
 def layer_norm_cf_hip(x, weight, bias, eps=1e-5, out_channel_last=False, out_dtype=None):
     """LayerNorm over axis 1 of a channel-first (B, C, *spatial) GPU tensor.
 

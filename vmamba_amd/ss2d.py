@@ -25,7 +25,8 @@ from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
 from .linear import linear_cl_hip, linear_fusable
-from .norm import LayerNorm, LayerNorm2d, layer_norm_cf_hip, needs_grad
+from .norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip,
+                   needs_grad)
 
 
 class Linear2d(nn.Linear):
@@ -189,16 +190,33 @@ class SS2D(nn.Module):
         """out_norm on the merged (B, D, L) map, in the block's layout (vmamba.py:641-646)."""
         return self.layers.out_norm(self.out_norm, y.view(B, D, H, W), self.channel_first, dtype)
 
+    def _forward_with_post_norm(self, x, residual, pre_norm, post_norm):
+        fuse = (residual is not None and not self.channel_first and isinstance(post_norm, nn.LayerNorm)
+                and post_norm.elementwise_affine and add_layer_norm_fusable(residual, residual)
+                and not self._narrow(residual, self.out_proj)
+                and not needs_grad(residual, self.out_proj.weight, self.out_proj.bias, post_norm.weight, post_norm.bias))
+        if not fuse:
+            total = self.forward(x, residual, pre_norm)
+            return total, post_norm(total)
+        proj = self.forward(x, None, pre_norm)
+        return add_layer_norm_hip(proj, residual, post_norm.weight, post_norm.bias, post_norm.eps)
+
     def _narrow(self, x, linear, *extra):
         """True when ss2d_linear_cl serves this projection: channel-last, 16-bit, width 96, no autograd."""
         return (not self.channel_first and isinstance(linear, nn.Linear) and not isinstance(linear, Linear2d)
                 and linear_fusable(x, linear.weight) and not needs_grad(x, linear.weight, linear.bias, *extra))
 
-    def forward(self, x, residual=None, pre_norm=None):
+    def forward(self, x, residual=None, pre_norm=None, post_norm=None):
         """``pre_norm``: the block's LayerNorm, applied to x first (vmamba.py:1227); ``residual`` (same layout as x) is
         added to the result (:1228).  A channel-last block of width 96 runs norm + in_proj and out_proj + add as one
         HIP kernel each (ss2d_linear_cl); otherwise channel-last blocks without an out_proj bias fold the addition
-        into the out_proj GEMM (one pass over the activation fewer than the block's separate add)."""
+        into the out_proj GEMM (one pass over the activation fewer than the block's separate add).
+
+        ``post_norm``: the block's second LayerNorm (:1229).  When given, the result is the pair
+        (sum, post_norm(sum)); in channel-last 16-bit inference the add and the LayerNorm are one kernel
+        (ss2d_add_layer_norm) behind a plain out_proj GEMM."""
+        if post_norm is not None:
+            return self._forward_with_post_norm(x, residual, pre_norm, post_norm)
         if (pre_norm is not None and isinstance(pre_norm, nn.LayerNorm) and pre_norm.elementwise_affine
                 and self._narrow(x, self.in_proj, pre_norm.weight, pre_norm.bias)):
             x = linear_cl_hip(x, self.in_proj.weight, self.in_proj.bias, None, pre_norm.weight, pre_norm.bias, pre_norm.eps)

@@ -49,6 +49,11 @@ class Mlp(nn.Module):
         self.act = nn.GELU()
         self.fc2 = Linear(hidden, dim)
 
+    def takes_norm(self, x):
+        """True when forward runs the fused kernel for x (which then takes the preceding LayerNorm as a prologue)."""
+        return (self.fused and not self.channel_first and mlp_fusable(x, self.fc1, self.fc2)
+                and not needs_grad(x, self.fc1.weight, self.fc2.weight, self.fc1.bias, self.fc2.bias))
+
     def forward(self, x, residual=None, pre_norm=None):
         """fc2(GELU(fc1(h))) (+ residual), h = x or pre_norm(x) (the block's second LayerNorm, vmamba.py:1229).
         Channel-last 16-bit inference at widths 96 / 192 runs as one HIP kernel that normalises the rows on the way
@@ -79,8 +84,11 @@ class VSSBlock(nn.Module):
         self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
     def forward(self, x):
-        x = self.op(x, residual=x, pre_norm=self.norm)
-        return self.mlp(x, residual=x, pre_norm=self.norm2)
+        if self.mlp.takes_norm(x):                    # the fused MLP kernel normalises its input itself
+            x = self.op(x, residual=x, pre_norm=self.norm)
+            return self.mlp(x, residual=x, pre_norm=self.norm2)
+        x, h = self.op(x, residual=x, pre_norm=self.norm, post_norm=self.norm2)
+        return self.mlp(h, residual=x)
 
 
 class VSSM(nn.Module):
