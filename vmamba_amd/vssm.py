@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 
 from .mlp import mlp_fusable, mlp_fused_hip
-from .norm import needs_grad
+from .norm import add_layer_norm_fusable, add_layer_norm_hip, needs_grad
 from .ss2d import SS2D, HipLayers, Linear2d
 
 
@@ -84,11 +84,44 @@ class VSSBlock(nn.Module):
         self.mlp = Mlp(dim, int(dim * mlp_ratio), channel_first)
 
     def forward(self, x):
+        x, pending = self.step(x, None)
+        return x if pending is None else x + pending
+
+    def step(self, x, pending):
+        """One block on the residual stream x, with ``pending`` (or None) a term the previous block has not added to x
+        yet; returns (x, pending) in the same sense.  Deferring the MLP's residual add lets the next block do it
+        together with its first LayerNorm in one kernel (ss2d_add_layer_norm); it is only deferred where that kernel
+        exists (channel-last 16-bit inference)."""
+        inp, pre = x, self.norm
+        if pending is not None:
+            if self._fusable_add_norm(x, pending, self.norm):
+                x, inp = add_layer_norm_hip(pending, x, self.norm.weight, self.norm.bias, self.norm.eps)
+                pre = None
+            else:
+                x = inp = x + pending
         if self.mlp.takes_norm(x):                    # the fused MLP kernel normalises its input itself
-            x = self.op(x, residual=x, pre_norm=self.norm)
-            return self.mlp(x, residual=x, pre_norm=self.norm2)
-        x, h = self.op(x, residual=x, pre_norm=self.norm, post_norm=self.norm2)
-        return self.mlp(h, residual=x)
+            x = self.op(inp, residual=x, pre_norm=pre)
+            return self.mlp(x, residual=x, pre_norm=self.norm2), None
+        x, h = self.op(inp, residual=x, pre_norm=pre, post_norm=self.norm2)
+        m = self.mlp(h)
+        if self._fusable_add_norm(x, m, self.norm):
+            return x, m
+        return x + m, None
+
+    def _fusable_add_norm(self, x, term, norm):
+        return (not self.op.channel_first and isinstance(norm, nn.LayerNorm) and norm.elementwise_affine
+                and add_layer_norm_fusable(x, term) and x.dtype != torch.float32
+                and not needs_grad(x, term, norm.weight, norm.bias))
+
+
+class BlockSequence(nn.Sequential):
+    """The blocks of one stage; threads the deferred residual term from block to block (see VSSBlock.step)."""
+
+    def forward(self, x):
+        pending = None
+        for block in self:
+            x, pending = block.step(x, pending)
+        return x if pending is None else x + pending
 
 
 class VSSM(nn.Module):
@@ -108,7 +141,7 @@ class VSSM(nn.Module):
             down = (nn.Sequential(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
                                   Norm(dims[i + 1]))
                     if i + 1 < len(dims) else nn.Identity())
-            stages.append(nn.Sequential(OrderedDict(blocks=nn.Sequential(*blocks), downsample=down)))
+            stages.append(nn.Sequential(OrderedDict(blocks=BlockSequence(*blocks), downsample=down)))
         self.layers = nn.ModuleList(stages)
         self.classifier = nn.Sequential(OrderedDict(
             norm=Norm(dims[-1]), permute=_to_cf(cf), avgpool=nn.AdaptiveAvgPool2d(1), flatten=nn.Flatten(1),
