@@ -93,6 +93,30 @@ def test_host_api_rejects_cpu_tensors_and_unsupported_modes():
         va.selective_scan_fn(u, u, torch.zeros(4, 1), torch.zeros(1, 4, 1, 8), torch.zeros(1, 4, 1, 8), backend="torch")
 
 
+def test_block_level_wrappers_have_no_cpu_path():
+    """The harness-side kernels (fused MLP, narrow projection, LayerNorm variants, depthwise conv, fused core) raise on
+    CPU tensors instead of computing anything there, and their 'fusable' predicates are False off the GPU."""
+    import torch
+    from vmamba_amd.conv import dwconv3x3_silu_hip
+    from vmamba_amd.core import dt_proj_hip, ss2d_core_hip
+    from vmamba_amd.linear import linear_cl_hip, linear_fusable
+    from vmamba_amd.mlp import mlp_fusable, mlp_fused_hip
+    from vmamba_amd.norm import add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip, layer_norm_hip
+    x = torch.zeros(4, 96, dtype=torch.bfloat16)
+    w1, w2, w = torch.zeros(384, 96, dtype=torch.bfloat16), torch.zeros(96, 384, dtype=torch.bfloat16), torch.zeros(96, 96, dtype=torch.bfloat16)
+    for call in (lambda: mlp_fused_hip(x, w1, None, w2, None), lambda: linear_cl_hip(x, w), lambda: layer_norm_hip(x, None, None),
+                 lambda: add_layer_norm_hip(x, x, None, None), lambda: layer_norm_cf_hip(torch.zeros(1, 8, 4), None, None),
+                 lambda: dwconv3x3_silu_hip(torch.zeros(1, 4, 4, 8), torch.zeros(8, 1, 3, 3), None, in_channel_last=True)):
+        with pytest.raises(NotImplementedError):
+            call()
+    with pytest.raises(RuntimeError):
+        ss2d_core_hip(torch.zeros(1, 2, 3, 3), torch.zeros(4, 2, 1, 9), torch.zeros(4, 1, 9), torch.zeros(4, 1, 9), torch.zeros(8))
+    with pytest.raises(RuntimeError):
+        dt_proj_hip(torch.zeros(4, 6, 8, dtype=torch.bfloat16), torch.zeros(4, 96, 6, dtype=torch.bfloat16))
+    lin1, lin2 = torch.nn.Linear(96, 384).bfloat16(), torch.nn.Linear(384, 96).bfloat16()
+    assert not mlp_fusable(x, lin1, lin2) and not linear_fusable(x, w) and not add_layer_norm_fusable(x, x)
+
+
 def test_torch_extension_shim_loads_and_validates_on_cpu():
     import torch
     from vmamba_amd import oflex_ext
