@@ -84,44 +84,7 @@ __global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
             }
             wave_lds_sync();
             if constexpr (kLN) {
-                // two lanes per row, each half of the channels; statistics meet through one lane exchange
-                constexpr int kHalf = K / 2, kVec = kHalf / 8;
-                static_assert(kHalf % 8 == 0, "whole 16-byte pieces per half row");
-                uint16_t *row = stage + j * PS + kh * kHalf;
-                float v[kHalf];
-                float sum = 0.0f;
-#pragma unroll
-                for (int i = 0; i < kVec; ++i) {
-                    const uint4 q4 = *reinterpret_cast<const uint4 *>(row + 8 * i);
-                    const uint32_t ww[4] = {q4.x, q4.y, q4.z, q4.w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[8 * i + 2 * e] = unpack_lo<T>(ww[e]);
-                        v[8 * i + 2 * e + 1] = unpack_hi<T>(ww[e]);
-                        sum += v[8 * i + 2 * e] + v[8 * i + 2 * e + 1];
-                    }
-                }
-                sum += __shfl_xor(sum, 32);
-                const float mean = sum * (1.0f / K);
-                float sq = 0.0f;
-#pragma unroll
-                for (int i = 0; i < kHalf; ++i) { const float c = v[i] - mean; sq = fmaf(c, c, sq); }
-                sq += __shfl_xor(sq, 32);
-                const float rstd = __builtin_amdgcn_rsqf(sq * (1.0f / K) + p.eps);
-#pragma unroll
-                for (int i = 0; i < kVec; ++i) {
-                    const uint4 g4 = *reinterpret_cast<const uint4 *>(gamma_l + kh * kHalf + 8 * i);
-                    const uint4 b4 = *reinterpret_cast<const uint4 *>(beta_l + kh * kHalf + 8 * i);
-                    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
-                    uint32_t ow[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float lo = fmaf((v[8 * i + 2 * e] - mean) * rstd, unpack_lo<T>(gw[e]), unpack_lo<T>(bw[e]));
-                        const float hi = fmaf((v[8 * i + 2 * e + 1] - mean) * rstd, unpack_hi<T>(gw[e]), unpack_hi<T>(bw[e]));
-                        ow[e] = pack2_from_f32<T>(lo, hi);
-                    }
-                    *reinterpret_cast<uint4 *>(row + 8 * i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
-                }
+                layer_norm_tile_rows<T, K>(stage, PS, lane, gamma_l, beta_l, p.eps);
                 wave_lds_sync();
             }
 #pragma unroll

@@ -143,6 +143,53 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// LayerNorm of the 32 rows of a wavefront-private LDS tile of 16-bit values, in place: row j (pitch `pitch` elements,
+// K channels) is normalised by lanes j and j + 32, each owning half of the channels; fp32 statistics with the centred
+// variance, result rounded to T.  gamma / beta: K 16-bit values each in LDS (16-byte aligned).  The caller brackets
+// the call with wave_lds_sync().
+template <typename T, int K>
+__device__ __forceinline__ void layer_norm_tile_rows(uint16_t *tile, int pitch, int lane, const uint16_t *gamma,
+                                                     const uint16_t *beta, float eps) {
+    constexpr int kHalf = K / 2, kVec = kHalf / 8;
+    static_assert(kHalf % 8 == 0, "whole 16-byte pieces per half row");
+    const int j = lane & 31, kh = lane >> 5;
+    uint16_t *row = tile + j * pitch + kh * kHalf;
+    float v[kHalf];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const uint4 q4 = *reinterpret_cast<const uint4 *>(row + 8 * i);
+        const uint32_t ww[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[8 * i + 2 * e] = unpack_lo<T>(ww[e]);
+            v[8 * i + 2 * e + 1] = unpack_hi<T>(ww[e]);
+            sum += v[8 * i + 2 * e] + v[8 * i + 2 * e + 1];
+        }
+    }
+    sum += __shfl_xor(sum, 32);
+    const float mean = sum * (1.0f / K);
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kHalf; ++i) { const float c = v[i] - mean; sq = fmaf(c, c, sq); }
+    sq += __shfl_xor(sq, 32);
+    const float rstd = __builtin_amdgcn_rsqf(sq * (1.0f / K) + eps);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const uint4 g4 = *reinterpret_cast<const uint4 *>(gamma + kh * kHalf + 8 * i);
+        const uint4 b4 = *reinterpret_cast<const uint4 *>(beta + kh * kHalf + 8 * i);
+        const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, bw[4] = {b4.x, b4.y, b4.z, b4.w};
+        uint32_t ow[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = fmaf((v[8 * i + 2 * e] - mean) * rstd, unpack_lo<T>(gw[e]), unpack_lo<T>(bw[e]));
+            const float hi = fmaf((v[8 * i + 2 * e + 1] - mean) * rstd, unpack_hi<T>(gw[e]), unpack_hi<T>(bw[e]));
+            ow[e] = pack2_from_f32<T>(lo, hi);
+        }
+        *reinterpret_cast<uint4 *>(row + 8 * i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+}
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? SS2D_OK : SS2D_ELAUNCH; }
 
 }  // namespace ss2d
