@@ -337,7 +337,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
                                f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}, {gemm_mode}; "
-                               f"SS2D core on HIP kernels"},
+                               f"SS2D core, LayerNorm, depthwise conv, narrow-stage MLP and projections on HIP kernels"},
         "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "kernels": kernels,
     }))
 
