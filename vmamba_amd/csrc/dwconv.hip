@@ -209,10 +209,11 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
                 for (int ci = 0; ci < 8; ++ci) acc[ci] = fmaf(wt[ci][kh * 3 + kw], xv[ci], acc[ci]);
             }
 #pragma unroll
-        for (int ci = 0; ci < 8; ++ci) {
-            T o = from_f32<T>(acc[ci] + bv[ci]);
-            if (kSilu) o = from_f32<T>(silu_fast(to_f32(o)));
-            out_tile[(cv * 8 + ci) * out_pitch + pidx] = o.bits;
+        for (int ci = 0; ci < 8; ci += 2) {
+            uint32_t o = pack2_from_f32<T>(acc[ci] + bv[ci], acc[ci + 1] + bv[ci + 1]);            // conv output as stored
+            if (kSilu) o = pack2_from_f32<T>(silu_fast(unpack_lo<T>(o)), silu_fast(unpack_hi<T>(o)));
+            out_tile[(cv * 8 + ci) * out_pitch + pidx] = (uint16_t)(o & 0xffffu);
+            out_tile[(cv * 8 + ci + 1) * out_pitch + pidx] = (uint16_t)(o >> 16);
         }
     }
     __syncthreads();
