@@ -274,8 +274,8 @@ def main():
                 import torch.cuda.tunable as tunable
                 tunable.enable(True)
                 tunable.tuning_enable(True)
-                for setter, value in (("set_filename", "/tmp/vmamba_amd_tunableop.csv"), ("set_max_tuning_duration", 30),
-                                      ("set_max_tuning_iterations", 20)):
+                for setter, value in (("set_filename", "/tmp/vmamba_amd_tunableop.csv"), ("set_max_tuning_duration", 60),
+                                      ("set_max_tuning_iterations", 60)):
                     if hasattr(tunable, setter):
                         getattr(tunable, setter)(value)
                 t_tune = time.perf_counter()
