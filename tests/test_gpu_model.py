@@ -101,6 +101,62 @@ def test_vmamba_tiny_logits_match_reference_core(channel_first):
     assert torch.allclose(got, want, rtol=2e-3, atol=2e-3)
 
 
+def test_vmamba_tiny_bf16_benchmark_layout_matches_fp32_reference():
+    """The benchmark's model at its own resolution: bf16, 224^2 (stage maps 56 / 28 / 14 / 7, so every stage takes the
+    kernels it takes in the benchmark -- the fused core with its per-stage tile choices, LayerNorm + MLP in one kernel
+    at widths 96 / 192, the narrow projections, add + LayerNorm between blocks).  Checked against the all-torch fp32
+    CPU model holding the same bf16-rounded weights, and against the channel-first bf16 model, which shares the
+    weights but none of the block-level kernels.  22 blocks of bf16 activations: the bound is the bf16 one (2e-2)
+    on the scale of the logits."""
+    print("CASE vssm-bf16-224", flush=True)
+    torch.manual_seed(14)
+    ref = reference_vmamba_tiny().eval().bfloat16().float()          # weights exactly representable in bf16
+    x = torch.randn(2, 3, 224, 224, generator=torch.Generator().manual_seed(15)).bfloat16()
+    with torch.no_grad():
+        want = ref(x.float())
+    scale = want.abs().max().item()
+    got = {}
+    for channel_first in (False, True):
+        hip = vmamba_tiny_s1l8(channel_first=channel_first).eval()
+        hip.load_state_dict(ref.state_dict())
+        hip = hip.bfloat16().to(DEV)
+        with torch.no_grad():
+            got[channel_first] = hip(x.to(DEV)).float().cpu()
+        err = (got[channel_first] - want).abs().max().item()
+        print(f"channel_first={channel_first}: max |logit error| {err:.3e} on a scale of {scale:.3e}", flush=True)
+        assert got[channel_first].shape == (2, 1000)
+        assert err <= 2e-2 * scale, f"channel_first={channel_first}"
+    assert (got[True] - got[False]).abs().max().item() <= 2e-2 * scale
+
+
+def test_vmamba_tiny_bf16_1024px_batch4():
+    """Benchmark config 4: the full backbone on a batch of four 1024^2 images in bf16.  Stage maps 256 / 128 / 64 / 32:
+    stages 1-2 (L = 65536, 16384) take the three separate operators -- the scan splits each row over the four
+    wavefronts of a workgroup and carries the state from 2048-chunk to chunk -- stages 3-4 the fused core.  One image
+    is checked against the all-torch fp32 CPU model (same bf16-rounded weights), all four between the channel-last
+    and the channel-first model."""
+    print("CASE vssm-bf16-1024", flush=True)
+    torch.manual_seed(16)
+    ref = reference_vmamba_tiny().eval().bfloat16().float()
+    x = torch.randn(4, 3, 1024, 1024, generator=torch.Generator().manual_seed(17)).bfloat16()
+    with torch.no_grad():
+        want = ref(x[3:4].float())
+    scale = want.abs().max().item()
+    got = {}
+    for channel_first in (False, True):
+        hip = vmamba_tiny_s1l8(channel_first=channel_first).eval()
+        hip.load_state_dict(ref.state_dict())
+        hip = hip.bfloat16().to(DEV)
+        with torch.no_grad():
+            got[channel_first] = hip(x.to(DEV)).float().cpu()
+        del hip
+        err = (got[channel_first][3:4] - want).abs().max().item()
+        print(f"channel_first={channel_first}: max |logit error| {err:.3e} on a scale of {scale:.3e}", flush=True)
+        assert got[channel_first].shape == (4, 1000) and torch.isfinite(got[channel_first]).all()
+        assert err <= 2e-2 * scale, f"channel_first={channel_first}"
+    assert (got[True] - got[False]).abs().max().item() <= 2e-2 * scale
+
+
 def test_small_vssm_trains_on_the_gpu():
     """One training step: gradients of a small model on the GPU (HIP scan / cross-scan / cross-merge backward, torch
     autograd for the rest) against the all-torch CPU model with the same weights."""
