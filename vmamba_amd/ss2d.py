@@ -149,6 +149,23 @@ class SS2D(nn.Module):
         dts = torch.bmm(consts["Wdt"], dts.reshape(B * K, R, L)).view(B, K * D, L)
         return dts, Bs, Cs
 
+    def project_from_map(self, x, consts):
+        """The same dts, B, C as ``project(cross_scan(x))`` from the map x (B, D, H, W) itself: a projection is a
+        per-position contraction, so x_proj is applied once to x in its natural order with the four directions' weights
+        stacked, and only its small output (R + 2N rows per direction instead of D) is put into scan order, each
+        direction's rows in that direction's order.  x_proj then reads the map once instead of its four copies."""
+        B, D, H, W = x.shape
+        K, L, R, N = self.k_group, H * W, self.dt_rank, self.d_state
+        proj = torch.bmm(consts["Wx_all"], x.reshape(B, D, L)).view(B, K, R + 2 * N, H, W)
+        x_dbl = cross_scan_fn(proj, in_channel_first=True, out_channel_first=True, one_by_one=True, scans=0)   # (B, K, R+2N, L)
+        dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
+        dts = dts.reshape(B * K, R, L)
+        if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK and not needs_grad(dts, self.dt_projs_weight):
+            dts = dt_proj_hip(dts, consts["Wdt"])                     # one (image, direction) problem per weight copy
+        else:
+            dts = torch.bmm(consts["Wdt"], dts)
+        return dts.view(B, K * D, L), Bs, Cs
+
     def forward_core_fused(self, x, consts):
         """One state per channel: the three operators as ONE kernel (ss2d_core_fwd).
 
@@ -180,7 +197,7 @@ class SS2D(nn.Module):
         if self.d_state == 1 and self.fused_core and not trains and core_fits(H, W, x.dtype):
             return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
-        dts, Bs, Cs = self.project(xs, consts)
+        dts, Bs, Cs = self.project_from_map(x, consts)
         ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
                                True, True)                                                     # fp32 (oflex)
         y = cross_merge_fn(ys.view(B, K, D, H, W), in_channel_first=True, out_channel_first=True, scans=0)
