@@ -171,6 +171,15 @@ int ss2d_layer_norm(const void *x, const void *weight, const void *bias, void *y
  */
 int ss2d_add_layer_norm(const void *x, const void *residual, const void *weight, const void *bias, void *sum_out, void *y,
                         int64_t rows, int C, float eps, int in_dtype, int w_dtype, int out_dtype, void *stream);
+/*
+ * Per-channel bias add and LayerNorm in one pass: y = LayerNorm(x + pre_bias), pre_bias (C) of the weight type, the sum
+ * rounded to the input type as a separate add would leave it.  Serves the convolution bias of the patch-embedding and
+ * downsampling layers, each a Conv2d directly followed by a LayerNorm (classification/models/vmamba.py:1403-1417,
+ * 1430-1437): the convolution then runs without its bias.  Same dtype triples and row conditions as
+ * ss2d_add_layer_norm.
+ */
+int ss2d_bias_layer_norm(const void *x, const void *pre_bias, const void *weight, const void *bias, void *y, int64_t rows,
+                         int C, float eps, int in_dtype, int w_dtype, int out_dtype, void *stream);
 int ss2d_layer_norm_cf(const void *x, const void *weight, const void *bias, void *y, int B, int C, int L, float eps,
                        int in_dtype, int w_dtype, int out_dtype, int out_channel_last, void *stream);
 

@@ -6,7 +6,8 @@ import torch
 
 from oracle import torch_ref
 from vmamba_amd import _lib
-from vmamba_amd.norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip,
+from vmamba_amd.norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, bias_layer_norm_fusable,
+                             bias_layer_norm_hip, layer_norm_cf_hip,
                              layer_norm_hip)
 
 pytestmark = pytest.mark.gpu
@@ -68,6 +69,34 @@ def test_add_layer_norm_rejections():
     with pytest.raises(NotImplementedError):
         add_layer_norm_hip(x.cpu(), x.cpu(), None, None)
     assert _lib.lib().ss2d_add_layer_norm(x.data_ptr(), None, None, None, x.data_ptr(), x.data_ptr(), 4, 96, 1e-5, 1, 1, 1, None) == _lib.SS2D_EINVAL
+
+
+@pytest.mark.parametrize("rows,C", [(3, 8), (500, 48), (401, 96), (77, 192), (50, 384), (33, 768), (9, 1024)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+def test_bias_layer_norm_is_the_add_then_the_norm(rows, C, dt):
+    """LayerNorm(x + per-channel bias) in one kernel: bit-identical to the rows kernel applied to the separately added
+    (and rounded) sum, and within tolerance of the torch reference."""
+    print("CASE bias-ln", rows, C, dt, flush=True)
+    g = torch.Generator().manual_seed(7 * rows + C)
+    x = (torch.randn(rows, C, generator=g) * 2 + 0.5).to(dt)
+    pb = torch.randn(C, generator=g).to(dt)
+    w, b = (torch.randn(C, generator=g) + 1).to(dt), torch.randn(C, generator=g).to(dt)
+    got = bias_layer_norm_hip(_dev(x), _dev(pb), _dev(w), _dev(b), 1e-6)
+    total = x + pb
+    assert torch.equal(got, layer_norm_hip(_dev(total), _dev(w), _dev(b), 1e-6))
+    assert torch.allclose(got.cpu().float(), torch_ref.layer_norm_rows(total, w, b, 1e-6, dt).float(), **_tol(dt))
+
+
+def test_bias_layer_norm_rejections():
+    x = torch.randn(4, 100, device=DEV).bfloat16()          # C % 8 != 0: no fused kernel
+    assert not bias_layer_norm_fusable(x.dtype, 100) and bias_layer_norm_fusable(x.dtype, 96)
+    with pytest.raises(_lib.Ss2dError):
+        bias_layer_norm_hip(x, x[0], None, None)
+    with pytest.raises(ValueError):
+        bias_layer_norm_hip(x, x[0, :50], None, None)
+    with pytest.raises(NotImplementedError):
+        bias_layer_norm_hip(x.cpu(), x[0].cpu(), None, None)
+    assert _lib.lib().ss2d_bias_layer_norm(x.data_ptr(), None, None, None, x.data_ptr(), 4, 96, 1e-5, 1, 1, 1, None) == _lib.SS2D_EINVAL
 
 
 def test_layer_norm_rows_without_affine_and_known_answers():

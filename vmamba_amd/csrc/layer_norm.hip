@@ -61,15 +61,24 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__r
                                                                  const w_t *__restrict__ bias, out_t *__restrict__ y,
                                                                  int64_t rows, int C, float eps,
                                                                  const in_t *__restrict__ residual = nullptr,
-                                                                 in_t *__restrict__ sum_out = nullptr) {
+                                                                 in_t *__restrict__ sum_out = nullptr,
+                                                                 const w_t *__restrict__ pre_bias = nullptr) {
     constexpr int kRowsPerBlock = kBlock / kGroup;
     const int g = threadIdx.x % kGroup;
     const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kGroup;
     const bool row_ok = row < rows;
     const in_t *xr = x + (row_ok ? row : 0) * C;
     float v[kChunks][kLnItems];
+    float pb[kChunks][kLnItems];
     bool have[kChunks];
     float s = 0.0f;
+    if (pre_bias) {                                  // requested ahead of the row so that the two loads overlap
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) {
+            const int c0 = (j * kGroup + g) * kLnItems;
+            if (c0 < C) ln_load8<w_t>(pre_bias + c0, pb[j]);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
         const int c0 = (j * kGroup + g) * kLnItems;
@@ -83,6 +92,11 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__r
 #pragma unroll
                 for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + r[i]));
                 ln_store8<in_t>(sum_out + row * C + c0, v[j]);
+            }
+            if (pre_bias) {
+                // the row is x + pre_bias (one value per channel), rounded as the separate add would leave it
+#pragma unroll
+                for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + pb[j][i]));
             }
         } else {
 #pragma unroll
@@ -421,13 +435,15 @@ static bool ln_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p)
 
 template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_rows(const void *x, const void *w, const void *b, void *y, int64_t rows, int C, float eps,
-                          hipStream_t stream, const void *residual = nullptr, void *sum_out = nullptr) {
+                          hipStream_t stream, const void *residual = nullptr, void *sum_out = nullptr,
+                          const void *pre_bias = nullptr) {
     const in_t *xp = (const in_t *)x; const w_t *wp = (const w_t *)w; const w_t *bp = (const w_t *)b; out_t *yp = (out_t *)y;
-    const in_t *rp = (const in_t *)residual; in_t *sp = (in_t *)sum_out;
+    const in_t *rp = (const in_t *)residual; in_t *sp = (in_t *)sum_out; const w_t *pp = (const w_t *)pre_bias;
     const bool fast = C % kLnItems == 0 && C <= kWave * kLnItems * kLnMaxChunks && ln_aligned16(x) && ln_aligned16(y) &&
-                      (!w || ln_aligned16(w)) && (!b || ln_aligned16(b)) && ln_aligned16(residual) && ln_aligned16(sum_out);
+                      (!w || ln_aligned16(w)) && (!b || ln_aligned16(b)) && ln_aligned16(residual) && ln_aligned16(sum_out) &&
+                      ln_aligned16(pre_bias);
     if (!fast) {
-        if (residual) return SS2D_ENOTSUP;          // the fused add exists for vectorisable rows only
+        if (residual || pre_bias) return SS2D_ENOTSUP;          // the fused adds exist for vectorisable rows only
         const int64_t n_wg = (rows + kBlock / kWave - 1) / (kBlock / kWave);
         if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
         hipLaunchKernelGGL((layer_norm_rows_generic_kernel<in_t, w_t, out_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
@@ -440,7 +456,7 @@ static int launch_ln_rows(const void *x, const void *w, const void *b, void *y, 
         const int64_t n_wg = (rows + kBlock / GROUP - 1) / (kBlock / GROUP);                                             \
         if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;                                                                      \
         hipLaunchKernelGGL((layer_norm_rows_kernel<in_t, w_t, out_t, GROUP, CHUNKS>), dim3((uint32_t)n_wg), dim3(kBlock), \
-                           0, stream, xp, wp, bp, yp, rows, C, eps, rp, sp);                                             \
+                           0, stream, xp, wp, bp, yp, rows, C, eps, rp, sp, pp);                                         \
     }
     if (vecs <= 4) SS2D_LN_LAUNCH(4, 1)
     else if (vecs <= 8) SS2D_LN_LAUNCH(8, 1)
@@ -574,6 +590,18 @@ extern "C" int ss2d_add_layer_norm(const void *x, const void *residual, const vo
     if (!x || !residual || !sum_out || !y) return SS2D_EINVAL;
     hipStream_t s = (hipStream_t)stream;
 #define SS2D_CALL(I, W, O) launch_ln_rows<I, W, O>(x, weight, bias, y, rows, C, eps, s, residual, sum_out)
+    SS2D_LN_DISPATCH(SS2D_CALL)
+#undef SS2D_CALL
+}
+
+extern "C" int ss2d_bias_layer_norm(const void *x, const void *pre_bias, const void *weight, const void *bias, void *y,
+                                    int64_t rows, int C, float eps, int in_dtype, int w_dtype, int out_dtype, void *stream) {
+    using namespace ss2d;
+    if (rows < 0 || C < 0 || !ln_dtype_ok(in_dtype) || !ln_dtype_ok(w_dtype) || !ln_dtype_ok(out_dtype)) return SS2D_EINVAL;
+    if (rows == 0 || C == 0) return SS2D_OK;
+    if (!x || !pre_bias || !y) return SS2D_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+#define SS2D_CALL(I, W, O) launch_ln_rows<I, W, O>(x, weight, bias, y, rows, C, eps, s, nullptr, nullptr, pre_bias)
     SS2D_LN_DISPATCH(SS2D_CALL)
 #undef SS2D_CALL
 }

@@ -64,6 +64,32 @@ def add_layer_norm_hip(x, residual, weight, bias, eps=1e-5):
     return total, y
 
 
+def bias_layer_norm_fusable(dtype, C):
+    """True when ss2d_bias_layer_norm takes rows of C channels of this dtype (vectorisable: C % 8 == 0, C <= 1024)."""
+    return dtype in _DTYPE_CODE and C % 8 == 0 and C <= 1024
+
+
+def bias_layer_norm_hip(x, pre_bias, weight, bias, eps=1e-5):
+    """LayerNorm(x + pre_bias) over the last axis in one pass, pre_bias one value per channel; the sum is rounded to
+    x.dtype first, as the separate add would leave it."""
+    if not x.is_cuda:
+        raise NotImplementedError("bias_layer_norm_hip: vmamba_amd runs on the GPU only")
+    C = x.shape[-1]
+    if pre_bias.shape != (C,):
+        raise ValueError("bias_layer_norm_hip: pre_bias must hold one value per channel")
+    x = x.contiguous()
+    weight, bias, wdt = _params(weight, bias)
+    pre_bias = pre_bias.to(wdt).contiguous()
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_bias_layer_norm(x.data_ptr(), pre_bias.data_ptr(), weight.data_ptr() if weight is not None else None,
+                                             bias.data_ptr() if bias is not None else None, y.data_ptr(),
+                                             x.numel() // max(C, 1), C, eps, _DTYPE_CODE[x.dtype], _DTYPE_CODE[wdt],
+                                             _DTYPE_CODE[y.dtype], torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_bias_layer_norm")
+    return y
+
+
 def layer_norm_cf_hip(x, weight, bias, eps=1e-5, out_channel_last=False, out_dtype=None):
     """LayerNorm over axis 1 of a channel-first (B, C, *spatial) GPU tensor.
 

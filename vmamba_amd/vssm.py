@@ -19,7 +19,8 @@ import torch
 import torch.nn as nn
 
 from .mlp import mlp_fusable, mlp_fused_hip
-from .norm import add_layer_norm_fusable, add_layer_norm_hip, needs_grad
+from .norm import LayerNorm as HipLayerNorm
+from .norm import add_layer_norm_fusable, add_layer_norm_hip, bias_layer_norm_fusable, bias_layer_norm_hip, needs_grad
 from .ss2d import SS2D, HipLayers, Linear2d
 
 
@@ -38,6 +39,34 @@ def _to_cl(channel_first):      # (B,C,H,W) -> block layout
 
 def _to_cf(channel_first):      # block layout -> (B,C,H,W)
     return nn.Identity() if channel_first else Permute(0, 3, 1, 2)
+
+
+class ConvNormSequence(nn.Sequential):
+    """The patch-embedding and downsampling stacks (vmamba.py:1403-1417, 1430-1437).  Where a Conv2d with a bias is
+    followed by the permute to channel-last and this package's LayerNorm, the convolution runs without its bias and
+    the LayerNorm kernel adds it on the way in (ss2d_bias_layer_norm): one pass over the activation fewer."""
+
+    def forward(self, x):
+        mods = list(self)
+        i = 0
+        while i < len(mods):
+            conv = mods[i]
+            if i + 2 < len(mods) and self._fusable(x, conv, mods[i + 1], mods[i + 2]):
+                norm = mods[i + 2]
+                x = conv._conv_forward(x, conv.weight, None).permute(0, 2, 3, 1)
+                x = bias_layer_norm_hip(x, conv.bias, norm.weight, norm.bias, norm.eps)
+                i += 3
+            else:
+                x = conv(x)
+                i += 1
+        return x
+
+    @staticmethod
+    def _fusable(x, conv, permute, norm):
+        return (isinstance(conv, nn.Conv2d) and conv.bias is not None and isinstance(permute, Permute)
+                and tuple(permute.dims) == (0, 2, 3, 1) and isinstance(norm, HipLayerNorm) and norm.elementwise_affine
+                and x.is_cuda and x.dim() == 4 and bias_layer_norm_fusable(x.dtype, conv.out_channels)
+                and not needs_grad(x, conv.weight, conv.bias, norm.weight, norm.bias))
 
 
 class Mlp(nn.Module):
@@ -131,14 +160,14 @@ class VSSM(nn.Module):
         cf = channel_first
         Norm = layers.LayerNorm2d if cf else layers.LayerNorm
         d0 = dims[0]
-        self.patch_embed = nn.Sequential(
+        self.patch_embed = ConvNormSequence(
             nn.Conv2d(in_chans, d0 // 2, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0 // 2), _to_cf(cf),
             nn.GELU(),
             nn.Conv2d(d0 // 2, d0, kernel_size=3, stride=2, padding=1), _to_cl(cf), Norm(d0))
         stages = []
         for i, (depth, dim) in enumerate(zip(depths, dims)):
             blocks = [VSSBlock(dim, d_state, ssm_ratio, mlp_ratio, ss2d_cls, cf, layers, **ss2d_kwargs) for _ in range(depth)]
-            down = (nn.Sequential(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
+            down = (ConvNormSequence(_to_cf(cf), nn.Conv2d(dim, dims[i + 1], kernel_size=3, stride=2, padding=1), _to_cl(cf),
                                   Norm(dims[i + 1]))
                     if i + 1 < len(dims) else nn.Identity())
             stages.append(nn.Sequential(OrderedDict(blocks=BlockSequence(*blocks), downsample=down)))
