@@ -7,10 +7,12 @@
 //   * one MFMA tile = 32 positions x 32 channels x 8 ranks (v_mfma_f32_32x32x8, bf16 or f16 operands, fp32
 //     accumulate -- the arithmetic of the library GEMM it replaces: products of 16-bit values summed in fp32,
 //     one rounding to the 16-bit output);
-//   * a wavefront owns blocks of 128 consecutive positions.  The x rows of a block are fetched with 16-byte loads
-//     into a wavefront-private LDS tile and read back as MFMA fragments; the results of four tiles (128 positions
-//     x 32 channels) are parked in a second private LDS tile and written out as 16 bytes per lane, four channels x
-//     256 contiguous bytes per store instruction;
+//   * a wavefront owns blocks of 64 consecutive positions.  The x rows of a block are fetched with 16-byte loads
+//     into a wavefront-private LDS tile and read back as MFMA fragments; the results of two tiles (64 positions
+//     x 32 channels) are parked in a second private LDS tile and written out as 16 bytes per lane, eight channels x
+//     128 contiguous bytes per store instruction.  (Blocks of 128 positions -- 256-byte runs -- were slower at every
+//     stage shape: the LDS tiles bound the resident wavefronts, and it is their number that hides each one's
+//     load -> MFMA -> store latency.)
 //   * the MFMA row index is mapped to positions through a permutation chosen so that a lane's 16 accumulators are
 //     16 consecutive positions of one channel (two 16-byte LDS writes);
 //   * the W fragments of up to 96 channels stay in registers for all blocks of the wavefront.
@@ -19,8 +21,10 @@
 namespace ss2d {
 
 constexpr int kDtTile = 32;          // positions (and channels) per MFMA tile
-constexpr int kDtBlock = 128;        // positions per block: four tiles
-constexpr int kDtPitch = kDtBlock + 8;   // LDS row pitch in elements (272 bytes: 16-byte aligned, banks spread)
+constexpr int kDtTiles = 2;          // MFMA tiles per block
+constexpr int kDtBlock = kDtTiles * kDtTile;   // positions per block
+constexpr int kDtPitch = kDtBlock + 8;   // LDS row pitch in elements (144 bytes: 16-byte aligned, banks spread)
+constexpr int kDtPieces = kDtBlock / 8;  // 16-byte pieces per row of a block
 constexpr int kDtGroups = 3;         // channel groups of 32 per wavefront
 constexpr int kDtMaxRank = 48;
 constexpr uint32_t kDtOutOfRange = 0x7ffffff0u;   // byte offset beyond any buffer here (spans are checked < 2^31 - 16)
@@ -36,6 +40,7 @@ struct DtArgs {
 template <typename T, int kSteps>
 __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
     extern __shared__ __align__(16) uint16_t dt_smem[];
+    constexpr int kTiles = kDtTiles, kPieces = kDtPieces;
     constexpr int kRows = 8 * kSteps;                         // x rows held in LDS (rows >= R stay zero)
     constexpr int kWaveLds = (kRows + kDtTile) * kDtPitch;    // elements per wavefront: x tile + output tile
     const int lane = threadIdx.x & (kWave - 1);
@@ -95,9 +100,9 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
     const int64_t block1 = block0 + p.blocks_per_wave < p.n_blocks ? block0 + p.blocks_per_wave : p.n_blocks;
     for (int64_t blk = block0; blk < block1; ++blk) {
         const int64_t n0 = blk * kDtBlock;
-        // ---- x rows of the block -> LDS: 16 lanes x 16 bytes per row
-        for (int idx = lane; idx < p.R * 16; idx += kWave) {
-            const int r = idx >> 4, c = idx & 15;
+        // ---- x rows of the block -> LDS: kPieces lanes x 16 bytes per row
+        for (int idx = lane; idx < p.R * kPieces; idx += kWave) {
+            const int r = idx / kPieces, c = idx % kPieces;
             const int64_t n = n0 + 8 * c;
             uint4 v;
             if (p.vec_ok) {
@@ -119,10 +124,10 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
             *reinterpret_cast<uint4 *>(xs + r * kDtPitch + 8 * c) = v;
         }
         wave_lds_sync();
-        // ---- x fragments of the four tiles (MFMA rows = positions)
-        uint32_t xf[4][kSteps][2];
+        // ---- x fragments of the tiles (MFMA rows = positions)
+        uint32_t xf[kTiles][kSteps][2];
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < kTiles; ++t)
 #pragma unroll
             for (int s = 0; s < kSteps; ++s) {
                 const uint16_t *src = xs + (8 * s + 4 * kh) * kDtPitch + t * kDtTile + p_in;
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
         for (int g = 0; g < kDtGroups; ++g) {
             if (d_base + g * kDtTile < p.D) {                         // uniform over the wavefront
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
+                for (int t = 0; t < kTiles; ++t) {
                     floatx16_t acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                     for (int s = 0; s < kSteps; ++s) acc = mfma_32x32x8(T{}, xf[t][s], wf[g][s], acc);
@@ -147,10 +152,11 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
                     dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
                 }
                 wave_lds_sync();
-                // ---- 32 channels x 128 positions out: lane -> (channel lane/16 + 4*it, 16-byte piece lane%16)
+                // ---- 32 channels x kDtBlock positions out: lane -> (channel lane/kPieces + .., 16-byte piece lane%kPieces)
+                constexpr int kChPerStore = kWave / kPieces;
 #pragma unroll
-                for (int it = 0; it < 8; ++it) {
-                    const int ch = (lane >> 4) + 4 * it, c = lane & 15;
+                for (int it = 0; it < kDtTile / kChPerStore; ++it) {
+                    const int ch = lane / kPieces + kChPerStore * it, c = lane % kPieces;
                     const int d = d_base + g * kDtTile + ch;
                     const int64_t n = n0 + 8 * c;
                     const uint4 v = *reinterpret_cast<const uint4 *>(ob + ch * kDtPitch + 8 * c);
