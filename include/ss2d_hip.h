@@ -267,6 +267,19 @@ int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H, int W, in
 int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, int elem_bytes, void *stream);
 
 /*
+ * First layer of the patch embedding in one pass (classification/models/vmamba.py:1403-1411, patch-embed v2:
+ * Conv2d(3, Cout, kernel 3, stride 2, padding 1) -> permute -> LayerNorm(Cout) -> permute -> GELU):
+ *   y = GELU(LayerNorm(conv2d(x, weight, bias))), exact (erf) GELU, the three results rounded to dtype in turn.
+ *   x (B, 3, H, W) contiguous; weight (Cout, 3, 3, 3) taken through weight_strides[4] (elements: out channel, in
+ *   channel, tap row, tap column -- contiguous or channels-last weights alike); bias, ln_weight, ln_bias (Cout) or
+ *   NULL; y (B, Ho, Wo, Cout) contiguous, channel-last, Ho = (H - 1)/2 + 1, Wo = (W - 1)/2 + 1.
+ * dtype SS2D_BF16 or SS2D_F16 for all tensors, Cout 48 or 64; anything else returns SS2D_ENOTSUP.
+ */
+int ss2d_stem_conv_ln_gelu(const void *x, const void *weight, const int64_t *weight_strides, const void *bias,
+                           const void *ln_weight, const void *ln_bias, float eps, void *y, int B, int H, int W, int Cout,
+                           int dtype, void *stream);
+
+/*
  * dt_proj of the SS2D core: the per-direction rank-R -> D projection between x_proj and the scan.
  * Replaces the grouped conv1d / einsum of SS2Dv2.forward_corev2 (classification/models/vmamba.py:608-609, 614-615):
  *   delta[k, d, n] = sum_r weight[k, d, r] * x[k*x_dir_stride + r*x_rank_stride + n]

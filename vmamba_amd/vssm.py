@@ -22,6 +22,7 @@ from .mlp import mlp_fusable, mlp_fused_hip
 from .norm import LayerNorm as HipLayerNorm
 from .norm import add_layer_norm_fusable, add_layer_norm_hip, bias_layer_norm_fusable, bias_layer_norm_hip, needs_grad
 from .ss2d import SS2D, HipLayers, Linear2d
+from .stem import stem_conv_ln_gelu_hip, stem_fusable
 
 
 class Permute(nn.Module):
@@ -51,7 +52,11 @@ class ConvNormSequence(nn.Sequential):
         i = 0
         while i < len(mods):
             conv = mods[i]
-            if i + 2 < len(mods) and self._fusable(x, conv, mods[i + 1], mods[i + 2]):
+            if i + 4 < len(mods) and self._stem(x, conv, *mods[i + 1:i + 5]):
+                norm = mods[i + 2]                    # conv, LayerNorm and GELU in one kernel; the result is channel-last
+                x = stem_conv_ln_gelu_hip(x, conv.weight, conv.bias, norm.weight, norm.bias, norm.eps).permute(0, 3, 1, 2)
+                i += 5
+            elif i + 2 < len(mods) and self._fusable(x, conv, mods[i + 1], mods[i + 2]):
                 norm = mods[i + 2]
                 x = conv._conv_forward(x, conv.weight, None).permute(0, 2, 3, 1)
                 x = bias_layer_norm_hip(x, conv.bias, norm.weight, norm.bias, norm.eps)
@@ -60,6 +65,13 @@ class ConvNormSequence(nn.Sequential):
                 x = conv(x)
                 i += 1
         return x
+
+    @staticmethod
+    def _stem(x, conv, to_cl, norm, to_cf, act):
+        return (isinstance(conv, nn.Conv2d) and isinstance(to_cl, Permute) and tuple(to_cl.dims) == (0, 2, 3, 1)
+                and isinstance(norm, HipLayerNorm) and isinstance(to_cf, Permute) and tuple(to_cf.dims) == (0, 3, 1, 2)
+                and isinstance(act, nn.GELU) and stem_fusable(x, conv, norm, act)
+                and not needs_grad(x, conv.weight, conv.bias, norm.weight, norm.bias))
 
     @staticmethod
     def _fusable(x, conv, permute, norm):
