@@ -118,12 +118,15 @@ __global__ __launch_bounds__(kBlock) void stem_conv_ln_gelu_kernel(const StemArg
             const int c = k / 9, t = k - 9 * c, th = t / 3, tw = t - 3 * th;
             koff[s][e] = k < kStemTaps ? (c * rows_in + th) * Wp + tw : -1;
         }
-    // this lane's channels: value i < 16 is channel 8 (i/4) + 4 kh + i%4, value 16 + i is channel 32 + 8 (i/4) + 4 kh + i%4
-    float bias_v[kPerLane], gamma_v[kPerLane], beta_v[kPerLane];
+    // this lane's channels: value i < 16 is channel 8 (i/4) + 4 kh + i%4, value 16 + i is channel 32 + 8 (i/4) + 4 kh + i%4.
+    // The bias rides in as the accumulators' initial value.
+    floatx16_t bias_acc[2];
+    float gamma_v[kPerLane], beta_v[kPerLane];
 #pragma unroll
-    for (int i = 0; i < kPerLane; ++i) {
+    for (int i = 0; i < 32; ++i) {
         const int ch = (i < 16 ? 0 : 32) + 8 * ((i & 15) / 4) + 4 * kh + (i & 3);
-        bias_v[i] = prm[ch]; gamma_v[i] = prm[kCout + ch]; beta_v[i] = prm[2 * kCout + ch];
+        bias_acc[i / 16][i & 15] = ch < kCout ? prm[ch] : 0.0f;
+        if (i < kPerLane) { gamma_v[i] = prm[kCout + ch]; beta_v[i] = prm[2 * kCout + ch]; }
     }
 
     T *y = reinterpret_cast<T *>(p.y);
@@ -136,25 +139,22 @@ __global__ __launch_bounds__(kBlock) void stem_conv_ln_gelu_kernel(const StemArg
         const int base = (2 * (int)rl) * Wp + 2 * (int)ow + kStemPad - 1;        // the patch's first element (tap 0,0 of channel 0)
         floatx16_t acc[2];
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mt][v] = 0.0f;
-#pragma unroll
         for (int s = 0; s < 2; ++s) {
             uint32_t e[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) e[q] = in_tile[koff[s][q] < 0 ? n_in : base + koff[s][q]];
             const u32x4_t xf = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) acc[mt] = mfma_32x32x16(T{}, wf[mt][s], xf, acc[mt]);
+            for (int mt = 0; mt < 2; ++mt) acc[mt] = mfma_32x32x16(T{}, wf[mt][s], xf, s == 0 ? bias_acc[mt] : acc[mt]);
         }
-        // convolution output as stored (+ bias, rounded), LayerNorm over the position's kCout channels
+        // convolution output as stored (bias included, rounded), LayerNorm over the position's kCout channels
         float v[kPerLane];
         float sum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kPerLane; ++i) {
-            v[i] = to_f32(from_f32<T>((i < 16 ? acc[0][i] : acc[1][i - 16]) + bias_v[i]));
-            sum += v[i];
+        for (int i = 0; i < kPerLane; i += 2) {
+            const uint32_t w2 = pack2_from_f32<T>(i < 16 ? acc[0][i] : acc[1][i - 16], i < 16 ? acc[0][i + 1] : acc[1][i - 15]);
+            v[i] = unpack_lo<T>(w2); v[i + 1] = unpack_hi<T>(w2);
+            sum += v[i] + v[i + 1];
         }
         sum += __shfl_xor(sum, 32);
         const float mean = sum * (1.0f / kCout);
