@@ -129,6 +129,17 @@ def kernel_lines(reps):
                 fused.update(ln_in_proj_us=t_i * 1e6, ln_in_proj_GBs=2 * M * D * 2 / t_i / 1e9,
                              out_proj_add_us=t_o * 1e6, out_proj_add_GBs=3 * M * D * 2 / t_o / 1e9)
             del xa, w1, w2, wp
+            if name == "stage1":
+                # the patch embedding's first layer (conv 3x3 stride 2 + LayerNorm + GELU in one kernel): the image
+                # batch in, the (B, 112, 112, 48) activation out
+                from vmamba_amd.stem import stem_conv_ln_gelu_hip
+                img = torch.randn(B, 3, 4 * H, 4 * W, device=dev, generator=g).bfloat16()
+                wc = (torch.randn(48, 3, 3, 3, device=dev, generator=g) * 0.2).bfloat16()
+                v48 = torch.ones(48, device=dev).bfloat16()
+                t_s = time_op(lambda: stem_conv_ln_gelu_hip(img, wc, v48, v48, v48, 1e-5), reps)
+                b_s = img.numel() * 2 + B * (2 * H) * (2 * W) * 48 * 2
+                fused.update(stem_us=t_s * 1e6, stem_GBs=b_s / t_s / 1e9)
+                del img
         out.append(dict(shape=name, B=B, D=D, H=H, W=W, N=N,
                         cross_scan_us=t_cs * 1e6, cross_scan_GBs=b_cs / t_cs / 1e9,
                         scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9,
@@ -339,7 +350,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
                                f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}, {gemm_mode}; "
-                               f"SS2D core, LayerNorm, depthwise conv, narrow-stage MLP and projections on HIP kernels"},
+                               f"SS2D core, LayerNorm, depthwise conv, patch-embedding stem, narrow-stage MLP and projections on HIP kernels"},
         "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "kernels": kernels,
     }))
 
