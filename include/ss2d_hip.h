@@ -319,6 +319,16 @@ int ss2d_mlp_fused(const void *x, const void *ln_weight, const void *ln_bias, fl
 int ss2d_linear_cl(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
                    const void *bias, const void *residual, void *out, int64_t M, int K, int N, int dtype, void *stream);
 
+/*
+ * The same projection fed by the SS2D core: x is the fp32 channel-first map (B, K, L) that ss2d_core_fwd (or
+ * CrossMerge) leaves, the LayerNorm is the block's out_norm over the K channels of each position, computed from the
+ * fp32 values and rounded to dtype as the separate operator does (classification/models/vmamba.py:641-646), and
+ * out (B*L, N) = out_norm(x) weight^T + bias + residual is the block's out_proj with its residual add (:662, :1228).
+ * dtype (weights, residual, out) SS2D_BF16 or SS2D_F16; K = N = 96 and L a multiple of 32, else SS2D_ENOTSUP.
+ */
+int ss2d_linear_cf_ln(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
+                      const void *bias, const void *residual, void *out, int B, int L, int K, int N, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,3 +77,43 @@ def test_linear_cl_rejections():
     assert L.ss2d_linear_cl(None, None, None, 1e-5, None, None, None, None, 8, 96, 96, _lib.SS2D_BF16, None) == _lib.SS2D_EINVAL
     assert L.ss2d_linear_cl(x.data_ptr(), None, gamma.data_ptr(), 1e-5, w.data_ptr(), None, None, x.data_ptr(), 8, 96, 96,
                             _lib.SS2D_BF16, None) == _lib.SS2D_EINVAL          # LayerNorm bias without weight
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("B,L", [(1, 32), (3, 64), (2, 3136), (5, 96)])
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_linear_cf_ln_matches_out_norm_then_out_proj(B, L, dtype, with_residual):
+    """out_norm over the channels of the fp32 channel-first map (fp32 statistics, result rounded to the 16-bit type), then
+    the projection (+ bias, rounded) and the residual add (rounded): the separate operators on the CPU in fp32."""
+    from vmamba_amd.linear import linear_cf_ln_hip
+    print("CASE linear_cf_ln", B, L, dtype, with_residual, flush=True)
+    K = N = 96
+    g = torch.Generator().manual_seed(B * 7 + L)
+    y = torch.randn(B, K, L, generator=g) * 2 + 0.3
+    gamma, beta = (torch.randn(K, generator=g) * 0.3 + 1).to(dtype), (torch.randn(K, generator=g) * 0.3).to(dtype)
+    w, bias = (torch.randn(N, K, generator=g) * K ** -0.5).to(dtype), (torch.randn(N, generator=g) * 0.1).to(dtype)
+    res = torch.randn(B, L, N, generator=g).to(dtype) if with_residual else None
+    r = lambda t: t.to(dtype).float()
+    normed = r(torch.nn.functional.layer_norm(y.permute(0, 2, 1), (K,), gamma.float(), beta.float(), 1e-5))
+    want = r(normed @ w.float().t() + bias.float())
+    if with_residual:
+        want = r(want + res.float())
+    dev = lambda t: None if t is None else t.to(DEV)
+    got = linear_cf_ln_hip(dev(y), dev(gamma), dev(beta), 1e-5, dev(w), dev(bias), dev(res))
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == (B, L, N)
+    assert torch.allclose(got.cpu().float(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_linear_cf_ln_rejections():
+    from vmamba_amd.linear import linear_cf_ln_fusable, linear_cf_ln_hip
+    w = torch.zeros(96, 96, device=DEV, dtype=torch.bfloat16)
+    assert linear_cf_ln_fusable(96, w, 64) and not linear_cf_ln_fusable(96, w, 49) and not linear_cf_ln_fusable(96, w.float(), 64)
+    with pytest.raises(_lib.Ss2dError) as e:
+        linear_cf_ln_hip(torch.zeros(1, 96, 49, device=DEV), w[0], None, 1e-5, w)                       # L % 32 != 0
+    assert e.value.code == _lib.SS2D_ENOTSUP
+    with pytest.raises(TypeError):
+        linear_cf_ln_hip(torch.zeros(1, 96, 64, device=DEV, dtype=torch.bfloat16), w[0], None, 1e-5, w)  # the map must be fp32
+    with pytest.raises(ValueError):
+        linear_cf_ln_hip(torch.zeros(1, 96, 64, device=DEV), None, None, 1e-5, w)
+    assert linear_cf_ln_hip(torch.zeros(0, 96, 64, device=DEV), w[0], None, 1e-5, w).shape == (0, 64, 96)

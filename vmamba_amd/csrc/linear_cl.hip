@@ -19,10 +19,15 @@ struct LinArgs {
     int64_t M;
     float eps;
     int tiles_per_wg;
+    int L;                  // kCfIn: positions per image (a multiple of 32)
 };
 
-template <typename T, int K, int N, int kCT, bool kLN>
+// kCfIn: x is the fp32 channel-first map (B, K, L) -- the merged output of the SS2D core -- and the LayerNorm (the
+// block's out_norm, classification/models/vmamba.py:641-646) is computed from the fp32 values, as the separate
+// operator does, before its result is rounded to T and multiplied.
+template <typename T, int K, int N, int kCT, bool kLN, bool kCfIn = false>
 __global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
+    static_assert(!kCfIn || (kLN && K % 8 == 0), "the channel-first input path normalises");
     constexpr int kSteps = K / 16;                  // k-steps of the contraction
     constexpr int kOG = N / 32;                     // output-channel groups
     constexpr int PK = K + 8;                       // weight row pitch (elements): 16-byte rows, banks spread
@@ -74,18 +79,62 @@ __global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
         u32x4_t xf[kCT][kSteps];
 #pragma unroll
         for (int ct = 0; ct < kCT; ++ct) {
+            if constexpr (kCfIn) {
+                // 32 positions of one image (L % 32 == 0, M % 32 == 0): lane (channel group cs = lane / 8, quad = lane % 8)
+                // loads positions 4 quad .. + 3 of channels cs, cs + 8, ..., 16 bytes each
+                constexpr int kCPL = K / 8;
+                const int64_t tpos = pos0 + ct * 32;
+                const int64_t tb = (tpos < p.M ? tpos : 0) / p.L;
+                const int l0 = (int)((tpos < p.M ? tpos : 0) - tb * p.L);
+                const int cs = lane >> 3, quad = lane & 7;
+                const float *src = reinterpret_cast<const float *>(p.x) + ((size_t)tb * K + cs) * p.L + l0 + 4 * quad;
+                float4 v[kCPL];
+                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int it = 0; it < kPiecesIn / kWave; ++it) {
-                const int idx = lane + it * kWave;
-                const int r = idx / (K / 8), q = idx % (K / 8);
-                int64_t pos = pos0 + ct * 32 + r;
-                pos = pos < p.M ? pos : p.M - 1;                     // rows past the end: any valid row, never stored
-                *reinterpret_cast<uint4 *>(stage + r * PS + 8 * q) = *reinterpret_cast<const uint4 *>(x + pos * K + 8 * q);
-            }
-            wave_lds_sync();
-            if constexpr (kLN) {
-                layer_norm_tile_rows<T, K>(stage, PS, lane, gamma_l, beta_l, p.eps);
+                for (int i = 0; i < kCPL; ++i) {
+                    v[i] = *reinterpret_cast<const float4 *>(src + (size_t)(8 * i) * p.L);
+                    sum[0] += v[i].x; sum[1] += v[i].y; sum[2] += v[i].z; sum[3] += v[i].w;
+                }
+                float mean[4], sq[4] = {0.0f, 0.0f, 0.0f, 0.0f}, rstd[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sum[e] += __shfl_xor(sum[e], 8); sum[e] += __shfl_xor(sum[e], 16); sum[e] += __shfl_xor(sum[e], 32);
+                    mean[e] = sum[e] * (1.0f / K);
+                }
+#pragma unroll
+                for (int i = 0; i < kCPL; ++i) {
+                    const float d0 = v[i].x - mean[0], d1 = v[i].y - mean[1], d2 = v[i].z - mean[2], d3 = v[i].w - mean[3];
+                    sq[0] = fmaf(d0, d0, sq[0]); sq[1] = fmaf(d1, d1, sq[1]); sq[2] = fmaf(d2, d2, sq[2]); sq[3] = fmaf(d3, d3, sq[3]);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sq[e] += __shfl_xor(sq[e], 8); sq[e] += __shfl_xor(sq[e], 16); sq[e] += __shfl_xor(sq[e], 32);
+                    rstd[e] = __builtin_amdgcn_rsqf(sq[e] * (1.0f / K) + p.eps);
+                }
+#pragma unroll
+                for (int i = 0; i < kCPL; ++i) {
+                    const int c = cs + 8 * i;
+                    const float g = to_f32(T{gamma_l[c]}), bt = to_f32(T{beta_l[c]});
+                    const float in[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        stage[(4 * quad + e) * PS + c] = from_f32<T>(fmaf((in[e] - mean[e]) * rstd[e], g, bt)).bits;
+                }
                 wave_lds_sync();
+            } else {
+#pragma unroll
+                for (int it = 0; it < kPiecesIn / kWave; ++it) {
+                    const int idx = lane + it * kWave;
+                    const int r = idx / (K / 8), q = idx % (K / 8);
+                    int64_t pos = pos0 + ct * 32 + r;
+                    pos = pos < p.M ? pos : p.M - 1;                     // rows past the end: any valid row, never stored
+                    *reinterpret_cast<uint4 *>(stage + r * PS + 8 * q) = *reinterpret_cast<const uint4 *>(x + pos * K + 8 * q);
+                }
+                wave_lds_sync();
+                if constexpr (kLN) {
+                    layer_norm_tile_rows<T, K>(stage, PS, lane, gamma_l, beta_l, p.eps);
+                    wave_lds_sync();
+                }
             }
 #pragma unroll
             for (int s = 0; s < kSteps; ++s) xf[ct][s] = *reinterpret_cast<const u32x4_t *>(stage + j * PS + 16 * s + 8 * kh);
@@ -138,7 +187,7 @@ __global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
     }
 }
 
-template <typename T, int K, int N, int kCT>
+template <typename T, int K, int N, int kCT, bool kCfIn = false>
 static int launch_linear(LinArgs a, hipStream_t stream) {
     constexpr int kMaxKN = K > N ? K : N;
     const size_t smem = (size_t)(N * (K + 8) + (kBlock / kWave) * 32 * (kMaxKN + 8) + N + 2 * K) * sizeof(uint16_t);
@@ -156,14 +205,16 @@ static int launch_linear(LinArgs a, hipStream_t stream) {
     const int64_t n_wg = (tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     if (smem > 64 * 1024) {
-        const void *fn = a.ln_w ? reinterpret_cast<const void *>(&linear_cl_kernel<T, K, N, kCT, true>)
+        const void *fn = kCfIn  ? reinterpret_cast<const void *>(&linear_cl_kernel<T, K, N, kCT, true, kCfIn>)
+                       : a.ln_w ? reinterpret_cast<const void *>(&linear_cl_kernel<T, K, N, kCT, true>)
                                 : reinterpret_cast<const void *>(&linear_cl_kernel<T, K, N, kCT, false>);
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
             (void)hipGetLastError();
             return SS2D_ENOTSUP;
         }
     }
-    if (a.ln_w) hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    if constexpr (kCfIn) hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, true, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
+    else if (a.ln_w) hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
     else hipLaunchKernelGGL((linear_cl_kernel<T, K, N, kCT, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a);
     return launch_status();
 }
@@ -187,8 +238,28 @@ extern "C" int ss2d_linear_cl(const void *x, const void *ln_weight, const void *
         if (q && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return SS2D_ENOTSUP;
     LinArgs a;
     a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.w = weight; a.bias = bias; a.residual = residual; a.out = out;
-    a.M = M; a.eps = eps; a.tiles_per_wg = 1;
+    a.M = M; a.eps = eps; a.tiles_per_wg = 1; a.L = 0;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == SS2D_BF16) return launch_linear<bf16_t, 96, 96, 2>(a, s);
     return launch_linear<f16_t, 96, 96, 2>(a, s);
+}
+
+extern "C" int ss2d_linear_cf_ln(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
+                                 const void *bias, const void *residual, void *out, int B, int L, int K, int N, int dtype,
+                                 void *stream) {
+    using namespace ss2d;
+    if (B < 0 || L < 0 || K <= 0 || N <= 0) return SS2D_EINVAL;
+    if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
+    if (B == 0 || L == 0) return SS2D_OK;
+    if (!x || !ln_weight || !weight || !out) return SS2D_EINVAL;
+    if (dtype == SS2D_F32 || K != 96 || N != 96 || L % 32 != 0) return SS2D_ENOTSUP;
+    const void *ptrs[] = {x, ln_weight, ln_bias, weight, bias, residual, out};
+    for (const void *q : ptrs)
+        if (q && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return SS2D_ENOTSUP;
+    LinArgs a;
+    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.w = weight; a.bias = bias; a.residual = residual; a.out = out;
+    a.M = (int64_t)B * L; a.eps = eps; a.tiles_per_wg = 1; a.L = L;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == SS2D_BF16) return launch_linear<bf16_t, 96, 96, 2, true>(a, s);
+    return launch_linear<f16_t, 96, 96, 2, true>(a, s);
 }

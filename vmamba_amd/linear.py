@@ -41,3 +41,38 @@ def linear_cl_hip(x, weight, bias=None, residual=None, ln_weight=None, ln_bias=N
                                        torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "ss2d_linear_cl")
     return out
+
+
+def linear_cf_ln_fusable(K, weight, L):
+    """True when ss2d_linear_cf_ln takes an fp32 channel-first map (B, K, L) with this 16-bit GPU weight (N, K)."""
+    return (weight.is_cuda and weight.dtype in _DTYPE_CODE and weight.dim() == 2 and weight.shape[1] == K
+            and (K, weight.shape[0]) in FUSED_SHAPES and L % 32 == 0)
+
+
+def linear_cf_ln_hip(y, ln_weight, ln_bias, eps, weight, bias=None, residual=None):
+    """y (B, K, L) fp32 channel-first (the merged output of the SS2D core), weight (N, K) bf16 / fp16: returns
+    layer_norm(y over K, computed in fp32, rounded to the weight's dtype) @ weight.T + bias + residual as the
+    channel-last tensor (B, L, N) -- out_norm and out_proj of the block (vmamba.py:641-646, :662) in one kernel."""
+    if not y.is_cuda:
+        raise NotImplementedError("linear_cf_ln_hip: vmamba_amd runs on the GPU only")
+    if y.dtype != torch.float32 or y.dim() != 3 or weight.dtype not in _DTYPE_CODE:
+        raise TypeError("linear_cf_ln_hip: y must be (B, K, L) float32 and the weight bf16 or fp16")
+    B, K, L = y.shape
+    if weight.dim() != 2 or weight.shape[1] != K:
+        raise ValueError(f"linear_cf_ln_hip: weight must be (N, {K}), got {tuple(weight.shape)}")
+    N, dt = weight.shape[0], weight.dtype
+    y = y.contiguous()
+    out = torch.empty((B, L, N), device=y.device, dtype=dt)
+    if residual is not None and (residual.numel() != out.numel() or residual.dtype != dt):
+        raise ValueError("linear_cf_ln_hip: residual must have the size and dtype of the result")
+    small = [None if t is None else t.to(dt).contiguous() for t in (ln_weight, ln_bias, bias)]
+    if small[0] is None:
+        raise ValueError("linear_cf_ln_hip: the LayerNorm weight is required")
+    keep = [weight.contiguous(), None if residual is None else residual.contiguous()]
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(y.device):
+        rc = _lib.lib().ss2d_linear_cf_ln(y.data_ptr(), ptr(small[0]), ptr(small[1]), float(eps), keep[0].data_ptr(), ptr(small[2]),
+                                          ptr(keep[1]), out.data_ptr(), B, L, K, N, _DTYPE_CODE[dt],
+                                          torch.cuda.current_stream(y.device).cuda_stream)
+    _lib.check(rc, "ss2d_linear_cf_ln")
+    return out

@@ -24,7 +24,7 @@ from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
-from .linear import linear_cl_hip, linear_fusable
+from .linear import linear_cf_ln_fusable, linear_cf_ln_hip, linear_cl_hip, linear_fusable
 from .norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip,
                    needs_grad)
 
@@ -188,13 +188,17 @@ class SS2D(nn.Module):
         return ss2d_core_hip(x, delta, x_dbl[:, R], x_dbl[:, R + 1], consts["As"].view(-1), consts["Ds"],
                              consts["dt_bias"], True)
 
+    def _fused_core_applies(self, x):
+        """The fused kernel is an inference kernel for one-state models whose map fits its LDS planes; under autograd
+        the three operators (each with a backward) run."""
+        trains = needs_grad(x, self.x_proj_weight, self.dt_projs_weight, self.A_logs, self.Ds, self.dt_projs_bias)
+        return self.d_state == 1 and self.fused_core and not trains and core_fits(x.shape[2], x.shape[3], x.dtype)
+
     def forward_core(self, x):
         B, D, H, W = x.shape
         K, L = self.k_group, H * W
         consts = self._inference_constants(B)
-        # the fused kernel is an inference kernel; under autograd the three operators (each with a backward) run
-        trains = needs_grad(x, self.x_proj_weight, self.dt_projs_weight, self.A_logs, self.Ds, self.dt_projs_bias)
-        if self.d_state == 1 and self.fused_core and not trains and core_fits(H, W, x.dtype):
+        if self._fused_core_applies(x):
             return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
         dts, Bs, Cs = self.project_from_map(x, consts)
@@ -223,6 +227,16 @@ class SS2D(nn.Module):
         return (not self.channel_first and isinstance(linear, nn.Linear) and not isinstance(linear, Linear2d)
                 and linear_fusable(x, linear.weight) and not needs_grad(x, linear.weight, linear.bias, *extra))
 
+    def _norm_proj_fusable(self, x, residual):
+        """True when ss2d_linear_cf_ln serves out_norm + out_proj (+ residual) of this block for the conv output x."""
+        L = x.shape[2] * x.shape[3]
+        return (not self.channel_first and isinstance(self.out_norm, LayerNorm) and self.out_norm.elementwise_affine
+                and isinstance(self.out_proj, nn.Linear) and not isinstance(self.out_proj, Linear2d)
+                and self.out_proj.weight.dtype == x.dtype and self._fused_core_applies(x)
+                and x.is_cuda and linear_cf_ln_fusable(self.d_inner, self.out_proj.weight, L)
+                and (residual is None or residual.dtype == x.dtype)
+                and not needs_grad(residual, self.out_proj.weight, self.out_proj.bias, self.out_norm.weight, self.out_norm.bias))
+
     def forward(self, x, residual=None, pre_norm=None, post_norm=None):
         """``pre_norm``: the block's LayerNorm, applied to x first (vmamba.py:1227); ``residual`` (same layout as x) is
         added to the result (:1228).  A channel-last block of width 96 runs norm + in_proj and out_proj + add as one
@@ -244,6 +258,12 @@ class SS2D(nn.Module):
             x, z = x.chunk(2, dim=(1 if self.channel_first else -1))
             z = self.act(z)
         x = self.layers.conv_act(self.conv2d if self.with_dconv else None, x, self.channel_first)   # (B, D, H, W)
+        if z is None and self._norm_proj_fusable(x, residual):
+            # out_norm, out_proj and the residual add in one kernel, straight from the core's fp32 map
+            B, _, H, W = x.shape
+            y = self.forward_core_fused(x, self._inference_constants(B))                        # (B, D, L) fp32
+            return linear_cf_ln_hip(y, self.out_norm.weight, self.out_norm.bias, self.out_norm.eps, self.out_proj.weight,
+                                    self.out_proj.bias, residual).view(B, H, W, self.d_model)
         y = self.forward_core(x)
         if z is not None:
             y = y * z
