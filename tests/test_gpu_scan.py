@@ -98,6 +98,9 @@ GRID = [
     (1, 8, 4, 16, 49), (1, 8, 4, 16, 520), (1, 4, 2, 16, 3136), (2, 6, 2, 2, 100), (1, 6, 3, 5, 777), (1, 4, 1, 8, 2500),
     (1, 2, 1, 64, 300),
     (3, 40, 4, 1, 8), (2, 100, 4, 1, 9), (5, 24, 4, 1, 57), (2, 64, 4, 16, 25), (1, 96, 4, 1, 1023), (3, 7, 1, 1, 130),
+    # rows that end at most 128 positions past a full 512-position pass (the one-state kernel walks those one per lane):
+    # across a 2048-chunk boundary, two tail passes with the second partial, exactly two, a short one, no full pass
+    (1, 8, 4, 1, 2112), (2, 8, 4, 1, 1128), (1, 8, 2, 1, 128), (2, 8, 4, 1, 520), (1, 8, 4, 1, 72),
 ]
 
 

@@ -22,6 +22,8 @@
 
 namespace ss2d {
 
+constexpr int kScanTailMax = 2;     // the short-tail row kernel takes up to this many 64-position tail passes
+
 struct ScanArgs {
     const void *u, *delta, *B, *C;
     const float *A, *D, *bias;
@@ -37,8 +39,9 @@ struct ScanArgs {
 // kN == 1: the single state lives in registers and inputs are fetched in bursts.
 // kN == 0: any dstate; the per-wave states (running product, h) live in LDS, 2*dstate floats per wave: they
 //          are wave-uniform, and keeping 3*dstate of them in vector registers (tried for dstate 16) spills.
-template <typename in_t, typename out_t, int kN, bool kVec, bool kSoftplus>
+template <typename in_t, typename out_t, int kN, bool kVec, bool kSoftplus, bool kShortTail = false>
 __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
+    static_assert(!kShortTail || (kN == 1 && kVec), "the short tail belongs to the one-state vector kernel");
     extern __shared__ __align__(16) float dyn_state[];   // kN == 0 only: [wave][N][2]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -83,17 +86,24 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     // each wavefront keeps several KB in flight.
     constexpr bool kBurstBC = kN == 1;
     constexpr int kBurst = kN == 1 ? 4 : 1;
-    const int n_pass = (L + kPass - 1) / kPass;
+    // kShortTail (chosen by the host when a row ends with at most kScanTailMax * 64 positions past its last full pass;
+    // 56 x 56 maps: 6 passes + 64): those positions are walked one per lane -- about a fifth of the cost of a full
+    // pass each -- instead of as an eighth-full pass of 8 per lane.  It is an instantiation of its own because the
+    // extra code costs the register that lets five wavefronts share a SIMD, which the other row lengths keep.
+    const int tail = L % kPass;
+    const bool short_tail = kShortTail;
+    const int n_pass = short_tail ? L / kPass : (L + kPass - 1) / kPass;
+    const int L_body = short_tail ? n_pass * kPass : L;              // what the 8-per-lane passes cover
     for (int pass0 = 0; pass0 < n_pass; pass0 += kBurst) {
         Raw8<in_t> u_burst[kBurst], dl_burst[kBurst], B_burst[kBurst], C_burst[kBurst];
 #pragma unroll
         for (int s = 0; s < kBurst; ++s) {
             const int pos_s = (pass0 + s) * kPass + lane * kItems;
-            u_burst[s] = load_raw<in_t, kVec>(u_row, pos_s, L);
-            dl_burst[s] = load_raw<in_t, kVec>(dl_row, pos_s, L, delta_fill<kSoftplus>());
+            u_burst[s] = load_raw<in_t, kVec>(u_row, pos_s, L_body);
+            dl_burst[s] = load_raw<in_t, kVec>(dl_row, pos_s, L_body, delta_fill<kSoftplus>());
             if constexpr (kBurstBC) {
-                B_burst[s] = load_raw<in_t, kVec>(B_row, pos_s, L);
-                C_burst[s] = load_raw<in_t, kVec>(C_row, pos_s, L);
+                B_burst[s] = load_raw<in_t, kVec>(B_row, pos_s, L_body);
+                C_burst[s] = load_raw<in_t, kVec>(C_row, pos_s, L_body);
             }
         }
 #pragma unroll
@@ -105,8 +115,8 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
         Raw8<in_t> B_raw, C_raw;
         if constexpr (kBurstBC) { B_raw = B_burst[s]; C_raw = C_burst[s]; }
         float dl[kItems], du[kItems], y[kItems];
-        prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
-        const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || pass == n_pass - 1);
+        prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L_body - pos, bias, Dv, dl, du, y);
+        const bool chunk_end = x_row && ((pass + 1) % kPassesPerChunk == 0 || (pass == n_pass - 1 && !short_tail));
         float *x_out = chunk_end ? x_row + (size_t)(pass / kPassesPerChunk) * 2 * N : nullptr;
 
         if constexpr (kN > 0) {
@@ -156,7 +166,37 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
                 }
             }
         }
-        store_items<out_t, kVec>(o_row, pos, L, y);
+        store_items<out_t, kVec>(o_row, pos, L_body, y);
+        }
+    }
+    if constexpr (kShortTail) {
+        if (short_tail) {
+#pragma unroll
+            for (int t = 0; t < kScanTailMax; ++t) {
+                if (t * kWave >= tail) break;
+                const int tp = L_body + t * kWave + lane;
+                const bool ok = tp < L;
+                const int tq = ok ? tp : L - 1;
+                const float tu = ok ? to_f32(u_row[tq]) : 0.0f;                  // u = 0 and dl = 0: the identity pair
+                const float tdl = ok ? to_f32(dl_row[tq]) : delta_fill<kSoftplus>();
+                const float tB = to_f32(B_row[tq]), tC = to_f32(C_row[tq]);
+                float dl;
+                if constexpr (kSoftplus) dl = softplus_log2(fmaf(tdl, kLog2e, bias * kLog2e));
+                else dl = ok ? tdl + bias : 0.0f;
+                const float a = __builtin_amdgcn_exp2f(dl * A_reg[0]);
+                const float bb = tB * (dl * tu);
+                float a_ex, h_ex, a_tot, h_tot;
+                wave_scan_pairs(a, bb, a_ex, h_ex, a_tot, h_tot);
+                const float hv = fmaf(a, fmaf(a_ex, h_reg[0], h_ex), bb);
+                if (ok) o_row[tp] = from_f32<out_t>(fmaf(tC, hv, Dv * tu));
+                h_reg[0] = fmaf(a_tot, h_reg[0], h_tot);
+                ap_reg[0] *= a_tot;
+            }
+            // the tail belongs to the chunk of pass n_pass: it ends that chunk (and the row)
+            if (x_row && lane == 0) {
+                float *x_out = x_row + (size_t)(n_pass / kPassesPerChunk) * 2 * N;
+                x_out[0] = ap_reg[0]; x_out[1] = h_reg[0];
+            }
         }
     }
 }
@@ -464,6 +504,17 @@ static int launch_scan(const ScanArgs &a, hipStream_t stream) {
 #define SS2D_LAUNCH_ROW(N, SP, SMEM) \
     hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, N, kVec, SP>), dim3(n_wg), dim3(kBlock), SMEM, stream, a)
     if (a.N == 1) {
+        const int tail = a.L % kPass;
+        if constexpr (kVec) {
+            if (tail > 0 && tail <= kScanTailMax * kWave) {
+                if (a.softplus) {
+                    hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 1, true, true, true>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+                } else {
+                    hipLaunchKernelGGL((scan_row_kernel<in_t, out_t, 1, true, false, true>), dim3(n_wg), dim3(kBlock), 0, stream, a);
+                }
+                return launch_status();
+            }
+        }
         if (a.softplus) SS2D_LAUNCH_ROW(1, true, 0); else SS2D_LAUNCH_ROW(1, false, 0);
     } else {
         const size_t smem = (size_t)kWavesPerWg * 2 * a.N * sizeof(float);
