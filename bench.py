@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # `bench.py --kernels-only`, each counter scaled by what it reads for the 1 GiB calibration copy (FETCH_SIZE x2.0,
 # WRITE_SIZE x1.0); the summary is profiles/ss2d_core_kernels_vmamba_t_bs128.txt.  Counters cannot be read from
 # inside the timed process, so this is the last profiled value, refreshed whenever the kernel changes.
-SCAN_STAGE1_MEASURED_TRAFFIC_BYTES = 668.4e6 + 617.1e6
+SCAN_STAGE1_MEASURED_TRAFFIC_BYTES = 668.2e6 + 617.0e6    # FETCH_SIZE 326288 KiB x 2.0, WRITE_SIZE 602539 KiB
 CORE_STAGE1_MEASURED_TRAFFIC_BYTES = 437.0e6 + 154.1e6    # same profile: FETCH_SIZE 213382 KiB x 2.0, WRITE_SIZE 150528 KiB
 
 
@@ -113,7 +113,7 @@ def kernel_lines(reps):
             # block-level kernels of the narrow stages (harness side): fused LayerNorm + MLP + residual, and at width 96
             # the two projections with their LayerNorm / residual.  Bytes: activations in and out once (+ residual).
             from vmamba_amd.mlp import mlp_fused_hip
-            from vmamba_amd.linear import linear_cl_hip, linear_fusable
+            from vmamba_amd.linear import linear_cf_ln_fusable, linear_cf_ln_hip, linear_cl_hip, linear_fusable
             M = B * L
             xa = torch.randn(M, D, device=dev, generator=g).bfloat16()
             w1 = (torch.randn(4 * D, D, device=dev, generator=g) * D ** -0.5).bfloat16()
@@ -128,6 +128,12 @@ def kernel_lines(reps):
                 t_o = time_op(lambda: linear_cl_hip(xa, wp, None, xa), reps)
                 fused.update(ln_in_proj_us=t_i * 1e6, ln_in_proj_GBs=2 * M * D * 2 / t_i / 1e9,
                              out_proj_add_us=t_o * 1e6, out_proj_add_GBs=3 * M * D * 2 / t_o / 1e9)
+                if linear_cf_ln_fusable(D, wp, H * W):
+                    # out_norm + out_proj + residual straight from the core's fp32 channel-first map
+                    ycf = torch.randn(B, D, H * W, device=dev, generator=g)
+                    t_n = time_op(lambda: linear_cf_ln_hip(ycf, gam, bet, 1e-5, wp, None, xa), reps)
+                    fused.update(norm_out_proj_add_us=t_n * 1e6, norm_out_proj_add_GBs=M * D * (4 + 2 + 2) / t_n / 1e9)
+                    del ycf
             del xa, w1, w2, wp
             if name == "stage1":
                 # the patch embedding's first layer (conv 3x3 stride 2 + LayerNorm + GELU in one kernel): the image
