@@ -329,6 +329,14 @@ int ss2d_linear_cl(const void *x, const void *ln_weight, const void *ln_bias, fl
 int ss2d_linear_cf_ln(const void *x, const void *ln_weight, const void *ln_bias, float eps, const void *weight,
                       const void *bias, const void *residual, void *out, int B, int L, int K, int N, int dtype, void *stream);
 
+/*
+ * Global average pool of a channel-last map: y (B, C) = mean over the L positions of x (B, L, C), fp32 sum times 1/L
+ * rounded once to dtype -- the AdaptiveAvgPool2d(1) of the classifier head (classification/models/vmamba.py:1357-1363)
+ * on the channel-last activation.  One pass, no workspace, no counters: the result does not depend on scheduling.
+ * dtype SS2D_BF16 or SS2D_F16, C a multiple of 8, x 16-byte aligned; anything else returns SS2D_ENOTSUP.
+ */
+int ss2d_mean_pool_cl(const void *x, void *y, int B, int L, int C, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

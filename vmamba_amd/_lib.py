@@ -17,7 +17,7 @@ ABI_VERSION = 1
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
            "ss2d_layer_norm", "ss2d_add_layer_norm", "ss2d_bias_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
            "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_merge_flex",
-           "ss2d_selective_scan_bwd", "ss2d_transpose_bcl", "ss2d_mlp_fused", "ss2d_linear_cl", "ss2d_linear_cf_ln", "ss2d_stem_conv_ln_gelu")
+           "ss2d_selective_scan_bwd", "ss2d_transpose_bcl", "ss2d_mlp_fused", "ss2d_linear_cl", "ss2d_linear_cf_ln", "ss2d_stem_conv_ln_gelu", "ss2d_mean_pool_cl")
 
 
 class ScanParams(ctypes.Structure):
@@ -127,6 +127,8 @@ def lib():
         L.ss2d_linear_cf_ln.restype = ctypes.c_int
         L.ss2d_linear_cf_ln.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_float] + [ctypes.c_void_p] * 4 +
                                         [ctypes.c_int] * 5 + [ctypes.c_void_p])
+        L.ss2d_mean_pool_cl.restype = ctypes.c_int
+        L.ss2d_mean_pool_cl.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
         if L.ss2d_abi_version() != ABI_VERSION:
             raise ImportError(f"{LIB_PATH}: ABI version {L.ss2d_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L

@@ -22,6 +22,7 @@ from .mlp import mlp_fusable, mlp_fused_hip
 from .norm import LayerNorm as HipLayerNorm
 from .norm import add_layer_norm_fusable, add_layer_norm_hip, bias_layer_norm_fusable, bias_layer_norm_hip, needs_grad
 from .ss2d import SS2D, HipLayers, Linear2d
+from .pool import GlobalAvgPool2d
 from .stem import stem_conv_ln_gelu_hip, stem_fusable
 
 
@@ -185,7 +186,7 @@ class VSSM(nn.Module):
             stages.append(nn.Sequential(OrderedDict(blocks=BlockSequence(*blocks), downsample=down)))
         self.layers = nn.ModuleList(stages)
         self.classifier = nn.Sequential(OrderedDict(
-            norm=Norm(dims[-1]), permute=_to_cf(cf), avgpool=nn.AdaptiveAvgPool2d(1), flatten=nn.Flatten(1),
+            norm=Norm(dims[-1]), permute=_to_cf(cf), avgpool=GlobalAvgPool2d(), flatten=nn.Flatten(1),
             head=nn.Linear(dims[-1], num_classes)))
         self.apply(self._init_weights)
 
