@@ -284,7 +284,7 @@ def main():
             torch.cuda.synchronize()
         return graph, out
 
-    gemm_mode = "library-default GEMM solutions"
+    gemm_mode, tuned = "library-default GEMM solutions", False
     sub_batches = args.sub_batches if (not args.eager and args.sub_batches > 1 and args.batch % args.sub_batches == 0) else 1
     with torch.no_grad():
         model(x)
@@ -305,6 +305,7 @@ def main():
                 model(x if sub_batches == 1 else x.chunk(sub_batches)[0])
                 torch.cuda.synchronize()
                 tunable.tuning_enable(False)
+                tuned = True
                 gemm_mode = "GEMM solutions picked by PyTorch TunableOp"
                 log(f"GEMM tuning forward: {time.perf_counter() - t_tune:.1f} s, {len(tunable.get_results())} shapes")
             except Exception as e:      # an optimisation of library calls, never a requirement
@@ -327,6 +328,11 @@ def main():
                 log(f"sub-batch graph capture failed ({type(e).__name__}: {e}); one graph for the whole batch")
                 runner = None
         if not args.eager and runner is None:
+            if tuned and sub_batches > 1:   # the GEMM shapes of the whole batch have not been tuned yet
+                tunable.tuning_enable(True)
+                model(x)
+                torch.cuda.synchronize()
+                tunable.tuning_enable(False)
             try:
                 captured = capture_forward()
             except Exception as e:          # capture is an optimisation of the launch path, never a requirement
