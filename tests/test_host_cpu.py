@@ -111,3 +111,22 @@ def test_gelu_table_is_what_the_generator_writes_and_matches_erf():
     for s in (1.0, -1.0):
         g = 0.5 * s * x + x * vals
         assert np.allclose(g, 0.5 * s * x * (1.0 + erf(s * x / np.sqrt(2.0))), rtol=0, atol=1e-6)
+
+
+def test_inference_constants_are_kept_per_batch_size_and_follow_the_parameters():
+    """A = -exp(A_logs) etc. (vmamba.py:619-623) are cached per batch size -- the sub-batches of a runner alternate with
+    whole batches -- and recomputed when a parameter changes or autograd is on."""
+    m = SS2D(d_model=8, d_state=1, ssm_ratio=1.0, dt_rank=2, channel_first=False)
+    with torch.no_grad():
+        c2, c3 = m._inference_constants(2), m._inference_constants(3)
+        assert m._inference_constants(2) is c2 and m._inference_constants(3) is c3
+        assert c2["Wx"].shape[0] == 2 * 4 and c3["Wx"].shape[0] == 3 * 4
+        assert torch.equal(c2["As"], -m.A_logs.float().exp())
+        for b in range(4, 10):                                   # the cache stays small
+            m._inference_constants(b)
+        assert len(m._const_cache) <= 4
+        m.A_logs.add_(0.5)                                       # in-place update bumps the version: everything stale
+        fresh = m._inference_constants(2)
+        assert fresh is not c2 and torch.equal(fresh["As"], -m.A_logs.float().exp())
+        assert all(k[0] == 2 for k in m._const_cache)
+    assert m._inference_constants(2) is not m._inference_constants(2)      # under autograd nothing is kept

@@ -118,20 +118,29 @@ class SS2D(nn.Module):
     def _inference_constants(self, batch):
         """Tensors that depend only on the parameters (and the batch size): A = -exp(A_logs), fp32 D and dt bias
         (vmamba.py:619-623) and the projection weights repeated over the batch so each projection is ONE
-        strided-batched GEMM over B*K problems.  Recomputed whenever autograd is on or a parameter changed."""
+        strided-batched GEMM over B*K problems.  Recomputed whenever autograd is on or a parameter changed; kept for up to
+        four batch sizes."""
         params = (self.A_logs, self.Ds, self.dt_projs_bias, self.x_proj_weight, self.dt_projs_weight)
         key = (batch, torch.is_grad_enabled(), tuple((p._version, p.data_ptr(), p.dtype, p.device) for p in params))
-        cached = getattr(self, "_const_cache", None)
-        if cached is not None and cached[0] == key:
-            return cached[1]
+        cache = self.__dict__.setdefault("_const_cache", {})
+        if key in cache:
+            return cache[key]
         K = self.k_group
         consts = dict(
             As=-self.A_logs.float().exp(), Ds=self.Ds.float(), dt_bias=self.dt_projs_bias.reshape(-1).float(),
             Wx_all=self.x_proj_weight.reshape(1, -1, self.d_inner).expand(batch, -1, -1).contiguous(),
             Wx=self.x_proj_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, -1, self.d_inner).contiguous(),
             Wdt=self.dt_projs_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, self.d_inner, -1).contiguous())
-        if not torch.is_grad_enabled():
-            self._const_cache = (key, consts)
+        # kept per batch size (sub-batches of a runner alternate with whole batches); never from inside a graph capture,
+        # whose allocations live in the graph's memory pool and are overwritten by its replays
+        capturing = consts["As"].is_cuda and torch.cuda.is_current_stream_capturing()
+        if not torch.is_grad_enabled() and not capturing:
+            stale = [k for k in cache if k[2] != key[2]]
+            for k in stale:
+                del cache[k]
+            if len(cache) >= 4:
+                cache.pop(next(iter(cache)))
+            cache[key] = consts
         return consts
 
     def project(self, xs, consts=None):
