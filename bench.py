@@ -380,7 +380,8 @@ def main():
         "value": value, "unit": "img/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
+        "config": {"sub_batches": sub_batches if runner is not None else 1,
+                   "workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
                                f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}, {gemm_mode}; "
                                f"SS2D core, LayerNorm, depthwise conv, patch-embedding stem, narrow-stage MLP and projections on HIP kernels"},
         "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "kernels": kernels,
