@@ -458,7 +458,12 @@ static int launch_ln_rows(const void *x, const void *w, const void *b, void *y, 
         hipLaunchKernelGGL((layer_norm_rows_kernel<in_t, w_t, out_t, GROUP, CHUNKS>), dim3((uint32_t)n_wg), dim3(kBlock), \
                            0, stream, xp, wp, bp, yp, rows, C, eps, rp, sp, pp);                                         \
     }
-    if (vecs <= 4) SS2D_LN_LAUNCH(4, 1)
+    // widths of 3 * 2^k vectors would leave a quarter of a power-of-two group idle: three chunks per lane instead
+    // (C = 192: 23.7 -> 18.7 us, with the residual add 33.7 -> 28.1; C = 384: 13.1 -> 12.3 and 19.2 -> 16.6; at C = 96
+    // the add variant got slower and C = 768 did not change, so those keep the layouts below)
+    if (vecs == 24) SS2D_LN_LAUNCH(8, 3)
+    else if (vecs == 48) SS2D_LN_LAUNCH(16, 3)
+    else if (vecs <= 4) SS2D_LN_LAUNCH(4, 1)
     else if (vecs <= 8) SS2D_LN_LAUNCH(8, 1)
     else if (vecs <= 16) SS2D_LN_LAUNCH(16, 1)
     else if (vecs <= 32) SS2D_LN_LAUNCH(32, 1)
