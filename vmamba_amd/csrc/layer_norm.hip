@@ -460,7 +460,8 @@ static int launch_ln_rows(const void *x, const void *w, const void *b, void *y, 
     }
     // widths of 3 * 2^k vectors would leave a quarter of a power-of-two group idle: three chunks per lane instead
     // (C = 192: 23.7 -> 18.7 us, with the residual add 33.7 -> 28.1; C = 384: 13.1 -> 12.3 and 19.2 -> 16.6; at C = 96
-    // the add variant got slower and C = 768 did not change, so those keep the layouts below)
+    // the add variant got slower -- and the layout is chosen by width alone, so that the add variant and the plain one sum
+    // in the same order and agree bit for bit -- and C = 768 did not change, so those keep the layouts below)
     if (vecs == 24) SS2D_LN_LAUNCH(8, 3)
     else if (vecs == 48) SS2D_LN_LAUNCH(16, 3)
     else if (vecs <= 4) SS2D_LN_LAUNCH(4, 1)
