@@ -47,9 +47,11 @@ def core_bytes(B, D, L, s_in, K=4):
     return B * D * L * (s_in + K * s_in + 4) + 2 * B * K * L * s_in + 4 * K * D * 3
 
 
-def time_op(fn, reps, warm=5):
+def time_op(fn, reps, warm=None):
     import torch
-    for _ in range(warm):
+    # as many untimed launches as timed ones: the first few dozen launches of a kernel over freshly allocated
+    # tensors read ~5 % slower than its steady state
+    for _ in range(reps if warm is None else warm):
         fn()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
