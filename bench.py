@@ -11,7 +11,13 @@ roofline = the dominant kernel of that forward: the fused SS2D core (CrossScan +
            peak = 8 TB/s.  scan_roofline = the same for the stand-alone selective-scan kernel behind
            selective_scan_fn (the "scan GB/s" of the metric), which the three-operator path still uses.
 cpu_baseline = the torch-on-CPU restatement of the reference path (oracle/) run through the same
-           model on a bounded sample, on this box's host cores.
+           model on a bounded sample, on this box's host cores (img/s, the metric's unit).
+cpu_baseline_op / parity = benchmark config 0 (the reference's CPU-runnable SS2D operator: fp32, x (2,96,56,56) ->
+           CrossScan -> selective scan -> CrossMerge, seed 0) timed on the host cores with the torch restatement and
+           with the C oracle, beside the GPU's time on the same bits, and the GPU's error against that CPU result.
+Extra keys: ms_per_step_eager / ms_per_step_one_graph / ms_per_step_concurrent (the three launch modes of the same
+           forward; `value` is the fastest validated one and `config.launch` names it), config4 (4 x 1024^2 forward),
+           fp32 (the same batch-128 forward at the reference harness's precision).
 
 One JSON line is printed on stdout; progress goes to stderr.
 """
@@ -25,12 +31,27 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the stage-1 scan kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --kernels-only`, each counter scaled by what it reads for the 1 GiB calibration copy (FETCH_SIZE x2.0,
-# WRITE_SIZE x1.0); the summary is profiles/ss2d_core_kernels_vmamba_t_bs128.txt.  Counters cannot be read from
-# inside the timed process, so this is the last profiled value, refreshed whenever the kernel changes.
-SCAN_STAGE1_MEASURED_TRAFFIC_BYTES = 668.2e6 + 617.0e6    # FETCH_SIZE 326288 KiB x 2.0, WRITE_SIZE 602539 KiB
-CORE_STAGE1_MEASURED_TRAFFIC_BYTES = 437.0e6 + 154.1e6    # same profile: FETCH_SIZE 213382 KiB x 2.0, WRITE_SIZE 150528 KiB
+FP32_VECTOR_PEAK_TFLOPS = 157.3
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "ss2d_core_kernels_vmamba_t_bs128.txt")
+
+
+def measured_traffic(kernel_tag):
+    """HBM bytes per launch of a kernel from the committed rocprofv3 counter summary.  Counters cannot be read from
+    inside the timed process; the summary holds one line per kernel of the form
+        TRAFFIC <tag> fetch_kib=<FETCH_SIZE per dispatch> write_kib=<WRITE_SIZE per dispatch> fetch_scale=<f> write_scale=<w>
+    (the scales are what the same counters read for the 1 GiB calibration copy of `bench.py --kernels-only`).
+    Returns (bytes, "file: line") or (None, reason)."""
+    try:
+        with open(PROFILE_SUMMARY) as f:
+            for n, line in enumerate(f, 1):
+                parts = line.split()
+                if len(parts) >= 6 and parts[0] == "TRAFFIC" and parts[1] == kernel_tag:
+                    kv = dict(p.split("=", 1) for p in parts[2:])
+                    total = 1024.0 * (float(kv["fetch_kib"]) * float(kv["fetch_scale"]) + float(kv["write_kib"]) * float(kv["write_scale"]))
+                    return total, f"{os.path.relpath(PROFILE_SUMMARY, ROOT)}:{n}"
+    except (OSError, KeyError, ValueError) as e:
+        return None, f"{type(e).__name__}: {e}"
+    return None, f"no TRAFFIC line for {kernel_tag} in {os.path.relpath(PROFILE_SUMMARY, ROOT)}"
 
 
 def log(*a):
@@ -111,6 +132,26 @@ def kernel_lines(reps):
             b_dt = 2 * K * (D + R) * B * L + 2 * K * D * R
             fused.update(dt_proj_us=t_dt * 1e6, dt_proj_GBs=b_dt / t_dt / 1e9)
             del delta_k, B_k, C_k, dts, Wdt
+        if N == 1 and name != "hires":
+            # the two ops around the core in a block: depthwise conv + SiLU on the channel-last in_proj output, writing the
+            # channel-first map (bytes: the map in and out once), and out_norm on the core's fp32 channel-first output,
+            # writing the channel-last 16-bit activation (bytes: 4 in + 2 out per element)
+            from vmamba_amd.conv import dwconv3x3_silu_hip
+            from vmamba_amd.norm import layer_norm_cf_hip
+            x_cl = x.permute(0, 2, 3, 1).contiguous()
+            wconv = (torch.randn(D, 1, 3, 3, device=dev, generator=g) * 0.3).bfloat16()
+            t_dw = time_op(lambda: dwconv3x3_silu_hip(x_cl, wconv, None, in_channel_last=True), reps)
+            ycf = torch.randn(B, D, H, W, device=dev, generator=g)
+            gam, bet = torch.ones(D, device=dev).bfloat16(), torch.zeros(D, device=dev).bfloat16()
+            t_ln = time_op(lambda: layer_norm_cf_hip(ycf, gam, bet, 1e-5, out_channel_last=True, out_dtype=torch.bfloat16), reps)
+            fused.update(dwconv_us=t_dw * 1e6, dwconv_GBs=E * 4 / t_dw / 1e9, layer_norm_cf_us=t_ln * 1e6,
+                         layer_norm_cf_GBs=E * 6 / t_ln / 1e9)
+            del x_cl, ycf, wconv
+        if N > 1:
+            # several states per channel: the fp32 work by the reference's own count (csms6s.py:139-160) against the
+            # fp32 vector peak, beside the HBM figure
+            flops = 9.0 * B * K * D * L * N + B * K * D * L
+            fused.update(scan_TFLOPs=flops / t_sc / 1e12, valu_frac=flops / t_sc / 1e12 / FP32_VECTOR_PEAK_TFLOPS)
         if name in ("stage1", "stage2"):
             # block-level kernels of the narrow stages (harness side): fused LayerNorm + MLP + residual, and at width 96
             # the two projections with their LayerNorm / residual.  Bytes: activations in and out once (+ residual).
@@ -179,12 +220,33 @@ def kernel_lines(reps):
     return out
 
 
+def host_cpu():
+    """(threads to use, description).  The box gives a job a share of the host's cores and exports it as
+    OMP_NUM_THREADS; more threads than that share only oversubscribe it."""
+    count = os.cpu_count() or 1
+    share = os.environ.get("OMP_NUM_THREADS")
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        affinity = count
+    threads = min(count, affinity, int(share)) if share and share.isdigit() and int(share) > 0 else min(count, affinity)
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return threads, dict(cpu_model=model, host_cpu_count=count, sched_affinity=affinity, omp_num_threads_env=share)
+
+
 def cpu_baseline(seconds_budget=20.0):
     """Reference torch CPU path through the same model, fp32, on a bounded sample."""
     import torch
     from oracle.ss2d_core_ref import reference_vmamba_tiny
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    cores, info = host_cpu()
     torch.set_num_threads(cores)
     torch.manual_seed(0)
     model = reference_vmamba_tiny().eval()
@@ -201,9 +263,142 @@ def cpu_baseline(seconds_budget=20.0):
             spent += time.perf_counter() - t0
             reps += 1
     per = spent / reps if reps else first
-    return dict(value=batch / per, unit="img/s", cores=cores, kind="port",
+    return dict(value=batch / per, unit="img/s", cores=cores, kind="port", **info,
                 sample=f"VMamba-T forward, batch {batch} @224^2 fp32, torch CPU restatement of selective_scan_ref + "
                        f"torch CrossScan/CrossMerge, {max(reps, 1)} timed forward(s) after 1 warm-up, {per:.2f} s each")
+
+
+def config0_inputs():
+    """Benchmark config 0, seed 0, generated on the CPU in fp32 (the GPU gets copies of the same bits)."""
+    import math
+    import torch
+    Bsz, Dn, H, W, K, N = 2, 96, 56, 56, 4, 1
+    L = H * W
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(Bsz, Dn, H, W, generator=g)
+    delta = torch.randn(Bsz, K * Dn, L, generator=g)
+    dt = torch.exp(torch.rand(K * Dn, generator=g) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3))
+    bias = dt + torch.log(-torch.expm1(-dt))
+    A = -torch.exp(torch.log(torch.arange(1, N + 1, dtype=torch.float32))).repeat(K * Dn, 1)
+    Bm, Cm = torch.randn(Bsz, K, N, L, generator=g), torch.randn(Bsz, K, N, L, generator=g)
+    return x, delta, A, Bm, Cm, torch.ones(K * Dn), bias
+
+
+def err_stats(got, want, rtol, atol):
+    import torch
+    diff = (got.double() - want.double()).abs()
+    return dict(max_abs_err=diff.max().item(), max_rel_err=(diff / want.double().abs().clamp_min(atol / rtol)).max().item(),
+                rtol=rtol, atol=atol, within_tolerance=bool(torch.allclose(got.float(), want.float(), rtol=rtol, atol=atol)))
+
+
+def cpu_baseline_op(reps=3):
+    """Config 0 on the host cores and on the GPU, same bits: seconds, GB/s over the same algorithmic bytes, and the GPU's
+    error against the CPU result.  max_rel_err = max |gpu - cpu| / max(|cpu|, atol/rtol) (the reference tests' mixed
+    tolerance, kernels/selective_scan/test_selective_scan.py:401-403, as one number: <= rtol means within tolerance)."""
+    import statistics
+    import torch
+    import vmamba_amd as va
+    from oracle import ss2d_oracle as orc
+    from oracle import torch_ref
+    from vmamba_amd.core import ss2d_core_hip
+    cores, info = host_cpu()
+    torch.set_num_threads(cores)
+    x, delta, A, Bm, Cm, Dv, bias = config0_inputs()
+    Bsz, Dn, H, W = x.shape
+    K, L, N = 4, H * W, 1
+    E = Bsz * Dn * L
+    b_cs, b_sc, b_cm = 5 * E * 4, scan_bytes(Bsz, K * Dn, L, N, K, 4, 4), 5 * E * 4
+    bytes_total = b_cs + b_sc + b_cm
+
+    def torch_path():
+        xs = torch_ref.cross_scan(x)
+        ys = torch_ref.selective_scan(xs.reshape(Bsz, K * Dn, L), delta, A, Bm, Cm, Dv, bias, True)
+        return xs, ys, torch_ref.cross_merge(ys.view(Bsz, K, Dn, H, W))
+
+    def c_path():
+        xs = orc.cross_scan(x)
+        ys = orc.selective_scan(xs.view(Bsz, K * Dn, L), delta, A, Bm, Cm, Dv, bias, True)
+        return xs, ys, orc.cross_merge(ys.view(Bsz, K, Dn, H, W))
+
+    def timed(fn):
+        fn()                                                    # warm-up
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            out = fn()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts), out
+
+    with torch.no_grad():
+        t_torch, (xs_t, ys_t, y_t) = timed(torch_path)
+        t_c, (xs_c, ys_c, y_c) = timed(c_path)
+        dev = "cuda:0"
+        xd, dd, Ad, Bd, Cd, Dd, bd = (t.to(dev) for t in (x, delta, A, Bm, Cm, Dv, bias))
+
+        def gpu_path():
+            xs = va.cross_scan_fn(xd)
+            ys = va.selective_scan_fn(xs.view(Bsz, K * Dn, L), dd, Ad, Bd, Cd, Dd, bd, True)
+            return xs, ys, va.cross_merge_fn(ys.view(Bsz, K, Dn, H, W))
+
+        delta_k = dd.view(Bsz, K, Dn, L).permute(1, 2, 0, 3).contiguous()
+        B_k, C_k = Bd.view(Bsz, K, L).permute(1, 0, 2).contiguous(), Cd.view(Bsz, K, L).permute(1, 0, 2).contiguous()
+        A1 = Ad.view(-1)
+        t_gpu = time_op(gpu_path, 30)
+        t_fused = time_op(lambda: ss2d_core_hip(xd, delta_k, B_k, C_k, A1, Dd, bd, True), 30)
+        xs_g, ys_g, y_g = (t.cpu() for t in gpu_path())
+        y_f = ss2d_core_hip(xd, delta_k, B_k, C_k, A1, Dd, bd, True).cpu()
+    parity = dict(
+        config="0: fp32, x (2,96,56,56) seed 0 -> CrossScan -> selective scan (softplus, N=1) -> CrossMerge",
+        cpu_formulations_agree=dict(cross_scan_bit_exact=bool(torch.equal(xs_t, xs_c)), scan=err_stats(ys_c, ys_t, 1e-3, 1e-4),
+                                    merged=err_stats(y_c, y_t, 1e-3, 4e-4)),
+        cross_scan_bit_exact=bool(torch.equal(xs_g, xs_t)),
+        scan_vs_torch_cpu=err_stats(ys_g, ys_t, 1e-3, 1e-4),
+        cross_merge_bit_exact_on_gpu_scan_output=bool(torch.equal(y_g, torch_ref.cross_merge(ys_g.view(Bsz, K, Dn, H, W)))),
+        three_operators_vs_torch_cpu=err_stats(y_g, y_t, 1e-3, 4e-4),
+        fused_core_vs_torch_cpu=err_stats(y_f, y_t, 1e-3, 4e-4))
+    base = dict(config="0", algorithmic_bytes=bytes_total, cores=cores, **info,
+                torch_cpu=dict(seconds=t_torch, GBs=bytes_total / t_torch / 1e9, kind="port",
+                               what=f"torch restatement of cross_scan_fwd + selective_scan_ref + cross_merge_fwd, median of {reps} after 1 warm-up"),
+                c_oracle_cpu=dict(seconds=t_c, GBs=bytes_total / t_c / 1e9, kind="port",
+                                  what=f"plain-C oracle (OpenMP over rows, {orc.num_threads()} threads), median of {reps} after 1 warm-up"),
+                gpu_three_operators=dict(seconds=t_gpu, GBs=bytes_total / t_gpu / 1e9),
+                gpu_fused_core=dict(seconds=t_fused, GBs=core_bytes(Bsz, Dn, L, 4) / t_fused / 1e9,
+                                    algorithmic_bytes=core_bytes(Bsz, Dn, L, 4)),
+                note="config 0 is 53 MB of traffic: on the GPU it is launch-bound (three launches of a few microseconds each)")
+    return base, parity
+
+
+def stage_parity(n_images=2):
+    """A slice of every GPU configuration (bf16, batch 128) against the C oracle: the fused core's output for the first
+    and the last ``n_images`` images of each VMamba-T stage shape."""
+    import torch
+    from oracle import ss2d_oracle as orc
+    from vmamba_amd.core import ss2d_core_hip
+    dev = "cuda:0"
+    out = {}
+    for name, (B, D, H, W) in dict(stage1=(128, 96, 56, 56), stage2=(128, 192, 28, 28), stage3=(128, 384, 14, 14),
+                                   stage4=(128, 768, 7, 7)).items():
+        L = H * W
+        g = torch.Generator(device=dev).manual_seed(B + D)
+        rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+        x, delta = rn(B, D, H, W).bfloat16(), (rn(4, D, B, L) * 0.5).bfloat16()
+        Bs, Cs = rn(4, B, L).bfloat16(), rn(4, B, L).bfloat16()
+        A, Dv, bias = -(0.5 + torch.rand(4 * D, device=dev, generator=g)), rn(4 * D), rn(4 * D) - 3.0
+        y = ss2d_core_hip(x, delta, Bs, Cs, A, Dv, bias, True)
+        worst = None
+        for b0 in (0, B - n_images):
+            sl = slice(b0, b0 + n_images)
+            xs = orc.cross_scan(x[sl].cpu())
+            ys = orc.selective_scan(xs.reshape(n_images, 4 * D, L), delta[:, :, sl].permute(2, 0, 1, 3).reshape(n_images, 4 * D, L).cpu(),
+                                    A.view(-1, 1).cpu(), Bs[:, sl].permute(1, 0, 2).unsqueeze(2).cpu(), Cs[:, sl].permute(1, 0, 2).unsqueeze(2).cpu(),
+                                    Dv.cpu(), bias.cpu(), True)
+            want = orc.cross_merge(ys.view(n_images, 4, D, H, W))
+            st = err_stats(y[sl].cpu(), want, 1e-3, 4e-4)
+            if worst is None or st["max_rel_err"] > worst["max_rel_err"]:
+                worst = st
+        out[name] = worst
+        del x, delta, Bs, Cs, y
+    return out
 
 
 def main():
@@ -215,14 +410,15 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--no-extra-forwards", action="store_true",
+                    help="skip the config-4 (4 x 1024^2) and fp32 forwards reported as extra keys")
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the model: time the SS2D-core kernels at the four stage shapes plus a 1 GiB "
                          "device copy (the known-size kernel profiler counters are scaled against)")
     ap.add_argument("--eager", action="store_true",
-                    help="time eager launches.  By default the forward is captured once into a HIP graph and the timed "
-                         "steps replay it (about 190 kernels per forward, many of them 10-20 us: 2 %% faster than eager "
-                         "launches); the replays are first checked bit for bit against the eager result, and any "
-                         "failure to capture or to reproduce it falls back to eager launches")
+                    help="time eager launches only.  By default three launch modes of the same forward are timed -- eager "
+                         "launches, one captured HIP graph, sub-batch graphs side by side -- each graph mode only after its "
+                         "replays reproduced the eager result bit for bit, and the fastest becomes `value`")
     ap.add_argument("--sub-batches", type=int, default=4,
                     help="run the batch as this many equal sub-batches, each captured into a HIP graph of its own and "
                          "replayed on its own stream, all launched together (kernels of one sub-batch fill the compute "
@@ -263,147 +459,205 @@ def main():
         model = model.to(memory_format=torch.channels_last)
     x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
 
-    def capture_forward():
+    def time_steps(step, warmup, steps):
+        """The reference's protocol (classification/main.py:346-363): warm-up, synchronise, time `steps` launches
+        between synchronisations.  Returns seconds for the `steps` launches."""
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    def capture_forward(net, inp):
         """Capture one forward into a HIP graph and check replays against the eager result (replays interleaved
         with eager work and synchronisations); returns (graph, static_output) or None if anything differs."""
-        eager = model(x).float()
+        eager = net(inp).float()
         torch.cuda.synchronize()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(3):
-                model(x)
+                net(inp)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            out = model(x)
+        with torch.cuda.graph(graph, stream=side):
+            out = net(inp)
         for _ in range(3):
             graph.replay()
             torch.cuda.synchronize()
             if not torch.equal(out.float(), eager):
                 return None
-            model(x)                       # eager work between replays
+            net(inp)                       # eager work between replays
             torch.cuda.synchronize()
         return graph, out
 
-    gemm_mode, tuned = "library-default GEMM solutions", False
-    sub_batches = args.sub_batches if (not args.eager and args.sub_batches > 1 and args.batch % args.sub_batches == 0) else 1
+    tunable = None
+
+    def tune(net, inp):
+        """One untimed forward in which PyTorch's TunableOp times the library's own GEMM solutions for every GEMM shape
+        it meets and keeps the fastest.  The projection / MLP GEMMs of stages 2-4 stay PyTorch-ROCm library calls."""
+        if tunable is None:
+            return
+        tunable.tuning_enable(True)
+        net(inp)
+        torch.cuda.synchronize()
+        tunable.tuning_enable(False)
+
+    gemm_mode = "library-default GEMM solutions"
+    sub_batches = args.sub_batches if (args.sub_batches > 1 and args.batch % args.sub_batches == 0) else 1
+    modes = {}          # launch mode -> seconds for args.steps steps
     with torch.no_grad():
         model(x)
         torch.cuda.synchronize()
         log("first forward done")
         if not args.no_gemm_tuning:
-            # The projection / MLP GEMMs stay PyTorch-ROCm library calls; TunableOp only picks, per GEMM shape, the
-            # fastest of the library's own solutions.  Tuning happens in this one untimed forward.
             try:
-                import torch.cuda.tunable as tunable
-                tunable.enable(True)
-                tunable.tuning_enable(True)
+                import torch.cuda.tunable as tunable_mod
+                tunable_mod.enable(True)
                 for setter, value in (("set_filename", "/tmp/vmamba_amd_tunableop.csv"), ("set_max_tuning_duration", 60),
                                       ("set_max_tuning_iterations", 60)):
-                    if hasattr(tunable, setter):
-                        getattr(tunable, setter)(value)
+                    if hasattr(tunable_mod, setter):
+                        getattr(tunable_mod, setter)(value)
+                tunable = tunable_mod
                 t_tune = time.perf_counter()
-                model(x if sub_batches == 1 else x.chunk(sub_batches)[0])
-                torch.cuda.synchronize()
-                tunable.tuning_enable(False)
-                tuned = True
+                tune(model, x)
                 gemm_mode = "GEMM solutions picked by PyTorch TunableOp"
                 log(f"GEMM tuning forward: {time.perf_counter() - t_tune:.1f} s, {len(tunable.get_results())} shapes")
             except Exception as e:      # an optimisation of library calls, never a requirement
                 log(f"TunableOp unavailable ({type(e).__name__}: {e}); library-default GEMM solutions")
                 try:
-                    tunable.enable(False)
+                    tunable_mod.enable(False)
                 except Exception:
                     pass
-        graph, runner = None, None
-        if sub_batches > 1:
-            # candidates: the requested number of sub-batches and half of it; the faster validated runner is kept
+                tunable = None
+
+        # ---- mode 1: eager launches, exactly the reference's loop ------------------------------------------------
+        modes["eager"] = time_steps(lambda: model(x), args.warmup, args.steps)
+        log(f"eager launches: {modes['eager'] / args.steps * 1e3:.2f} ms/step")
+
+        # ---- mode 2: the forward as one captured HIP graph -------------------------------------------------------
+        graph = None
+        if not args.eager:
+            try:
+                captured = capture_forward(model, x)
+                if captured is None:
+                    log("graph replay did not reproduce the eager result; no one-graph figure")
+                else:
+                    graph = captured[0]
+                    modes["one_graph"] = time_steps(graph.replay, args.warmup, args.steps)
+                    log(f"one graph per forward: {modes['one_graph'] / args.steps * 1e3:.2f} ms/step")
+            except Exception as e:          # capture is an optimisation of the launch path, never a requirement
+                log(f"graph capture failed ({type(e).__name__}: {e})")
+
+        # ---- mode 3: sub-batch graphs side by side ---------------------------------------------------------------
+        runner = None
+        if not args.eager and sub_batches > 1:
             from vmamba_amd.runner import ConcurrentGraphRunner
             for n in sorted({sub_batches, max(2, sub_batches // 2)}, reverse=True):
                 if args.batch % n != 0:
                     continue
                 try:
-                    if tuned and n != sub_batches:      # GEMM shapes of this sub-batch size
-                        tunable.tuning_enable(True)
-                        model(x.chunk(n)[0])
-                        torch.cuda.synchronize()
-                        tunable.tuning_enable(False)
+                    tune(model, x.chunk(n)[0])          # GEMM shapes of this sub-batch size
                     cand = ConcurrentGraphRunner(model, x, n)
                     replay_err = cand.max_replay_error(replays=5)
                     log(f"{n} concurrent sub-batch graphs: {cand.step_ms:.2f} ms per step; vs eager forwards over 5 replays: "
                         f"max abs difference {replay_err:g}")
                     if replay_err != 0.0:       # bit for bit, or not at all
                         log(f"{n} concurrent sub-batch graphs did not reproduce the eager result")
-                        cand = None
                     elif runner is None or cand.step_ms < runner.step_ms:
                         runner = cand
                     cand = None
                 except Exception as e:          # an optimisation of the launch path, never a requirement
                     log(f"sub-batch graph capture failed ({type(e).__name__}: {e})")
-            if runner is None:
-                log("no sub-batch runner; one graph for the whole batch")
-            else:
+            if runner is not None:
                 sub_batches = len(runner.graphs)
-        if not args.eager and runner is None:
-            if tuned and sub_batches > 1:   # the GEMM shapes of the whole batch have not been tuned yet
-                tunable.tuning_enable(True)
-                model(x)
-                torch.cuda.synchronize()
-                tunable.tuning_enable(False)
-            try:
-                captured = capture_forward()
-            except Exception as e:          # capture is an optimisation of the launch path, never a requirement
-                log(f"graph capture failed ({type(e).__name__}: {e}); timing eager launches")
-                captured = None
-            if captured is None:
-                log("graph replay did not reproduce the eager result; timing eager launches")
-            else:
-                graph = captured[0]
-        step = runner.replay if runner is not None else graph.replay if graph is not None else (lambda: model(x))
-        for i in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-    launch_mode = (f"the batch as {sub_batches} sub-batches of {args.batch // sub_batches}, one captured HIP graph each, replayed "
-                   f"concurrently (the caller's stream + {sub_batches - 1} more)" if runner is not None
-                   else "one captured HIP graph per forward" if graph is not None else "eager launches")
+                modes["concurrent"] = time_steps(runner.replay, args.warmup, args.steps)
+                log(f"{sub_batches} sub-batch graphs side by side: {modes['concurrent'] / args.steps * 1e3:.2f} ms/step")
+
+    launch = min(modes, key=modes.get)
+    dt = modes[launch]
+    launch_text = dict(eager="eager launches", one_graph="one captured HIP graph per forward",
+                       concurrent=f"the batch as {sub_batches} sub-batches of {args.batch // sub_batches}, one captured HIP graph each, "
+                                  f"replayed side by side (the caller's stream + {sub_batches - 1} more); replays checked bit for bit "
+                                  f"against the eager sub-batch forwards before timing")[launch]
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    log(f"VMamba-T bs{args.batch}: {ms:.2f} ms/step, {value:.0f} img/s")
+    log(f"VMamba-T bs{args.batch}: {ms:.2f} ms/step, {value:.0f} img/s ({launch})")
+    ms_of = lambda k: modes[k] / args.steps * 1e3 if k in modes else None
+
+    # ---- benchmark config 4 and the fp32 forward (extra keys; eager launches, short runs) ---------------------------
+    extra = {}
+    if not args.no_extra_forwards:
+        with torch.no_grad():
+            try:
+                runner = graph = None
+                x4 = torch.randn(4, 3, 1024, 1024, device=dev).bfloat16()
+                model(x4)
+                tune(model, x4)
+                t4 = time_steps(lambda: model(x4), 5, 10) / 10
+                extra["config4"] = dict(workload="VMamba-T forward, 4 x 1024^2, bf16, eager launches (stage maps 256/128/64/32)",
+                                        ms_per_forward=t4 * 1e3, img_per_s=4 / t4)
+                log("config 4:", extra["config4"])
+                del x4
+            except Exception as e:
+                log(f"config-4 forward failed ({type(e).__name__}: {e})")
+            try:
+                model32 = model.float()
+                x32 = x.float()
+                model32(x32)
+                t32 = time_steps(lambda: model32(x32), 3, 10) / 10
+                extra["fp32"] = dict(workload=f"VMamba-T forward, batch {args.batch} @224^2, fp32 activations and weights (the reference "
+                                              f"harness's precision, no AMP), eager launches, {gemm_mode.split(' picked')[0]} as met",
+                                     ms_per_step=t32 * 1e3, img_per_s=args.batch / t32)
+                log("fp32:", extra["fp32"])
+                del x32, model32
+            except Exception as e:
+                log(f"fp32 forward failed ({type(e).__name__}: {e})")
+        torch.cuda.empty_cache()
 
     kernels, roofline, scan_roofline = None, None, None
     if not args.no_kernels:
         with torch.no_grad():
             kernels = kernel_lines(args.kernel_reps)
         k1 = kernels[0]
+        core_traffic, core_src = measured_traffic("ss2d_core_kernel@stage1")
+        scan_traffic, scan_src = measured_traffic("scan_row_kernel@stage1")
         roofline = dict(bound="hbm", kernel="ss2d_core_kernel<bf16> (CrossScan+scan+CrossMerge fused) @ stage1 (B=128, D=96, 56x56, K=4)",
                         achieved=k1["core_fused_GBs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                        frac=k1["core_fused_GBs"] / HBM_PEAK_GBS, traffic=CORE_STAGE1_MEASURED_TRAFFIC_BYTES,
+                        frac=k1["core_fused_GBs"] / HBM_PEAK_GBS, traffic=core_traffic, traffic_source=core_src,
                         bytes_per_launch=k1["core_fused_bytes"], us_per_launch=k1["core_fused_us"],
                         note="14 algorithmic bytes per element instead of the 62 of the three-operator path it replaces "
                              "(cross_scan + scan + cross_merge); the kernel is bound by VALU/transcendental issue, not HBM")
         scan_roofline = dict(bound="hbm", kernel="scan_row_kernel<bf16,f32,N=1> @ stage1 (B=128, KD=384, L=3136)",
                              achieved=k1["scan_GBs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=k1["scan_GBs"] / HBM_PEAK_GBS,
-                             traffic=SCAN_STAGE1_MEASURED_TRAFFIC_BYTES, bytes_per_launch=k1["scan_bytes"],
+                             traffic=scan_traffic, traffic_source=scan_src, bytes_per_launch=k1["scan_bytes"],
                              us_per_launch=k1["scan_us"])
-    cpu = None if args.no_cpu_baseline else cpu_baseline()
+    cpu, cpu_op, parity = None, None, None
+    if not args.no_cpu_baseline:
+        cpu_op, parity = cpu_baseline_op()
+        log("cpu_baseline_op", cpu_op)
+        with torch.no_grad():
+            parity["fused_core_bf16_bs128_vs_c_oracle"] = stage_parity()
+        log("parity", parity)
+        cpu = cpu_baseline()
 
     print(json.dumps({
         "metric": "VMamba-T img/s @224^2 bs128 on 1xMI355X; SS2D scan HBM GB/s vs peak",
         "value": value, "unit": "img/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"sub_batches": sub_batches if runner is not None else 1,
+        "config": {"launch": launch, "sub_batches": sub_batches if launch == "concurrent" else 1,
                    "workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
-                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_mode}, {gemm_mode}; "
+                               f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_text}, {gemm_mode}; "
                                f"SS2D core, LayerNorm, depthwise conv, patch-embedding stem, narrow-stage MLP and projections on HIP kernels"},
-        "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "kernels": kernels,
+        "ms_per_step_eager": ms_of("eager"), "ms_per_step_one_graph": ms_of("one_graph"),
+        "ms_per_step_concurrent": ms_of("concurrent"), **extra,
+        "roofline": roofline, "scan_roofline": scan_roofline, "cpu_baseline": cpu, "cpu_baseline_op": cpu_op,
+        "parity": parity, "kernels": kernels,
     }))
 
 

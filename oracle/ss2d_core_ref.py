@@ -1,7 +1,8 @@
 """TEST INFRASTRUCTURE ONLY -- the SS2D block and model composed from torch-on-CPU reference operators.
 
-``RefSS2D`` is the package's SS2D block with ``forward_core`` replaced by the torch restatement
-(oracle/torch_ref.py) in the order of classification/models/vmamba.py:603-646, and ``TorchLayers`` supplies
+``RefSS2D`` takes only the parameter set (names, shapes, initialisation) from the package's SS2D block; its
+``forward`` / ``forward_core`` are restated here from classification/models/vmamba.py:603-663 on the torch
+restatement of the three operators (oracle/torch_ref.py) with the projections as the reference's einsums, and ``TorchLayers`` supplies
 the reference's own norm layers (nn.LayerNorm; LayerNorm2d = permute, F.layer_norm, permute, vmamba.py:52-57)
 instead of the package's HIP ones.  It is what model-level parity tests compare against and what the benchmark
 times as the "reference torch CPU path".
@@ -43,19 +44,43 @@ class TorchLayers:
 
 
 class RefSS2D(SS2D):
+    """Holds the parameters of the package's block (so state dicts are interchangeable) but computes nothing with the
+    package's forward code: ``forward_core`` and ``forward`` below are written from the reference's text."""
+
     def __init__(self, *args, **kwargs):
         kwargs.setdefault("layers", TorchLayers)
         super().__init__(*args, **kwargs)
 
     def forward_core(self, x):
+        # vmamba.py:603-646, the cross2d / non-cascade branch in its einsum spelling (:610-615)
         B, D, H, W = x.shape
-        K, L = self.k_group, H * W
-        xs = torch_ref.cross_scan(x)
-        dts, Bs, Cs = self.project(xs.contiguous())
-        ys = torch_ref.selective_scan(xs.reshape(B, K * D, L), dts, -self.A_logs.float().exp(), Bs.contiguous(),
-                                      Cs.contiguous(), self.Ds.float(), self.dt_projs_bias.view(-1).float(), True)
-        y = torch_ref.cross_merge(ys.view(B, K, D, H, W))
-        return self.finish_core(y, B, D, H, W, x.dtype)
+        K, L, R, N = self.k_group, H * W, self.dt_rank, self.d_state
+        xs = torch_ref.cross_scan(x)                                                         # (B, K, D, L)
+        x_dbl = torch.einsum("b k d l, k c d -> b k c l", xs, self.x_proj_weight)
+        dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
+        dts = torch.einsum("b k r l, k d r -> b k d l", dts, self.dt_projs_weight)
+        ys = torch_ref.selective_scan(xs.reshape(B, K * D, L), dts.contiguous().view(B, K * D, L),
+                                      -self.A_logs.float().exp(), Bs.contiguous(), Cs.contiguous(), self.Ds.float(),
+                                      self.dt_projs_bias.view(-1).float(), True)
+        y = torch_ref.cross_merge(ys.view(B, K, D, H, W))                                    # (B, D, L)
+        return TorchLayers.out_norm(self.out_norm, y.view(B, D, H, W), self.channel_first, x.dtype)
+
+    def forward(self, x, residual=None, pre_norm=None, post_norm=None):
+        # vmamba.py:648-663 (forwardv2), with the block's norms and residual of VSSBlock._forward (:1225-1229)
+        h = x if pre_norm is None else pre_norm(x)
+        h = self.in_proj(h)
+        z = None
+        if not self.disable_z:
+            h, z = h.chunk(2, dim=(1 if self.channel_first else -1))
+            z = self.act(z)
+        h = TorchLayers.conv_act(self.conv2d if self.with_dconv else None, h, self.channel_first)
+        y = self.forward_core(h)
+        if z is not None:
+            y = y * z
+        out = self.out_proj(y)
+        if residual is not None:
+            out = residual + out
+        return out if post_norm is None else (out, post_norm(out))
 
 
 def reference_vmamba_tiny(channel_first=True):

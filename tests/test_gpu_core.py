@@ -154,6 +154,82 @@ def test_core_equals_three_kernels_at_model_shape():
         assert torch.allclose(got, want, **TOL), f"max abs err {err}"
 
 
+# Benchmark configurations 1 and 2 at their own batch: the fused kernel picks its tile (images per workgroup) from the
+# batch -- 1 / 2 / 10 / 40 images at the four stage shapes, with a shorter last tile of 8 at the last two -- so the
+# tiles the benchmark runs only exist at B = 128.  Image ranges below cover the first tile, an interior tile and the
+# last (short) tile of every shape, and more than one tile where tiles are small.
+BENCH_TILES = [
+    ((128, 96, 56, 56), [(0, 2), (64, 66), (126, 128)]),
+    ((128, 192, 28, 28), [(0, 4), (62, 66), (124, 128)]),
+    ((128, 384, 14, 14), [(0, 10), (60, 70), (118, 128)]),
+    ((128, 768, 7, 7), [(0, 40), (40, 80), (118, 128)]),
+]
+
+
+@pytest.mark.parametrize("shape,ranges", BENCH_TILES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else None)
+def test_core_matches_oracle_at_benchmark_batch(shape, ranges):
+    """bf16, B = 128: the fused kernel against the CPU oracle's composition on whole tiles of images."""
+    B, D, H, W = shape
+    L = H * W
+    _announce("core bench-batch", shape)
+    g = torch.Generator(device=DEV).manual_seed(B + D + H)
+    rn = lambda *s: torch.randn(*s, generator=g, device=DEV)
+    x, delta = rn(B, D, H, W).bfloat16(), rn(4, D, B, L).bfloat16()
+    Bs, Cs = rn(4, B, L).bfloat16(), rn(4, B, L).bfloat16()
+    _, _, _, _, A, Dv, bias = make_core_inputs(B + D, 1, D, 2, 4, torch.bfloat16)       # the per-channel constants
+    got = ss2d_core_hip(x, delta, Bs, Cs, A.to(DEV), Dv.to(DEV), bias.to(DEV), True)
+    torch.cuda.synchronize()
+    assert got.shape == (B, D, L) and got.dtype == torch.float32
+    for b0, b1 in ranges:
+        want = oracle_core(x[b0:b1].cpu(), delta[:, :, b0:b1].cpu().contiguous(), Bs[:, b0:b1].cpu().contiguous(),
+                           Cs[:, b0:b1].cpu().contiguous(), A, Dv, bias)
+        err = (got[b0:b1].cpu() - want).abs().max().item()
+        assert torch.allclose(got[b0:b1].cpu(), want, **TOL), f"images {b0}..{b1 - 1}: max abs err {err}"
+
+
+def test_benchmark_config0_three_operators_and_fused_core():
+    """Benchmark config 0 verbatim: fp32, x (2, 96, 56, 56) ~ N(0,1) -> CrossScan -> u (2, 384, 3136); delta_raw ~ N(0,1);
+    dt log-uniform in [1e-3, 0.1], delta_bias = softplus^-1(dt); A = -exp(log 1) = -1; B, C (2, 4, 1, 3136) ~ N(0,1);
+    D = 1; selective scan with softplus; CrossMerge back to (2, 96, 3136).  Both GPU paths against the CPU oracle
+    (tolerances of kernels/selective_scan/test_selective_scan.py:401-403, fp32: rtol 1e-3; the permutation bit-exact,
+    the merge bit-exact on the GPU's own scan output)."""
+    import math
+    _announce("config0")
+    Bsz, Dn, H, W, K, N = 2, 96, 56, 56, 4, 1
+    L = H * W
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(Bsz, Dn, H, W, generator=g)
+    delta = torch.randn(Bsz, K * Dn, L, generator=g)
+    dt = torch.exp(torch.rand(K * Dn, generator=g) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3))
+    bias = dt + torch.log(-torch.expm1(-dt))
+    A = -torch.exp(torch.log(torch.arange(1, N + 1, dtype=torch.float32))).repeat(K * Dn, 1)
+    Bm, Cm = torch.randn(Bsz, K, N, L, generator=g), torch.randn(Bsz, K, N, L, generator=g)
+    Dv = torch.ones(K * Dn)
+    # CPU oracle
+    xs_ref = orc.cross_scan(x)
+    ys_ref = orc.selective_scan(xs_ref.view(Bsz, K * Dn, L), delta, A, Bm, Cm, Dv, bias, True)
+    y_ref = orc.cross_merge(ys_ref.view(Bsz, K, Dn, H, W))
+    # the torch restatement agrees with the C oracle on this very input (two formulations, one answer)
+    assert torch.equal(torch_ref.cross_scan(x), xs_ref)
+    # GPU: three operators
+    dev = lambda t: t.to(DEV)
+    xs = va.cross_scan_fn(dev(x))
+    ys = va.selective_scan_fn(xs.view(Bsz, K * Dn, L), dev(delta), dev(A), dev(Bm), dev(Cm), dev(Dv), dev(bias), True)
+    y = va.cross_merge_fn(ys.view(Bsz, K, Dn, H, W))
+    torch.cuda.synchronize()
+    assert torch.equal(xs.cpu(), xs_ref)
+    assert torch.allclose(ys.cpu(), ys_ref, rtol=1e-3, atol=1e-4), f"scan max abs err {(ys.cpu() - ys_ref).abs().max().item()}"
+    assert torch.equal(y.cpu(), orc.cross_merge(ys.cpu().view(Bsz, K, Dn, H, W)))
+    assert torch.allclose(y.cpu(), y_ref, **TOL)
+    # GPU: the fused kernel, projections handed over direction-major and batch-innermost
+    delta_k = delta.view(Bsz, K, Dn, L).permute(1, 2, 0, 3).contiguous()
+    B_k, C_k = Bm.view(Bsz, K, L).permute(1, 0, 2).contiguous(), Cm.view(Bsz, K, L).permute(1, 0, 2).contiguous()
+    y_fused = ss2d_core_hip(dev(x), dev(delta_k), dev(B_k), dev(C_k), dev(A.view(-1)), dev(Dv), dev(bias), True)
+    torch.cuda.synchronize()
+    err = (y_fused.cpu() - y_ref).abs().max().item()
+    assert torch.allclose(y_fused.cpu(), y_ref, **TOL), f"fused core max abs err {err}"
+
+
 def test_core_rejections():
     x, delta, Bs, Cs, A, Dv, bias = [t.to(DEV) for t in make_core_inputs(1, 2, 2, 4, 4, torch.bfloat16)]
     with pytest.raises(RuntimeError):

@@ -11,6 +11,16 @@ Which hardware queue a new stream lands on matters: the runtime deals its few ha
 turn, and a worker stream that shares its queue with the caller's stream queues up behind the joins the caller's stream
 carries -- its next launch then waits for the other sub-batches (measured: 6.7-7.0 ms per step instead of 5.4).  The
 mapping cannot be queried, so the runner times a few sets of freshly created streams and keeps the fastest.
+
+What a graph bakes in, and how the runner keeps it valid:
+  * library scratch.  PyTorch hands rocBLAS / hipBLASLt one workspace per (handle, stream); a GEMM captured on a stream
+    records that workspace's address.  Every sub-batch is therefore warmed up and captured on a stream of its own, kept
+    for the runner's lifetime and used for nothing else: graphs that replay side by side never share a workspace, and no
+    eager work ever touches one.
+  * per-module constants.  The SS2D blocks cache small tensors derived from their parameters; a capture pins the ones it
+    reads (``SS2D._inference_constants``) so that cache eviction cannot free them under a live graph.
+  * parameter values.  Those pinned constants are copies: after an in-place parameter update a replay would mix fresh
+    weights with stale copies, so ``replay()`` checks the parameters' version counters and refuses.
 """
 import time
 
@@ -32,9 +42,9 @@ class ConcurrentGraphRunner:
         self.graphs, self.outs = [], []
         dev = x.device
         cur = torch.cuda.current_stream(dev)
-        capture_stream = torch.cuda.Stream(device=dev)
+        self.capture_streams = [torch.cuda.Stream(device=dev) for _ in self.chunks]     # one per graph, never reused
         with torch.no_grad():
-            for c in self.chunks:
+            for c, capture_stream in zip(self.chunks, self.capture_streams):
                 capture_stream.wait_stream(cur)
                 with torch.cuda.stream(capture_stream):
                     for _ in range(warmup):
@@ -47,6 +57,8 @@ class ConcurrentGraphRunner:
                 self.graphs.append(g)
                 self.outs.append(out)
         torch.cuda.synchronize(dev)
+        self._params = [p for p in model.parameters()]
+        self._versions = [p._version for p in self._params]
         self.streams = self._pick_streams(sub_batches - 1, stream_sets)
         self.step_ms = self._time_step(self.streams) if sub_batches > 1 else None
 
@@ -90,7 +102,14 @@ class ConcurrentGraphRunner:
                 best = (ms, streams)
         return best[1]
 
+    def parameters_unchanged(self):
+        """False once any parameter of the model was updated in place after the capture."""
+        return all(p._version == v for p, v in zip(self._params, self._versions))
+
     def replay(self):
+        if not self.parameters_unchanged():
+            raise RuntimeError("ConcurrentGraphRunner: a parameter of the model changed after the graphs were captured; "
+                               "they hold copies derived from the old values -- build a new runner")
         self._replay_on(self.streams)
 
     def output(self):

@@ -20,6 +20,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from ._lib import SS2D_ENOTSUP, Ss2dError
 from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
@@ -119,11 +120,24 @@ class SS2D(nn.Module):
         """Tensors that depend only on the parameters (and the batch size): A = -exp(A_logs), fp32 D and dt bias
         (vmamba.py:619-623) and the projection weights repeated over the batch so each projection is ONE
         strided-batched GEMM over B*K problems.  Recomputed whenever autograd is on or a parameter changed; kept for up to
-        four batch sizes."""
+        four batch sizes.
+
+        Under a graph capture the kernels record the addresses of these tensors.  An entry the capture reads is therefore
+        moved to ``_pinned_consts``, which never evicts, so it outlives any graph that holds its address; an entry
+        missing during a capture is computed inside the graph (its memory then belongs to the graph and is rewritten by
+        every replay) and is not kept.  Pinned entries are copies of the parameter values at capture time: whoever
+        replays the graph must not do so after an in-place parameter update (ConcurrentGraphRunner.replay checks)."""
         params = (self.A_logs, self.Ds, self.dt_projs_bias, self.x_proj_weight, self.dt_projs_weight)
         key = (batch, torch.is_grad_enabled(), tuple((p._version, p.data_ptr(), p.dtype, p.device) for p in params))
         cache = self.__dict__.setdefault("_const_cache", {})
+        pinned = self.__dict__.setdefault("_pinned_consts", {})
+        capturing = self.A_logs.is_cuda and torch.cuda.is_current_stream_capturing()
+        if key in pinned:
+            return pinned[key]
         if key in cache:
+            if capturing:
+                pinned[key] = cache.pop(key)
+                return pinned[key]
             return cache[key]
         K = self.k_group
         consts = dict(
@@ -131,9 +145,6 @@ class SS2D(nn.Module):
             Wx_all=self.x_proj_weight.reshape(1, -1, self.d_inner).expand(batch, -1, -1).contiguous(),
             Wx=self.x_proj_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, -1, self.d_inner).contiguous(),
             Wdt=self.dt_projs_weight.unsqueeze(0).expand(batch, -1, -1, -1).reshape(batch * K, self.d_inner, -1).contiguous())
-        # kept per batch size (sub-batches of a runner alternate with whole batches); never from inside a graph capture,
-        # whose allocations live in the graph's memory pool and are overwritten by its replays
-        capturing = consts["As"].is_cuda and torch.cuda.is_current_stream_capturing()
         if not torch.is_grad_enabled() and not capturing:
             stale = [k for k in cache if k[2] != key[2]]
             for k in stale:
@@ -208,7 +219,11 @@ class SS2D(nn.Module):
         K, L = self.k_group, H * W
         consts = self._inference_constants(B)
         if self._fused_core_applies(x):
-            return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
+            try:
+                return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
+            except Ss2dError as e:          # a shape the fused kernel has no variant for: the three operators take it
+                if e.code != SS2D_ENOTSUP:
+                    raise
         xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
         dts, Bs, Cs = self.project_from_map(x, consts)
         ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
@@ -270,9 +285,15 @@ class SS2D(nn.Module):
         if z is None and self._norm_proj_fusable(x, residual):
             # out_norm, out_proj and the residual add in one kernel, straight from the core's fp32 map
             B, _, H, W = x.shape
-            y = self.forward_core_fused(x, self._inference_constants(B))                        # (B, D, L) fp32
-            return linear_cf_ln_hip(y, self.out_norm.weight, self.out_norm.bias, self.out_norm.eps, self.out_proj.weight,
-                                    self.out_proj.bias, residual).view(B, H, W, self.d_model)
+            try:
+                y = self.forward_core_fused(x, self._inference_constants(B))                    # (B, D, L) fp32
+            except Ss2dError as e:          # no fused variant for this shape: forward_core's three-operator path below
+                if e.code != SS2D_ENOTSUP:
+                    raise
+                y = None
+            if y is not None:
+                return linear_cf_ln_hip(y, self.out_norm.weight, self.out_norm.bias, self.out_norm.eps, self.out_proj.weight,
+                                        self.out_proj.bias, residual).view(B, H, W, self.d_model)
         y = self.forward_core(x)
         if z is not None:
             y = y * z
