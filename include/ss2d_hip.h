@@ -39,6 +39,7 @@ extern "C" {
 #define SS2D_EINVAL (-22)  /* bad shape, stride, pointer or flag            */
 #define SS2D_ENOTSUP (-95) /* valid request this build has no kernel for    */
 #define SS2D_ELAUNCH (-5)  /* the HIP runtime refused the launch            */
+#define SS2D_ENOMEM (-12)  /* the workspace is smaller than the call needs  */
 
 /* CrossMerge association orders */
 #define SS2D_MERGE_PAIRWISE 0      /* (y0 + flip y2) + T(y1 + flip y3): cross_merge_fwd,
@@ -257,6 +258,20 @@ int ss2d_cross_scan_flex(const void *x, void *y, int B, int C, int H, int W, int
                          int y_channel_last, int one_by_one, int scans, void *stream);
 int ss2d_cross_merge_flex(const void *y, void *x, int B, int C, int H, int W, int dtype, int x_channel_last,
                           int y_channel_last, int one_by_one, int scans, int order, void *stream);
+
+/*
+ * ss2d_cross_scan_flex with a staging buffer for the mixed-layout modes (x channel-first and y channel-last, or the
+ * reverse: the permute(...).contiguous() the reference inserts, classification/models/csm_triton.py:48-51, 116-119).
+ * The x-side tensor is first transposed into `workspace` (the layout of y), then the same-layout kernel runs: two
+ * copy-shaped launches instead of one gather through L2 (4-5x faster at model shapes).  Results are identical to
+ * ss2d_cross_scan_flex (a permutation).  `workspace`: device memory, 16-byte aligned, at least
+ * B * (one_by_one ? 4 : 1) * C * H * W * elem_bytes bytes; it is scratch (contents undefined afterwards) and must not be
+ * used by other work until the call's launches have finished.  SS2D_ENOMEM when workspace_bytes is too small.  When the two
+ * layouts agree the workspace is not touched (it may be NULL) and the call is ss2d_cross_scan_flex.
+ */
+int ss2d_cross_scan_flex_ws(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                            int y_channel_last, int one_by_one, int scans, void *workspace, int64_t workspace_bytes,
+                            void *stream);
 
 /*
  * Batched transpose (B, R, S) -> (B, S, R), any 1/2/4/8-byte element: the layout change between channel-first

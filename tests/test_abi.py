@@ -57,6 +57,22 @@ def test_cross_merge_argument_validation():
     assert L.ss2d_cross_merge(None, None, 1, 1, 1, 1, _lib.SS2D_F32, 2, None) == _lib.SS2D_EINVAL  # order
 
 
+def test_cross_scan_flex_workspace_validation():
+    """ss2d_cross_scan_flex_ws: argument and workspace checks happen before anything is launched."""
+    L = _lib.lib()
+    ws = ctypes.c_void_p(256)       # never dereferenced: every call below is refused first
+    mixed = (0, 1, 0, 0)            # x channel-first, y channel-last
+    assert L.ss2d_cross_scan_flex_ws(None, None, 0, 3, 4, 4, 2, *mixed, None, 0, None) == _lib.SS2D_OK       # empty
+    assert L.ss2d_cross_scan_flex_ws(None, None, 1, 3, 4, 4, 3, *mixed, ws, 1 << 20, None) == _lib.SS2D_EINVAL  # element size
+    assert L.ss2d_cross_scan_flex_ws(None, None, 1, 3, 4, 4, 2, 0, 2, 0, 0, ws, 1 << 20, None) == _lib.SS2D_EINVAL  # flag
+    assert L.ss2d_cross_scan_flex_ws(ws, ws, 1, 3, 4, 4, 2, *mixed, None, 1 << 20, None) == _lib.SS2D_EINVAL    # no workspace
+    assert L.ss2d_cross_scan_flex_ws(ws, ws, 1, 3, 4, 4, 2, *mixed, ctypes.c_void_p(260), 1 << 20, None) == _lib.SS2D_EINVAL  # alignment
+    need = 1 * 3 * 16 * 2
+    assert L.ss2d_cross_scan_flex_ws(ws, ws, 1, 3, 4, 4, 2, *mixed, ws, need - 1, None) == _lib.SS2D_ENOMEM
+    assert L.ss2d_cross_scan_flex_ws(ws, ws, 1, 3, 4, 4, 2, 0, 1, 1, 0, ws, 4 * need - 1, None) == _lib.SS2D_ENOMEM  # one-by-one: 4 slices
+    assert "workspace" in _lib.strerror(_lib.SS2D_ENOMEM)
+
+
 def test_scan_argument_validation():
     L = _lib.lib()
     assert L.ss2d_selective_scan_fwd(None, None) == _lib.SS2D_EINVAL

@@ -55,6 +55,34 @@ def test_cross_merge_every_mode_bit_exact(icf, ocf, obo, scans, dtype):
             assert torch.equal(got.cpu(), want), (B, C, H, W)
 
 
+@pytest.mark.parametrize("x_cl,obo,scans", [(0, 0, 0), (1, 0, 0), (0, 1, 0), (1, 1, 0), (0, 0, 2), (1, 0, 1), (1, 1, 2)])
+def test_staged_mixed_layout_scan_equals_the_route_kernel(x_cl, obo, scans):
+    """ss2d_cross_scan_flex_ws (transpose into the workspace + same-layout kernel) against ss2d_cross_scan_flex (one
+    gather) through the C ABI: the same permutation, bit for bit; a workspace larger than needed is fine."""
+    print("CASE scan-flex-ws", x_cl, obo, scans, flush=True)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    for (B, C, H, W) in [(2, 96, 14, 14), (3, 5, 7, 9), (1, 130, 5, 13)]:
+        K = 4 if obo else 1
+        x = torch.randint(-30000, 30000, (B * K * C * H * W,), dtype=torch.int16, device=DEV)
+        want = torch.empty(B * 4 * C * H * W, dtype=torch.int16, device=DEV)
+        got = torch.full_like(want, 7)
+        ws = torch.empty(x.numel() + 64, dtype=torch.int16, device=DEV)
+        y_cl = 1 - x_cl
+        assert L.ss2d_cross_scan_flex(x.data_ptr(), want.data_ptr(), B, C, H, W, 2, x_cl, y_cl, obo, scans, stream) == 0
+        assert L.ss2d_cross_scan_flex_ws(x.data_ptr(), got.data_ptr(), B, C, H, W, 2, x_cl, y_cl, obo, scans, ws.data_ptr(),
+                                         ws.numel() * 2, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (B, C, H, W)
+    # same layout on both sides: the workspace is not needed
+    x = torch.randint(-9, 9, (2 * 3 * 4 * 5,), dtype=torch.int16, device=DEV)
+    a, b = torch.empty(2 * 4 * 3 * 20, dtype=torch.int16, device=DEV), torch.empty(2 * 4 * 3 * 20, dtype=torch.int16, device=DEV)
+    assert L.ss2d_cross_scan_flex(x.data_ptr(), a.data_ptr(), 2, 3, 4, 5, 2, 1, 1, 0, 0, stream) == 0
+    assert L.ss2d_cross_scan_flex_ws(x.data_ptr(), b.data_ptr(), 2, 3, 4, 5, 2, 1, 1, 0, 0, None, 0, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
 def test_cross_merge_flex_left_to_right_order():
     y = torch.randn(2, 7, 5, 4, 6, generator=torch.Generator().manual_seed(1)).bfloat16()
     want = torch_ref.cross_merge_flex(y, False, False, False, 0, left_to_right=True)

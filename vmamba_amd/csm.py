@@ -56,20 +56,22 @@ def transpose_bcl_hip(x):
 
 
 def cross_scan_flex_hip(x, in_channel_first=True, out_channel_first=True, one_by_one=False, scans=0):
-    """Any layout / mode of CrossScan; bit-exact for any 1/2/4/8-byte dtype.  Mixed layouts first bring x (the small
-    side) to the layout of y with one tiled transpose, then run the same-layout kernel."""
+    """Any layout / mode of CrossScan; bit-exact for any 1/2/4/8-byte dtype.  Mixed layouts go through
+    ss2d_cross_scan_flex_ws, which first brings x (the small side) to the layout of y with one tiled transpose into a
+    staging buffer allocated here, then runs the same-layout kernel."""
     _require_gpu(x, "cross_scan")
     B, C, H, W = _flex_dims(x, in_channel_first, one_by_one, "cross_scan")
     x = x.contiguous()
     if in_channel_first != out_channel_first and x.numel():
-        K = 4 if one_by_one else 1
-        if in_channel_first:      # (B, K*C, L) -> (B, L, K*C)
-            x = transpose_bcl_hip(x.view(B, K * C, H * W)).view((B, H, W, 4, C) if one_by_one else (B, H, W, C))
-        else:                     # (B, L, K*C) -> (B, K*C, L)
-            x = transpose_bcl_hip(x.view(B, H * W, K * C)).view((B, 4, C, H, W) if one_by_one else (B, C, H, W))
-        in_channel_first = out_channel_first
-        if in_channel_first and scans == 0:
-            return cross_scan_1b1_hip(x) if one_by_one else cross_scan_hip(x)
+        y = x.new_empty((B, 4, C, H * W) if out_channel_first else (B, H * W, 4, C))
+        staging = torch.empty_like(x)          # one copy of x in the layout of y
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().ss2d_cross_scan_flex_ws(x.data_ptr(), y.data_ptr(), B, C, H, W, x.element_size(),
+                                                    0 if in_channel_first else 1, 0 if out_channel_first else 1,
+                                                    1 if one_by_one else 0, scans, staging.data_ptr(),
+                                                    staging.numel() * staging.element_size(), _stream(x))
+        _lib.check(rc, "ss2d_cross_scan_flex_ws")
+        return y
     y = x.new_empty((B, 4, C, H * W) if out_channel_first else (B, H * W, 4, C))
     with torch.cuda.device(x.device):
         rc = _lib.lib().ss2d_cross_scan_flex(x.data_ptr(), y.data_ptr(), B, C, H, W, x.element_size(),

@@ -305,3 +305,52 @@ extern "C" int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, i
     }
     return launch_status();
 }
+
+// ---- mixed layouts through a staging buffer --------------------------------------------------------------------
+// When x and y differ in layout the route kernel above gathers across the innermost axis of its source (through L2,
+// 4-5x slower than the copy-shaped cases).  Staged instead: the x-side tensor -- the small side, a fifth of the traffic
+// -- is first brought to the layout of y with the tiled transpose, then the same-layout kernel runs.  The staging buffer
+// holds one copy of x and is the caller's (a workspace argument).
+namespace ss2d {
+
+// Bytes of staging a mixed-layout CrossScan needs (0 when the layouts agree); negative status on bad arguments.
+static int64_t cross_scan_staging_bytes(int B, int C, int H, int W, int elem_bytes, int x_cl, int y_cl, int one_by_one, int scans) {
+    FlexArgs a;
+    const int rc = flex_fill(a, B, C, H, W, x_cl, y_cl, one_by_one, scans);
+    if (rc != SS2D_OK) return rc;
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return SS2D_EINVAL;
+    if (x_cl == y_cl) return 0;
+    return (int64_t)B * (one_by_one ? 4 : 1) * C * a.L * elem_bytes;
+}
+
+// The two launches.  Every limit either launch would refuse is checked before the first, so an error leaves nothing
+// enqueued.  `staging` must hold cross_scan_staging_bytes(...) bytes, 16-byte aligned.
+static int cross_scan_flex_staged(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_cl, int y_cl,
+                                  int one_by_one, int scans, void *staging, void *stream) {
+    const int64_t L = (int64_t)H * W, KC = (int64_t)(one_by_one ? 4 : 1) * C;
+    if (KC > 0x7fffffff || (int64_t)B * 4 * C * L > 0xffffffffll) return SS2D_ENOTSUP;
+    const int64_t r = x_cl ? L : KC, sdim = x_cl ? KC : L;           // x as (B, r, sdim) -> staging (B, sdim, r)
+    if ((int64_t)B * ((r + 63) / 64) * ((sdim + 63) / 64) > 0x7fffffff) return SS2D_ENOTSUP;
+    int rc = ss2d_transpose_bcl(x, staging, B, (int)r, (int)sdim, elem_bytes, stream);
+    if (rc != SS2D_OK) return rc;
+    if (y_cl) return ss2d_cross_scan_flex(staging, y, B, C, H, W, elem_bytes, 1, 1, one_by_one, scans, stream);
+    if (scans != 0) return ss2d_cross_scan_flex(staging, y, B, C, H, W, elem_bytes, 0, 0, one_by_one, scans, stream);
+    if (one_by_one) return ss2d_cross_scan_1b1(staging, y, B, C, H, W, elem_bytes, 4 * (int64_t)C * L, (int64_t)C * L, L, stream);
+    return ss2d_cross_scan(staging, y, B, C, H, W, elem_bytes, stream);
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_cross_scan_flex_ws(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                                       int y_channel_last, int one_by_one, int scans, void *workspace, int64_t workspace_bytes,
+                                       void *stream) {
+    using namespace ss2d;
+    const int64_t need = cross_scan_staging_bytes(B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans);
+    if (need < 0) return (int)need;
+    if (need == 0) return ss2d_cross_scan_flex(x, y, B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans, stream);
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (!x || !y) return SS2D_EINVAL;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) return SS2D_EINVAL;
+    if (workspace_bytes < need) return SS2D_ENOMEM;
+    return cross_scan_flex_staged(x, y, B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans, workspace, stream);
+}

@@ -598,6 +598,7 @@ extern "C" const char *ss2d_strerror(int code) {
         case SS2D_EINVAL: return "invalid argument (shape, stride, dtype, pointer or flag)";
         case SS2D_ENOTSUP: return "request is valid but not supported by this build";
         case SS2D_ELAUNCH: return "HIP runtime refused the kernel launch";
+        case SS2D_ENOMEM: return "workspace too small for this call (see the entry point's size rule)";
         default: return "unknown ss2d status";
     }
 }
