@@ -274,6 +274,22 @@ int ss2d_cross_scan_flex_ws(const void *x, void *y, int B, int C, int H, int W, 
                             void *stream);
 
 /*
+ * ss2d_cross_scan_flex_ws without the workspace argument: the staging buffer is a fixed array of
+ * SS2D_STATIC_STAGING_BYTES in device memory that belongs to the library (each GPU the library runs on holds its own
+ * copy until the process ends).  This entry point has no counterpart in the reference; it exists for callers that
+ * cannot allocate device memory around the call -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It calls no hipMalloc / hipFree or any allocating routine.  Same results as
+ * ss2d_cross_scan_flex.  SS2D_ENOMEM when the x-side tensor, B * (one_by_one ? 4 : 1) * C * H * W * elem_bytes bytes,
+ * exceeds SS2D_STATIC_STAGING_BYTES (nothing is launched then); same-layout modes need no staging and have no limit.
+ * All calls on one GPU share that GPU's array: calls whose launches can overlap on one GPU (different streams without
+ * an ordering between them) race on it.  The first call on a device looks up the array's address; make that call
+ * outside a graph capture.
+ */
+#define SS2D_STATIC_STAGING_BYTES (80 << 20)
+int ss2d_cross_scan_flex_static(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                                int y_channel_last, int one_by_one, int scans, void *stream);
+
+/*
  * Batched transpose (B, R, S) -> (B, S, R), any 1/2/4/8-byte element: the layout change between channel-first
  * (B, C, L) and channel-last (B, L, C) activations -- the permute(...).contiguous() of cross_scan_fwd / cross_merge_fwd
  * for mixed layouts (classification/models/csm_triton.py:48-51, 80-83).  The host serves the mixed-layout modes as

@@ -1,0 +1,61 @@
+"""ss2d_cross_scan_flex_static -- the entry point that allocates nothing (its staging buffer is a fixed device array
+inside the library) -- through the C ABI against ss2d_cross_scan_flex, the entry point it is a variant of: the same
+permutation, bit for bit, on two calls in a row, the second with a smaller input (the array keeps the first call's
+contents), and a clean refusal above the array's size."""
+import gc
+
+import pytest
+import torch
+
+from vmamba_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _pair(L, stream, shape, x_cl, obo, scans, seed):
+    B, C, H, W = shape
+    K = 4 if obo else 1
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.randint(-30000, 30000, (B * K * C * H * W,), dtype=torch.int16, device=DEV, generator=g)
+    want = torch.empty(B * 4 * C * H * W, dtype=torch.int16, device=DEV)
+    got = torch.full_like(want, 7)
+    y_cl = 1 - x_cl
+    assert L.ss2d_cross_scan_flex(x.data_ptr(), want.data_ptr(), B, C, H, W, 2, x_cl, y_cl, obo, scans, stream) == _lib.SS2D_OK
+    return x, want, got, (B, C, H, W, 2, x_cl, y_cl, obo, scans)
+
+
+@pytest.mark.parametrize("x_cl,obo,scans", [(0, 0, 0), (1, 0, 0), (1, 1, 0), (0, 1, 2)])
+def test_static_staging_matches_route_kernel_twice_in_a_row(x_cl, obo, scans):
+    print("CASE no-alloc", x_cl, obo, scans, flush=True)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    big = _pair(L, stream, (4, 96, 28, 28), x_cl, obo, scans, 1)
+    small = _pair(L, stream, (2, 5, 7, 9), x_cl, obo, scans, 2)         # inputs and outputs exist before the calls
+    torch.cuda.synchronize()
+    gc.collect()                                    # garbage of earlier tests must not be freed between the two readings
+    before = torch.cuda.memory_allocated()
+    for x, want, got, args in (big, small):
+        assert L.ss2d_cross_scan_flex_static(x.data_ptr(), got.data_ptr(), *args, stream) == _lib.SS2D_OK
+    assert torch.cuda.memory_allocated() <= before           # nothing came from torch's allocator either
+    torch.cuda.synchronize()
+    for x, want, got, args in (big, small):
+        assert torch.equal(got, want), args
+
+
+def test_static_staging_size_limit_and_same_layout():
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    x = torch.zeros(64, dtype=torch.int16, device=DEV)
+    # x-side tensor of 81 MiB: refused before anything is launched (the pointers are never followed)
+    assert L.ss2d_cross_scan_flex_static(x.data_ptr(), x.data_ptr(), 81, 1 << 9, 32, 32, 2, 0, 1, 0, 0, stream) == _lib.SS2D_ENOMEM
+    # exactly the limit is accepted as a size: 80 MiB as one-by-one slices would need real tensors, so only the arithmetic
+    # is probed through an argument error that is checked later than the size (a null pointer)
+    assert L.ss2d_cross_scan_flex_static(None, None, 80, 1 << 9, 32, 32, 2, 0, 1, 0, 0, stream) == _lib.SS2D_EINVAL
+    # same layout on both sides: no staging, plain ss2d_cross_scan_flex
+    x = torch.randint(-9, 9, (2 * 3 * 4 * 5,), dtype=torch.int16, device=DEV)
+    a, b = torch.empty(2 * 4 * 3 * 20, dtype=torch.int16, device=DEV), torch.empty(2 * 4 * 3 * 20, dtype=torch.int16, device=DEV)
+    assert L.ss2d_cross_scan_flex(x.data_ptr(), a.data_ptr(), 2, 3, 4, 5, 2, 0, 0, 0, 2, stream) == 0
+    assert L.ss2d_cross_scan_flex_static(x.data_ptr(), b.data_ptr(), 2, 3, 4, 5, 2, 0, 0, 0, 2, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)

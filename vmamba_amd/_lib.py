@@ -12,11 +12,12 @@ SS2D_F32, SS2D_BF16, SS2D_F16 = 0, 1, 2
 SS2D_OK, SS2D_EINVAL, SS2D_ENOTSUP, SS2D_ELAUNCH, SS2D_ENOMEM = 0, -22, -95, -5, -12
 MERGE_PAIRWISE, MERGE_LEFT_TO_RIGHT = 0, 1
 SCAN_CHUNK = 2048
+STATIC_STAGING_BYTES = 80 << 20
 ABI_VERSION = 1
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
            "ss2d_layer_norm", "ss2d_add_layer_norm", "ss2d_bias_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
-           "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_scan_flex_ws", "ss2d_cross_merge_flex",
+           "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_scan_flex_ws", "ss2d_cross_scan_flex_static", "ss2d_cross_merge_flex",
            "ss2d_selective_scan_bwd", "ss2d_transpose_bcl", "ss2d_mlp_fused", "ss2d_linear_cl", "ss2d_linear_cf_ln", "ss2d_stem_conv_ln_gelu", "ss2d_mean_pool_cl")
 
 
@@ -115,6 +116,8 @@ def lib():
         L.ss2d_cross_scan_flex_ws.restype = ctypes.c_int
         L.ss2d_cross_scan_flex_ws.argtypes = ([ctypes.c_void_p] * 2 + [ctypes.c_int] * 9 + [ctypes.c_void_p, ctypes.c_int64]
                                               + [ctypes.c_void_p])
+        L.ss2d_cross_scan_flex_static.restype = ctypes.c_int
+        L.ss2d_cross_scan_flex_static.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 9 + [ctypes.c_void_p]
         L.ss2d_cross_merge_flex.restype = ctypes.c_int
         L.ss2d_cross_merge_flex.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 10 + [ctypes.c_void_p]
         L.ss2d_selective_scan_bwd.restype = ctypes.c_int

@@ -10,6 +10,8 @@
 // OUTPUT element in the output's memory order (so stores are coalesced), the source found through the route.
 // Reads are coalesced whenever the route keeps the innermost dimension (every channel-last source, and the
 // non-transposing routes of channel-first sources); the transposing routes of channel-first sources gather through L2.
+#include <mutex>
+
 #include "ss2d_common.h"
 
 namespace ss2d {
@@ -353,4 +355,50 @@ extern "C" int ss2d_cross_scan_flex_ws(const void *x, void *y, int B, int C, int
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) return SS2D_EINVAL;
     if (workspace_bytes < need) return SS2D_ENOMEM;
     return cross_scan_flex_staged(x, y, B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans, workspace, stream);
+}
+
+// ---- the same with the library's own staging: an entry point that allocates nothing ---------------------------------
+// For callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc): the
+// staging buffer is a fixed array in device memory that comes with the library's code object.  Every device that runs
+// this library holds its own copy at its own address until the process ends; the address is looked up once per device.
+namespace ss2d {
+
+static __device__ __align__(256) unsigned char scratch[SS2D_STATIC_STAGING_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static void *scratch_ptr[kMaxDevices];       // device address of `scratch` on device i; host code never uses the name itself
+
+// The current device's copy of the array.  `scratch` in host code is only a handle for the runtime's symbol table, not
+// a device address: kernels and copies get the pointer resolved here.
+static int static_scratch(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return SS2D_ELAUNCH; }
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) { (void)hipGetLastError(); return SS2D_ELAUNCH; }
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return SS2D_OK;
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_cross_scan_flex_static(const void *x, void *y, int B, int C, int H, int W, int elem_bytes, int x_channel_last,
+                                           int y_channel_last, int one_by_one, int scans, void *stream) {
+    using namespace ss2d;
+    const int64_t need = cross_scan_staging_bytes(B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans);
+    if (need < 0) return (int)need;
+    if (need == 0) return ss2d_cross_scan_flex(x, y, B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans, stream);
+    if (B == 0 || C == 0 || H == 0 || W == 0) return SS2D_OK;
+    if (need > (int64_t)SS2D_STATIC_STAGING_BYTES) return SS2D_ENOMEM;
+    if (!x || !y) return SS2D_EINVAL;
+    void *staging = nullptr;
+    const int rc = static_scratch(&staging);
+    if (rc != SS2D_OK) return rc;
+    // the transpose overwrites every byte the second launch reads: nothing of an earlier call's contents survives into
+    // this one, so the array needs no clearing
+    return cross_scan_flex_staged(x, y, B, C, H, W, elem_bytes, x_channel_last, y_channel_last, one_by_one, scans, staging, stream);
 }
