@@ -111,6 +111,54 @@ def test_scan_matches_oracle(batch, dim, G, N, L, dtype):
     check(*make_inputs(21, batch, dim, G, N, L, dtype), True)
 
 
+# Several states per channel with enough channels per group: the channel-per-lane kernel (64 channels of one group per
+# workgroup, the four wavefronts splitting the states).  Groups of exactly one block, of 1.5 blocks (a half-filled
+# second block), of 48 channels (lanes idle); rows of one round, of whole steps, ending mid-step and mid-round;
+# 4 / 8 / 16 / 32 states.
+CHAN_GRID = [
+    (2, 128, 2, 16, 520), (1, 96, 1, 16, 200), (2, 192, 4, 8, 72), (1, 64, 1, 4, 1000), (1, 128, 2, 32, 136),
+    (3, 64, 2, 16, 8), (1, 256, 1, 16, 3136), (2, 96, 2, 16, 48), (1, 80, 2, 8, 2056),
+]
+
+
+@pytest.mark.parametrize("batch,dim,G,N,L", CHAN_GRID)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_scan_channel_per_lane_kernel_matches_oracle(batch, dim, G, N, L, dtype):
+    _announce("scan-chan", batch, dim, G, N, L, dtype)
+    args = make_inputs(31, batch, dim, G, N, L, dtype)
+    want = orc.selective_scan(*args, True, out_float=True)
+    got, _ = run_gpu(*args, True, True, want_x=False)
+    # Long rows of the reference's test distribution (A down to 1e-4: the state remembers the whole row and reaches
+    # |y| ~ 200 while single outputs cancel to ~0): fp32 recurrences agree to ~1e-5 of the output scale, which the
+    # absolute part of the tolerance has to carry there (the reference's own fp32 atol is 2e-3, test_selective_scan.py:401)
+    tol = TOL32 if L <= 2048 else dict(rtol=1e-3, atol=max(2e-3, 2e-5 * want.abs().max().item()))
+    assert torch.allclose(got, want, **tol), f"max abs err {(got - want).abs().max().item()}"
+    # the same rows with the chunk states requested go through the wavefront-scan kernel: two kernels, one answer
+    got_x, x = run_gpu(*args, True, True, want_x=True)
+    assert torch.allclose(got_x, want, **tol)
+    # SS2D-style constants (A = -(1..N), D = 1, dt bias), output in the input dtype
+    args = make_inputs(32, batch, dim, G, N, L, dtype, ss2d_like=True)
+    want = orc.selective_scan(*args, True, out_float=False)
+    got, _ = run_gpu(*args, True, False, want_x=False)
+    tol = TOL32 if dtype == torch.float32 else TOL16
+    assert got.dtype == dtype and torch.allclose(got.float(), want.float(), **tol)
+
+
+@pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False)])
+def test_scan_channel_per_lane_optional_arguments_and_delta_groups(has_D, has_bias, softplus):
+    _announce("scan-chan-opt", has_D, has_bias, softplus)
+    u, delta, A, B, C, D, bias = make_inputs(33, 2, 128, 2, 16, 264, torch.bfloat16)
+    args = (u, delta, A, B, C, D if has_D else None, bias if has_bias else None)
+    want = orc.selective_scan(*args, softplus, out_float=True)
+    got, _ = run_gpu(*args, softplus, True, want_x=False)
+    assert torch.allclose(got, want, **TOL32), f"max abs err {(got - want).abs().max().item()}"
+    # one delta row shared by 4 channels
+    u, delta, A, B, C, D, bias = make_inputs(34, 2, 128, 2, 8, 136, torch.float32, delta_dim=32)
+    want = orc.selective_scan(u, delta, A, B, C, D, bias, True, out_float=True)
+    got, _ = run_gpu(u, delta, A, B, C, D, bias, True, True, want_x=False)
+    assert torch.allclose(got, want, **TOL32)
+
+
 @pytest.mark.parametrize("batch,dim,G,N,L", [(2, 8, 4, 1, 3136), (1, 8, 4, 16, 784), (2, 16, 4, 1, 49), (1, 4, 4, 1, 333)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_scan_ss2d_init_recipe(batch, dim, G, N, L, dtype):

@@ -13,6 +13,24 @@ constexpr int kPassesPerChunk = SS2D_SCAN_CHUNK / kPass;  // 4
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// Arguments of the stand-alone scan kernels (selective_scan.hip, scan_chan.hip): the C ABI's ss2d_scan_params with
+// derived fields.  Strides in elements.
+struct ScanArgs {
+    const void *u, *delta, *B, *C;
+    const float *A, *D, *bias;
+    void *out;
+    float *x;
+    int32_t batch, dim, L, N, dim_per_group, dim_per_delta, n_chunks, softplus;
+    int64_t u_bs, u_ds, dl_bs, dl_ds, A_ds, A_ns, B_bs, B_gs, B_ns, C_bs, C_gs, C_ns, o_bs, o_ds;
+    int32_t rows;
+    uint32_t B_span_bytes, C_span_bytes;   // extent of B / C reachable through the strides (buffer-descriptor kernels)
+};
+
+// scan_chan.hip: the channel-per-lane kernel for several states per channel.  True when it takes this problem
+// (the caller has already established 16-byte vector I/O); launch returns an SS2D status.
+bool scan_chan_eligible(const ScanArgs &a);
+int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream);
+
 // ---- 8-wide loads / stores ------------------------------------------------------------
 // Eight consecutive elements of a row as they sit in registers before widening: 4 dwords for 16-bit
 // types, 8 for fp32.  Keeping loads in this form lets a pass issue the NEXT pass's loads before it

@@ -24,17 +24,6 @@ namespace ss2d {
 
 constexpr int kScanTailMax = 2;     // the short-tail row kernel takes up to this many 64-position tail passes
 
-struct ScanArgs {
-    const void *u, *delta, *B, *C;
-    const float *A, *D, *bias;
-    void *out;
-    float *x;
-    int32_t batch, dim, L, N, dim_per_group, dim_per_delta, n_chunks, softplus;
-    int64_t u_bs, u_ds, dl_bs, dl_ds, A_ds, A_ns, B_bs, B_gs, B_ns, C_bs, C_gs, C_ns, o_bs, o_ds;
-    int32_t rows;
-    uint32_t B_span_bytes, C_span_bytes;   // flat kernel: extent of B / C reachable through the strides
-};
-
 // ---- one wavefront per row ------------------------------------------------------------
 // kN == 1: the single state lives in registers and inputs are fetched in bursts.
 // kN == 0: any dstate; the per-wave states (running product, h) live in LDS, 2*dstate floats per wave: they
@@ -582,6 +571,8 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     const int64_t row_slots = ((int64_t)q->seqlen + kPass - 1) / kPass * kPass;
     const bool flat = flat_eligible(a, q) && (!vec || 10 * (int64_t)q->seqlen < 7 * row_slots);
     hipStream_t s = (hipStream_t)stream;
+    // several states per channel and enough channels per group to fill wavefronts: one channel per lane
+    if (vec && scan_chan_eligible(a)) return launch_scan_chan(a, q->in_dtype, q->out_dtype, s);
     if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, flat, s);
     if (q->in_dtype == SS2D_BF16) {
         return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, flat, s)
