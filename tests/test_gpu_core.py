@@ -74,6 +74,13 @@ CORE_SHAPES = [
     (9, 1, 6, 5),        # L = 30: two-element granularity handled element-wise
     (1, 1, 3, 3),        # smallest supported image
     (1, 2, 64, 48),      # L = 3072
+    # 7 x 7 and 14 x 14 maps whose streams start on 16-byte boundaries take the row-per-lane kernel (16-bit inputs):
+    (16, 5, 7, 7),       # two tiles of 8 maps; channels not a multiple of the 4 per workgroup
+    (24, 3, 7, 7),       # three tiles, three channels (one wavefront of the workgroup has no channel)
+    (40, 8, 7, 7),
+    (6, 5, 14, 14),      # tiles of 4 maps, the last one half full
+    (2, 1, 14, 14),      # a single, half-full tile
+    (12, 4, 14, 14),
 ]
 
 

@@ -31,6 +31,22 @@ struct ScanArgs {
 bool scan_chan_eligible(const ScanArgs &a);
 int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream);
 
+// Arguments of the fused core kernels (ss2d_core.hip, ss2d_core_small.hip): the C ABI's ss2d_core_params with derived
+// fields.  Strides in elements.
+struct CoreArgs {
+    const void *x, *delta, *Bm, *Cm;
+    const float *A, *Dv, *bias;
+    void *y;
+    int32_t B, D, H, W, L, CB, softplus, vec_ok, vec_out;
+    int64_t dl_ks, dl_ds, dl_bs;        // delta strides over direction, channel, batch (elements)
+    int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
+    uint32_t B_span_bytes, C_span_bytes;
+};
+
+// ss2d_core_small.hip: the row-per-lane kernel for small square maps.
+bool core_small_eligible(const CoreArgs &a, int in_dtype);
+int launch_core_small(const CoreArgs &a, int in_dtype, hipStream_t stream);
+
 // ---- 8-wide loads / stores ------------------------------------------------------------
 // Eight consecutive elements of a row as they sit in registers before widening: 4 dwords for 16-bit
 // types, 8 for fp32.  Keeping loads in this form lets a pass issue the NEXT pass's loads before it

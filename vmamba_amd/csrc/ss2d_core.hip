@@ -34,16 +34,6 @@
 
 namespace ss2d {
 
-struct CoreArgs {
-    const void *x, *delta, *Bm, *Cm;
-    const float *A, *Dv, *bias;
-    void *y;
-    int32_t B, D, H, W, L, CB, softplus, vec_ok, vec_out;
-    int64_t dl_ks, dl_ds, dl_bs;        // delta strides over direction, channel, batch (elements)
-    int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
-    uint32_t B_span_bytes, C_span_bytes;
-};
-
 // Index of logical element a in an LDS array of kBytes-wide elements that skips one word after every 32 words.
 template <int kBytes> __host__ __device__ __forceinline__ constexpr int lds_index(int a) {
     static_assert(kBytes == 2 || kBytes == 4, "16-bit or 32-bit elements");
@@ -512,6 +502,8 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     a.CB = 1; a.vec_ok = 0; a.vec_out = 0;
 
     hipStream_t s = (hipStream_t)stream;
+    // 7 x 7 and 14 x 14 maps in the batch-innermost layout: one map row per lane, everything in registers
+    if (core_small_eligible(a, q->in_dtype)) return launch_core_small(a, q->in_dtype, s);
     if (q->in_dtype == SS2D_F32) return launch_core<float>(a, s);
     if (q->in_dtype == SS2D_BF16) return launch_core<bf16_t>(a, s);
     return launch_core<f16_t>(a, s);

@@ -1,0 +1,302 @@
+// Fused SS2D core (CrossScan -> selective scan -> CrossMerge, d_state = 1) for SMALL square maps -- 7 x 7 and 14 x 14,
+// the last two stages of a 224 x 224 VMamba -- with one map ROW per lane and every index fixed at compile time.
+//
+// The general kernel (ss2d_core.hip) walks the images of a workgroup as one stream, 8 positions per lane; on maps of
+// 49 or 196 positions most of its instructions are bookkeeping: images start inside a lane's 8 items, B / C are gathered
+// in groups of 1 or 4, the transposed copies of the map and of the result are built element by element.  Here
+//   * a map of S x S positions occupies S lanes of a group of 8 or 16 lanes (the DPP row or half row), 4 or 8 maps per
+//     wavefront, the maps of a wavefront being consecutive images of one channel (their delta / B / C rows are adjacent
+//     in the batch-innermost layout, so a stream tile is fetched with one or two 16-byte loads per lane and parked in
+//     LDS as loaded); the four wavefronts of a workgroup are four channels on the same images and share the B / C tiles;
+//     everything a workgroup reads is requested before its arithmetic starts;
+//   * for the row-major directions (0, 2) lane i owns row i, for the column-major ones (1, 3) column i: either way its
+//     S positions are S consecutive stream items, which it scans serially in registers; the lane totals are combined
+//     by a DPP scan over the lane group (forward for directions 0 / 1, in reverse lane order for 2 / 3), and the state
+//     entering the lane is pushed through its items.  A map's first item is forced to a = 0, which stops anything
+//     arriving from the neighbouring group;
+//   * u comes from two register copies of the map (its row, and its column obtained through one LDS transposition);
+//     the outputs of directions 0 + 2 accumulate in registers indexed by column, those of 1 + 3 in registers indexed by
+//     row; one more LDS transposition brings the second set into row layout and out = (y0 + y2) + (y1 + y3) leaves
+//     as plain row stores -- the association order of cross_merge_fwd (classification/models/csm_triton.py:61-62).
+// No stream position, image boundary or LDS address is computed at run time.
+#include "scan_common.h"
+
+namespace ss2d {
+
+// Inclusive scan of (a, h) pairs over the 16-lane DPP row, in lane order or in reverse lane order; returns the
+// EXCLUSIVE h (the state entering this lane; 0 for the first lane of the row).  Lanes without a source keep their value.
+template <bool kReverse>
+__device__ __forceinline__ float row_scan_state_in(float a, float h) {
+    float hx = 0.0f;
+#define SS2D_ROW_STEP(CTRL)                                         \
+    "v_fmac_f32_dpp %1, %1, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t" \
+    "v_mul_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"  \
+    "s_nop 0\n\t"
+    if constexpr (!kReverse) {
+        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shr:1") SS2D_ROW_STEP("row_shr:2") SS2D_ROW_STEP("row_shr:4") SS2D_ROW_STEP("row_shr:8")
+            "s_nop 0\n\t"
+            "v_mov_b32_dpp %2, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0"
+            : "+v"(a), "+v"(h), "+v"(hx));
+    } else {
+        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shl:1") SS2D_ROW_STEP("row_shl:2") SS2D_ROW_STEP("row_shl:4") SS2D_ROW_STEP("row_shl:8")
+            "s_nop 0\n\t"
+            "v_mov_b32_dpp %2, %1 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0"
+            : "+v"(a), "+v"(h), "+v"(hx));
+    }
+#undef SS2D_ROW_STEP
+    return hx;
+}
+
+// kS consecutive 16-bit elements of an LDS tile as they sit there: dwords of two elements for even kS (element offsets
+// are even then: 4-byte reads), one element per register for odd kS.  item() widens element j.
+template <typename in_t, int kS> struct Run {
+    static constexpr bool kPacked = kS % 2 == 0;
+    uint32_t w[kPacked ? kS / 2 : kS];
+    __device__ __forceinline__ void read(const uint16_t *tile, int elem_off) {
+        if constexpr (kPacked) {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(tile + elem_off);
+#pragma unroll
+            for (int k = 0; k < kS / 2; ++k) w[k] = src[k];
+        } else {
+#pragma unroll
+            for (int j = 0; j < kS; ++j) w[j] = tile[elem_off + j];
+        }
+    }
+    __device__ __forceinline__ float item(int j) const {
+        if constexpr (kPacked) return (j & 1) ? unpack_hi<in_t>(w[j / 2]) : unpack_lo<in_t>(w[j / 2]);
+        else return to_f32(in_t{(uint16_t)w[j]});
+    }
+};
+
+constexpr int kSmallChans = kWavesPerWg;     // channels per workgroup: one per wavefront, all on the same images
+
+// Registers are capped so that as many workgroups share a CU as its LDS tiles allow (3 for 14 x 14, 5-6 for 7 x 7).
+template <typename in_t, int kS, bool kSoftplus>
+__global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kernel(const CoreArgs p, int chan_quads, FastDiv div_quads) {
+    constexpr int kLanes = kS <= 8 ? 8 : 16;                 // lanes per map
+    constexpr int kMaps = kWave / kLanes;                    // maps per wavefront
+    constexpr int kL = kS * kS;
+    constexpr int kTileElems = kMaps * kL;                   // one stream tile: the maps' rows are adjacent in memory
+    constexpr int kTileVecs = kTileElems / 8;                // in 16-byte pieces (392 or 784 elements: whole pieces)
+    constexpr int kVecsPerLane = (kTileVecs + kWave - 1) / kWave;
+    constexpr int kBcPieces = 8 * kTileVecs;                 // B and C tiles of the four directions
+    constexpr int kBcPerThread = (kBcPieces + kBlock - 1) / kBlock;
+    static_assert(kTileElems % 8 == 0 && sizeof(in_t) == 2, "16-bit streams in whole 16-byte pieces");
+    // Everything a workgroup reads is fetched before its arithmetic starts (one memory latency per workgroup; the
+    // registers that carry the loads are free again when the per-map arrays come alive):
+    //   shared by the four wavefronts (same images): the B and C tiles of the four directions   [dir][B|C][tile]
+    //   per wavefront (its channel): the four delta tiles, and one fp32 tile that first holds the x maps (16-bit) for
+    //   the row -> column transposition and at the end the (y1 + y3) sums for the column -> row transposition
+    __shared__ __align__(16) uint16_t s_bc[8 * kTileElems];
+    __shared__ __align__(16) uint16_t s_dl[kWavesPerWg * 4 * kTileElems];
+    __shared__ __align__(16) float s_tr[kWavesPerWg * kTileElems];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    uint32_t bt, dq;
+    divmod(blockIdx.x, div_quads, bt, dq);                   // neighbouring workgroups: other channels of the same images
+    const int d_raw = (int)dq * kSmallChans + wave;
+    const bool chan_ok = d_raw < p.D;                        // (a wavefront without a channel still helps to fetch B / C)
+    const int d = min(d_raw, p.D - 1);
+    const int b0 = (int)bt * kMaps;
+    const int nb = min(kMaps, p.B - b0);
+    const int g = lane / kLanes, i = lane % kLanes;
+    const bool active = g < nb && i < kS;
+    const int gc = min(g, nb - 1), ic = min(i, kS - 1);      // clamped: every lane addresses real memory
+
+    uint16_t *tile_dl = s_dl + wave * 4 * kTileElems;
+    float *tile_tr = s_tr + wave * kTileElems;
+
+    // ---- fetch ------------------------------------------------------------------------------------------------------
+    // delta: four tiles of this wavefront's channel, 16-byte buffer loads (range-checked: a short last tile reads zeros
+    // past its end)
+    uint4 r_dl[4][kVecsPerLane];
+    {
+        const in_t *dl_all = reinterpret_cast<const in_t *>(p.delta);
+        const int tile_bytes = nb * kL * 2;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const in_t *dl_k = dl_all + (int64_t)k * p.dl_ks + (int64_t)d * p.dl_ds + (int64_t)b0 * kL;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<in_t *>(dl_k), 0, tile_bytes, kBufferRsrcWord3);
+#pragma unroll
+            for (int v = 0; v < kVecsPerLane; ++v) {
+                const auto t = __builtin_amdgcn_raw_buffer_load_b128(rs, (v * kWave + lane) * 16, 0, 0);
+                r_dl[k][v] = make_uint4(t[0], t[1], t[2], t[3]);
+            }
+        }
+    }
+    // B / C: the workgroup's threads share the 8 tiles; one descriptor over each tensor, the tile chosen per lane (what
+    // lies behind a short last tile is other images' data or, past the tensor, zeros: finite either way, never stored)
+    uint4 r_bc[kBcPerThread];
+    {
+        const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bm), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rC = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Cm), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
+#pragma unroll
+        for (int n = 0; n < kBcPerThread; ++n) {
+            const int piece = n * kBlock + (int)threadIdx.x;     // [dir][B|C][piece of the tile]
+            const int t = min(piece, kBcPieces - 1) / kTileVecs, v = min(piece, kBcPieces - 1) % kTileVecs;
+            const int k = t >> 1;
+            const uint32_t off_B = (uint32_t)(k * p.B_ks + (int64_t)b0 * kL) * 2u + (uint32_t)v * 16u;
+            const uint32_t off_C = (uint32_t)(k * p.C_ks + (int64_t)b0 * kL) * 2u + (uint32_t)v * 16u;
+            const auto tb = __builtin_amdgcn_raw_buffer_load_b128(rB, (int)off_B, 0, 0);
+            const auto tc = __builtin_amdgcn_raw_buffer_load_b128(rC, (int)off_C, 0, 0);
+            const bool is_c = (t & 1) != 0;
+            r_bc[n] = make_uint4(is_c ? tc[0] : tb[0], is_c ? tc[1] : tb[1], is_c ? tc[2] : tb[2], is_c ? tc[3] : tb[3]);
+        }
+    }
+    // the map: this lane's row
+    float x_row[kS], x_col[kS];
+    {
+        const in_t *row = reinterpret_cast<const in_t *>(p.x) + ((int64_t)(b0 + gc) * p.D + d) * kL + ic * kS;
+        uint16_t *xt = reinterpret_cast<uint16_t *>(tile_tr);   // [map][row][col]
+        if constexpr (kS % 2 == 0) {
+            uint32_t w[kS / 2];
+#pragma unroll
+            for (int k = 0; k < kS / 2; ++k) w[k] = reinterpret_cast<const uint32_t *>(row)[k];
+#pragma unroll
+            for (int k = 0; k < kS / 2; ++k) {
+                x_row[2 * k] = unpack_lo<in_t>(w[k]);
+                x_row[2 * k + 1] = unpack_hi<in_t>(w[k]);
+                if (active) reinterpret_cast<uint32_t *>(xt + gc * kL + ic * kS)[k] = w[k];
+            }
+        } else {
+            uint16_t e[kS];
+#pragma unroll
+            for (int j = 0; j < kS; ++j) e[j] = row[j].bits;
+#pragma unroll
+            for (int j = 0; j < kS; ++j) {
+                x_row[j] = to_f32(in_t{e[j]});
+                if (active) xt[gc * kL + ic * kS + j] = e[j];
+            }
+        }
+    }
+    // ---- park the streams in LDS ------------------------------------------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int v = 0; v < kVecsPerLane; ++v) {
+            const int vec = v * kWave + lane;
+            if (vec < kTileVecs) *reinterpret_cast<uint4 *>(tile_dl + k * kTileElems + vec * 8) = r_dl[k][v];
+        }
+#pragma unroll
+    for (int n = 0; n < kBcPerThread; ++n) {
+        const int piece = n * kBlock + (int)threadIdx.x;
+        if (piece < kBcPieces) *reinterpret_cast<uint4 *>(s_bc + piece * 8) = r_bc[n];
+    }
+    __syncthreads();                                         // the only workgroup barrier: B / C tiles are in place
+    if (!chan_ok) return;
+    {
+        // ... and (through the x tile) this lane's column
+        const uint16_t *xt = reinterpret_cast<const uint16_t *>(tile_tr);
+#pragma unroll
+        for (int j = 0; j < kS; ++j) x_col[j] = to_f32(in_t{xt[gc * kL + j * kS + ic]});
+    }
+
+    float acc_rm[kS], acc_cm[kS];                            // y0 + y2 by column of row i;  y1 + y3 by row of column i
+#pragma unroll
+    for (int j = 0; j < kS; ++j) { acc_rm[j] = 0.0f; acc_cm[j] = 0.0f; }
+
+    auto direction = [&](auto dir_tag) {
+        constexpr int kDir = decltype(dir_tag)::value;
+        constexpr bool kRev = kDir >= 2, kCol = (kDir & 1) != 0;
+        // reversed directions: stream position t' = L-1-t, so the run holding this lane's row / column is run kS-1-i,
+        // met from its far end -- item j of the run is column (row) kS-1-j
+        const int run = gc * kL + (kRev ? kS - 1 - ic : ic) * kS;
+        Run<in_t, kS> raw, Bv, Cv;
+        raw.read(tile_dl + kDir * kTileElems, run);
+        Bv.read(s_bc + (2 * kDir) * kTileElems, run);
+        Cv.read(s_bc + (2 * kDir + 1) * kTileElems, run);
+
+        const int kd = kDir * p.D + d;
+        const float A2 = p.A[kd] * kLog2e;
+        const float Dk = p.Dv ? p.Dv[kd] : 0.0f;
+        const float bias = p.bias ? p.bias[kd] : 0.0f;
+        const bool first = kRev ? i == kS - 1 : i == 0;      // the lane that starts the map in this direction's order
+        float ac[kS], hh[kS];
+#pragma unroll
+        for (int j = 0; j < kS; ++j) {
+            const int m = kRev ? kS - 1 - j : j;             // column (directions 0 / 2) or row (1 / 3) of item j
+            const float u = kCol ? x_col[m] : x_row[m];
+            float dl;
+            if constexpr (kSoftplus) dl = softplus_log2(fmaf(raw.item(j), kLog2e, bias * kLog2e));
+            else dl = raw.item(j) + bias;
+            float a = __builtin_amdgcn_exp2f(dl * A2);
+            if (j == 0) a = first ? 0.0f : a;                // nothing enters a map from the lanes before it
+            const float bb = Bv.item(j) * (dl * u);
+            ac[j] = j == 0 ? a : ac[j - 1] * a;
+            hh[j] = j == 0 ? bb : fmaf(a, hh[j - 1], bb);
+        }
+        // lanes that hold no row pass the state through unchanged (and keep whatever they computed out of the scan)
+        const float a_tot = active ? ac[kS - 1] : 1.0f, h_tot = active ? hh[kS - 1] : 0.0f;
+        const float h_in = row_scan_state_in<kRev>(a_tot, h_tot);
+#pragma unroll
+        for (int j = 0; j < kS; ++j) {
+            const int m = kRev ? kS - 1 - j : j;
+            const float u = kCol ? x_col[m] : x_row[m];
+            const float y = fmaf(Cv.item(j), fmaf(ac[j], h_in, hh[j]), Dk * u);
+            if constexpr (kCol) acc_cm[m] += y; else acc_rm[m] += y;
+        }
+    };
+    // (y0 + y2) and (y1 + y3): the first addition into a zero is exact, the second rounds once
+    direction(std::integral_constant<int, 0>{});
+    direction(std::integral_constant<int, 2>{});
+    direction(std::integral_constant<int, 1>{});
+    direction(std::integral_constant<int, 3>{});
+
+    // ---- merge: bring (y1 + y3) from column layout to row layout through LDS, add, store the row --------------------
+    wave_lds_sync();                                         // every lane has read its column of the x tile
+    if (active) {                                            // (idle lanes address the last row / map: they must not write)
+#pragma unroll
+        for (int j = 0; j < kS; ++j) tile_tr[gc * kL + j * kS + ic] = acc_cm[j];   // this lane is column i: element (row j, col i)
+    }
+    wave_lds_sync();
+    float out[kS];
+#pragma unroll
+    for (int j = 0; j < kS; ++j) out[j] = acc_rm[j] + tile_tr[gc * kL + ic * kS + j];
+    if (active) {
+        float *yo = reinterpret_cast<float *>(p.y) + ((int64_t)(b0 + g) * p.D + d) * kL + i * kS;
+        if constexpr (kS % 2 == 0) {
+#pragma unroll
+            for (int k = 0; k < kS / 2; ++k) reinterpret_cast<float2 *>(yo)[k] = make_float2(out[2 * k], out[2 * k + 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kS; ++j) yo[j] = out[j];
+        }
+    }
+}
+
+bool core_small_eligible(const CoreArgs &a, int in_dtype) {
+    if (in_dtype != SS2D_BF16 && in_dtype != SS2D_F16) return false;
+    if (a.H != a.W || (a.H != 7 && a.H != 14)) return false;
+    const int64_t L = a.L;
+    // consecutive images adjacent in every stream (batch-innermost layout), all tile starts on 16-byte boundaries
+    if (a.dl_bs != L || a.B_bs != L || a.C_bs != L) return false;
+    auto al = [](const void *ptr, uintptr_t n) { return (reinterpret_cast<uintptr_t>(ptr) % n) == 0; };
+    if (!al(a.delta, 16) || !al(a.Bm, 16) || !al(a.Cm, 16) || !al(a.x, 4) || !al(a.y, 8)) return false;
+    if (a.dl_ks % 8 != 0 || a.dl_ds % 8 != 0 || a.B_ks % 8 != 0 || a.C_ks % 8 != 0) return false;
+    return true;
+}
+
+template <typename in_t, int kS>
+static int launch_core_small_typed(const CoreArgs &a, hipStream_t stream) {
+    constexpr int kMaps = kWave / (kS <= 8 ? 8 : 16);
+    const int tiles = (a.B + kMaps - 1) / kMaps;
+    const int quads = (a.D + kSmallChans - 1) / kSmallChans;
+    const int64_t n_wg = (int64_t)quads * tiles;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    const FastDiv dq = make_fastdiv((uint32_t)quads);
+    if (a.softplus) hipLaunchKernelGGL((ss2d_core_small_kernel<in_t, kS, true>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream, a, quads, dq);
+    else hipLaunchKernelGGL((ss2d_core_small_kernel<in_t, kS, false>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream, a, quads, dq);
+    return launch_status();
+}
+
+int launch_core_small(const CoreArgs &a, int in_dtype, hipStream_t stream) {
+    if (in_dtype == SS2D_BF16) {
+        return a.H == 7 ? launch_core_small_typed<bf16_t, 7>(a, stream) : launch_core_small_typed<bf16_t, 14>(a, stream);
+    }
+    return a.H == 7 ? launch_core_small_typed<f16_t, 7>(a, stream) : launch_core_small_typed<f16_t, 14>(a, stream);
+}
+
+}  // namespace ss2d
