@@ -36,6 +36,20 @@ template <typename T> __device__ __forceinline__ void unpack8(const uint4 raw, f
     }
 }
 
+// sum += a.lo * b.lo + a.hi * b.hi for dwords of two 16-bit values, fp32 accumulation: one instruction on the packed
+// data as loaded (v_dot2c_f32_bf16 / v_dot2_f32_f16) instead of two widenings and two fused multiply-adds.
+__device__ __forceinline__ float dot2_acc(bf16_t, uint32_t a, uint32_t b, float sum) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), sum, false);
+}
+__device__ __forceinline__ float dot2_acc(f16_t, uint32_t a, uint32_t b, float sum) {
+    typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2_t, a), __builtin_bit_cast(halfx2_t, b), sum, false);
+}
+// (lo half of a, lo half of b) and (hi half of a, hi half of b) as new dwords: two taps of one channel side by side
+__device__ __forceinline__ uint32_t pair_lo(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
+__device__ __forceinline__ uint32_t pair_hi(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
+
 // 16-bit element types, D % 8 == 0, 16-byte aligned tensors (host-checked).
 template <typename T, bool kSilu>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_kernel(const T *__restrict__ x, const T *__restrict__ weight,
@@ -167,24 +181,27 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             if (e < n_in) *reinterpret_cast<uint4 *>(in_tile + (size_t)e * kDwCh + cv * 8) = v[u];
         }
     }
-    // the 72 weights of the 8 channels: 9 consecutive 16-byte vectors
-    float wt[8][9];
+    // The 72 weights of the 8 channels (9 consecutive 16-byte vectors), regrouped for the dot instruction: per channel
+    // four dwords holding taps (0,1) (2,3) (4,5) (6,7) and one holding (tap 8, zero).
+    uint32_t wp2[8][5];
     float bv[8];
     {
         const int cw = min(c0, D - 8);                           // keep the loads in range; lanes with c0 >= D store nothing
-        const uint4 *wp = reinterpret_cast<const uint4 *>(weight + (size_t)cw * 9);
-        float flat[72];
+        const uint16_t *wsrc = reinterpret_cast<const uint16_t *>(weight + (size_t)cw * 9);
+        uint32_t wraw[36];
 #pragma unroll
         for (int k = 0; k < 9; ++k) {
-            float t8[8];
-            unpack8<T>(wp[k], t8);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) flat[k * 8 + i] = t8[i];
+            const uint4 v = reinterpret_cast<const uint4 *>(wsrc)[k];
+            wraw[4 * k] = v.x; wraw[4 * k + 1] = v.y; wraw[4 * k + 2] = v.z; wraw[4 * k + 3] = v.w;
         }
+        // element e = ci * 9 + t sits in half (e & 1) of dword e / 2
+        auto elem = [&](int e) -> uint32_t { return (e & 1) ? (wraw[e / 2] >> 16) : (wraw[e / 2] & 0xffffu); };
 #pragma unroll
-        for (int ci = 0; ci < 8; ++ci)
+        for (int ci = 0; ci < 8; ++ci) {
 #pragma unroll
-            for (int t = 0; t < 9; ++t) wt[ci][t] = flat[ci * 9 + t];
+            for (int tp = 0; tp < 4; ++tp) wp2[ci][tp] = elem(ci * 9 + 2 * tp) | (elem(ci * 9 + 2 * tp + 1) << 16);
+            wp2[ci][4] = elem(ci * 9 + 8);
+        }
 #pragma unroll
         for (int ci = 0; ci < 8; ++ci) bv[ci] = 0.0f;
         if (bias) unpack8<T>(*reinterpret_cast<const uint4 *>(bias + cw), bv);
@@ -196,21 +213,38 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     for (int pidx = threadIdx.x / 4; pidx < n_out; pidx += kBlock / 4) {
         uint32_t ph, pw;
         divmod((uint32_t)pidx, divW, ph, pw);
-        float acc[8];
-#pragma unroll
-        for (int ci = 0; ci < 8; ++ci) acc[ci] = 0.0f;
+        // nine taps as four pairs and a single: the two taps of a pair are brought side by side per channel (one byte
+        // permute per channel pair and tap pair) and multiplied-accumulated by one dot instruction per channel
+        uint4 tap[9];
 #pragma unroll
         for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
-            for (int kw = 0; kw < 3; ++kw) {
-                float xv[8];
-                unpack8<T>(*reinterpret_cast<const uint4 *>(in_tile + ((size_t)(ph + kh) * Wp + pw + kw) * kDwCh + cv * 8), xv);
+            for (int kw = 0; kw < 3; ++kw)
+                tap[kh * 3 + kw] = *reinterpret_cast<const uint4 *>(in_tile + ((size_t)(ph + kh) * Wp + pw + kw) * kDwCh + cv * 8);
+        float acc[8];
 #pragma unroll
-                for (int ci = 0; ci < 8; ++ci) acc[ci] = fmaf(wt[ci][kh * 3 + kw], xv[ci], acc[ci]);
+        for (int ci = 0; ci < 8; ++ci) acc[ci] = bv[ci];
+#pragma unroll
+        for (int tp = 0; tp < 4; ++tp) {
+            const uint32_t a[4] = {tap[2 * tp].x, tap[2 * tp].y, tap[2 * tp].z, tap[2 * tp].w};
+            const uint32_t b[4] = {tap[2 * tp + 1].x, tap[2 * tp + 1].y, tap[2 * tp + 1].z, tap[2 * tp + 1].w};
+#pragma unroll
+            for (int cp = 0; cp < 4; ++cp) {
+                acc[2 * cp] = dot2_acc(T{}, pair_lo(a[cp], b[cp]), wp2[2 * cp][tp], acc[2 * cp]);
+                acc[2 * cp + 1] = dot2_acc(T{}, pair_hi(a[cp], b[cp]), wp2[2 * cp + 1][tp], acc[2 * cp + 1]);
             }
+        }
+        {
+            const uint32_t a[4] = {tap[8].x, tap[8].y, tap[8].z, tap[8].w};
+#pragma unroll
+            for (int cp = 0; cp < 4; ++cp) {
+                acc[2 * cp] = dot2_acc(T{}, a[cp] & 0xffffu, wp2[2 * cp][4], acc[2 * cp]);
+                acc[2 * cp + 1] = dot2_acc(T{}, a[cp] >> 16, wp2[2 * cp + 1][4], acc[2 * cp + 1]);
+            }
+        }
 #pragma unroll
         for (int ci = 0; ci < 8; ci += 2) {
-            uint32_t o = pack2_from_f32<T>(acc[ci] + bv[ci], acc[ci + 1] + bv[ci + 1]);            // conv output as stored
+            uint32_t o = pack2_from_f32<T>(acc[ci], acc[ci + 1]);                                  // conv output as stored
             if (kSilu) o = pack2_from_f32<T>(silu_fast(unpack_lo<T>(o)), silu_fast(unpack_hi<T>(o)));
             out_tile[(cv * 8 + ci) * out_pitch + pidx] = (uint16_t)(o & 0xffffu);
             out_tile[(cv * 8 + ci + 1) * out_pitch + pidx] = (uint16_t)(o >> 16);
