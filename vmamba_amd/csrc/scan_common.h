@@ -37,7 +37,7 @@ struct CoreArgs {
     const void *x, *delta, *Bm, *Cm;
     const float *A, *Dv, *bias;
     void *y;
-    int32_t B, D, H, W, L, CB, softplus, vec_ok, vec_out;
+    int32_t B, D, H, W, L, CB, softplus, vec_ok, vec_out, stage_tiles, tile_merge;
     int64_t dl_ks, dl_ds, dl_bs;        // delta strides over direction, channel, batch (elements)
     int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
     uint32_t B_span_bytes, C_span_bytes;

@@ -44,12 +44,22 @@ template <int kBytes> __host__ __device__ __forceinline__ constexpr int lds_exte
     return (lds_index<kBytes>(n) + 8) & ~7;
 }
 
-// The x maps carry one extra aligned block of kItems zeros behind the last image: groups past the end of the stream
-// read their u there, so that u = 0 (and with it the drive term) needs no select.
-__host__ __device__ __forceinline__ constexpr int core_zero_block(int n) { return (n + kItems - 1) & ~(kItems - 1); }
-template <int kBytes> __host__ __device__ __forceinline__ constexpr int core_map_extent(int n) {
-    return lds_extent<kBytes>(core_zero_block(n) + kItems);
+// The x maps.  With 16-bit elements walked in aligned blocks of 8 (kFlat) every access of the passes is a 16-byte
+// access of consecutive lanes, which needs no padding: the maps are then plain arrays.  Otherwise they skip words
+// like the planes.  They carry one extra aligned block of kItems zeros behind the last image: groups past the end of
+// the stream read their u there, so that u = 0 (and with it the drive term) needs no select.
+template <int kBytes, bool kFlat> __host__ __device__ __forceinline__ constexpr int map_index(int a) {
+    return kFlat ? a : lds_index<kBytes>(a);
 }
+__host__ __device__ __forceinline__ constexpr int core_zero_block(int n) { return (n + kItems - 1) & ~(kItems - 1); }
+template <int kBytes, bool kFlat> __host__ __device__ __forceinline__ constexpr int core_map_extent(int n) {
+    return kFlat ? core_zero_block(n) + kItems : lds_extent<kBytes>(core_zero_block(n) + kItems);
+}
+template <typename in_t, int kGran> constexpr bool core_flat_maps() { return sizeof(in_t) == 2 && kGran == kItems; }
+
+// Wavefronts per SIMD the register allocation aims at: six for the 16-bit walks in blocks (what their LDS arrays allow;
+// a few values that only live before and after the pass loop are then parked in scratch memory), four otherwise.
+template <typename in_t, int kGran> constexpr int core_min_waves() { return sizeof(in_t) == 2 && kGran >= 4 ? 6 : 4; }
 
 constexpr int kCoreBurst = 2;     // passes whose delta / B / C loads are in flight per wavefront
 
@@ -60,18 +70,20 @@ struct CorePassLoads {
     static constexpr int kWords = gather_words<in_t, kGran>();
     Raw8<in_t> dl;
     uint32_t b[kGroups][kWords], c[kGroups][kWords];
-    uint32_t i0, j0;      // image and position of the lane's first item
+    uint32_t img, j0;     // first element of the image (its index times L) and position in it of the lane's first item
 };
 
 template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta>
-__global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD) {
+__global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD, FastDiv divTiles,
+                                                           FastDiv divWt) {
     extern __shared__ __align__(16) float core_smem[];
     constexpr int kEs = (int)sizeof(in_t);
     constexpr int kGroups = kItems / kGran;
+    constexpr bool kFlat = core_flat_maps<in_t, kGran>();
     using Loads = CorePassLoads<in_t, kGran>;
     const int L = p.L, H = p.H;
     const int n_max = p.CB * L;
-    const int plane_ext = lds_extent<4>(n_max), map_ext = core_map_extent<kEs>(n_max);
+    const int plane_ext = lds_extent<4>(n_max), map_ext = core_map_extent<kEs, kFlat>(n_max);
     float *planeA = core_smem;                           // fl(y0 + y2), row-major index
     float *planeB = planeA + plane_ext;                  // fl(y1 + y3), column-major index
     in_t *xR = reinterpret_cast<in_t *>(planeB + plane_ext);
@@ -96,8 +108,12 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Cm), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     const uint32_t B_soff = (uint32_t)(dir * p.B_ks + b0 * p.B_bs), C_soff = (uint32_t)(dir * p.C_ks + b0 * p.C_bs);
     const float A_log2e = p.A[kd] * kLog2e;
-    const float Dv = p.Dv ? p.Dv[kd] : 0.0f;
     const float bias = p.bias ? p.bias[kd] : 0.0f;
+    const bool reverse = dir >= 2;                       // uniform per wavefront
+    const uint32_t u_sel = reverse ? 0x05040706u : 0x03020100u;
+    // B / C rows of consecutive images adjacent in memory (what one x_proj GEMM per direction writes): a lane's offset
+    // into them is its stream position
+    const bool bc_dense = p.B_bs == L && p.C_bs == L;
     // passes of 512 positions; a remainder of at most 64 positions is walked one position per lane instead
     const int tail_len = n_el % kPass;
     const bool short_tail = tail_len > 0 && tail_len <= kWave;
@@ -105,9 +121,10 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
 
     // Image and position of this lane's first item in the pass issued next: passes are issued strictly in order, so
     // the pair just advances by 512 positions each time (no division in the loop).
-    uint32_t next_i, next_j, step_i, step_j;
-    divmod((uint32_t)(lane * kItems), divL, next_i, next_j);
-    divmod((uint32_t)kPass, divL, step_i, step_j);
+    uint32_t next_img, next_j, step_img, step_j;
+    divmod((uint32_t)(lane * kItems), divL, next_img, next_j);
+    divmod((uint32_t)kPass, divL, step_img, step_j);
+    next_img *= (uint32_t)L; step_img *= (uint32_t)L;
     auto issue = [&](int pass, Loads &r) {
         const int e0 = pass * kPass + lane * kItems;
         if constexpr (kVecDelta) {
@@ -124,11 +141,21 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         } else {
             r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
         }
-        r.i0 = next_i; r.j0 = next_j;
-        next_i += step_i; next_j += step_j;
-        if (next_j >= (uint32_t)L) { next_j -= (uint32_t)L; next_i += 1; }
+        r.img = next_img; r.j0 = next_j;
+        next_img += step_img; next_j += step_j;
+        if (next_j >= (uint32_t)L) { next_j -= (uint32_t)L; next_img += (uint32_t)L; }
+        if (bc_dense) {                                  // uniform
+#pragma unroll
+            for (int gi = 0; gi < kGroups; ++gi) {
+                gather_group_raw<in_t, kGran>(B_rsrc, (uint32_t)(e0 + gi * kGran), B_soff, r.b[gi]);
+                gather_group_raw<in_t, kGran>(C_rsrc, (uint32_t)(e0 + gi * kGran), C_soff, r.c[gi]);
+            }
+            return;
+        }
+        uint32_t i0, rem;
+        divmod(r.img, divL, i0, rem);
         const int k = kGran == kItems ? kItems : min(kItems, L - (int)r.j0);   // items before the next image starts
-        const uint32_t B_a = r.i0 * (uint32_t)p.B_bs + r.j0, C_a = r.i0 * (uint32_t)p.C_bs + r.j0;   // image i0
+        const uint32_t B_a = i0 * (uint32_t)p.B_bs + r.j0, C_a = i0 * (uint32_t)p.C_bs + r.j0;   // image i0
         const uint32_t B_b = B_a + (uint32_t)p.B_bs - (uint32_t)(r.j0 + k), C_b = C_a + (uint32_t)p.C_bs - (uint32_t)(r.j0 + k);
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
@@ -164,49 +191,46 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
                 if (idx < n_el) {
                     uint32_t h, w;
                     divmod(rr[u], divW, h, w);
-                    xR[lds_index<kEs>(idx)] = v[u];
-                    xT[lds_index<kEs>((int)(ii[u] * L + w * H + h))] = v[u];
+                    xR[map_index<kEs, kFlat>(idx)] = v[u];
+                    xT[map_index<kEs, kFlat>((int)(ii[u] * L + w * H + h))] = v[u];
                 }
             }
         }
     };
-    if constexpr (kGran == kItems && sizeof(in_t) == 2) {
-        if (p.W >= kItems) {
-            // rows are multiples of 8 elements (and 16-byte aligned, host-checked through kGran): 16-byte loads.  A block
-            // of 8 lies in one image and, with W >= 8, in at most two rows of it.
-            const int n_vec = n_el / kItems;
-            for (int base = 0; base < n_vec; base += 2 * kBlock) {
-                uint4 v[2];
-                uint32_t ii[2], rr[2];
+    // Plain 16-bit maps, H and W multiples of 4, x 8-byte aligned (host-checked): one 4 x 4 tile of a map per thread.
+    // Its four rows go into the row-major map as they are; its four columns are put together from the rows' dwords
+    // with byte permutes and go into the column-major map, 8 bytes at a time.
+    auto stage_tiles = [&]() {
+        const int n_tiles = nb * (int)divTiles.d;        // tiles per image: (H / 4) * (W / 4)
+        for (int q = threadIdx.x; q < n_tiles; q += kBlock) {
+            uint32_t img, rest, hb, wb;
+            divmod((uint32_t)q, divTiles, img, rest);
+            divmod(rest, divWt, hb, wb);
+            const int in_img = (int)hb * 4 * p.W + (int)wb * 4;
+            const in_t *src = xin + ((size_t)(b0 + img) * p.D + d) * L + in_img;
+            uint2 row[4];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int vi = base + u * kBlock + (int)threadIdx.x;
-                    divmod((uint32_t)min(vi, n_vec - 1) * kItems, divL, ii[u], rr[u]);
-                    v[u] = *reinterpret_cast<const uint4 *>(xin + ((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]);
-                }
+            for (int k = 0; k < 4; ++k) row[k] = *reinterpret_cast<const uint2 *>(src + k * p.W);
+            in_t *dr = xR + (int)img * L + in_img;
+            in_t *dt = xT + (int)img * L + (int)wb * 4 * H + (int)hb * 4;
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int vi = base + u * kBlock + (int)threadIdx.x;
-                    if (vi < n_vec) {
-                        const uint32_t w32[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
-                        uint32_t h, w;
-                        divmod(rr[u], divW, h, w);
-                        *reinterpret_cast<uint4 *>(xR + lds_index<kEs>(vi * kItems)) = v[u];   // no pad word inside the block
-                        // column-major index of element i: row h, column w + i while that is < W, then row h + 1
-                        const int n_first = p.W - (int)w;
-                        const int t0 = (int)(ii[u] * L + w * H + h);
-                        const int t1 = (int)(ii[u] * L + h + 1) - n_first * H;
+            for (int k = 0; k < 4; ++k) *reinterpret_cast<uint2 *>(dr + k * p.W) = row[k];
+            // column c: (row0[c], row1[c]) and (row2[c], row3[c]); element c of a row is half c % 2 of its dword c / 2
+            const uint32_t r0[2] = {row[0].x, row[0].y}, r1[2] = {row[1].x, row[1].y};
+            const uint32_t r2[2] = {row[2].x, row[2].y}, r3[2] = {row[3].x, row[3].y};
 #pragma unroll
-                        for (int i = 0; i < kItems; ++i) {
-                            const int at_t = (i < n_first ? t0 : t1) + i * H;
-                            xT[lds_index<kEs>(at_t)] = in_t{(uint16_t)(w32[i / 2] >> (16 * (i % 2)))};
-                        }
-                    }
-                }
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t sel = c % 2 ? 0x07060302u : 0x05040100u;    // (low source . half, high source . half)
+                uint2 col;
+                col.x = __builtin_amdgcn_perm(r1[c / 2], r0[c / 2], sel);
+                col.y = __builtin_amdgcn_perm(r3[c / 2], r2[c / 2], sel);
+                *reinterpret_cast<uint2 *>(dt + c * H) = col;
             }
-        } else {
-            stage_elements();
         }
+    };
+    if constexpr (kFlat) {
+        if (p.stage_tiles) stage_tiles();
+        else stage_elements();
     } else {
         stage_elements();
     }
@@ -217,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         for (int i = threadIdx.x; i < 2 * plane_ext / 4; i += kBlock) planes4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (threadIdx.x < 2 * kItems) {
             in_t *m = threadIdx.x < kItems ? xR : xT;
-            m[lds_index<kEs>(core_zero_block(n_max) + (int)(threadIdx.x % kItems))] = in_t{};
+            m[map_index<kEs, kFlat>(core_zero_block(n_max) + (int)(threadIdx.x % kItems))] = in_t{};
         }
     }
     __syncthreads();
@@ -229,12 +253,13 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         bool valid;        // inside the stream
     };
 
-    // One pass: the outputs in yv (scan order) and the plane slots of its groups.
+    // One pass: C * h of its 8 items in yv (scan order) and the plane slots of its groups.  The skip term D * u is the
+    // same multiple of x[r] in all four directions and is added once, in the merge.
     auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kItems], GroupSlot (&slot)[kGroups]) {
         const int e0 = pass * kPass + lane * kItems;
-        const int j0 = (int)r.j0, i0 = (int)r.i0;
+        const int j0 = (int)r.j0;
         const int k = kGran == kItems ? kItems : min(kItems, L - j0);
-        const int img_base = i0 * L;
+        const int img_base = (int)r.img;
         float raw[kItems], Bv[kItems], Cv[kItems], uv[kItems];
         unpack_raw<in_t>(r.dl, raw);
         bool first[kGroups];
@@ -257,12 +282,25 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             base = valid ? base : zero_block;                                // past the end: u = 0
             slot[gi].valid = valid;
             slot[gi].plane_idx = lds_index<4>(base);
-            const in_t *src = xs + lds_index<kEs>(base);                     // no pad word inside an aligned block
-            float um[kGran];
+            const in_t *src = xs + map_index<kEs, kFlat>(base);              // no pad word inside an aligned block
+            if constexpr (kFlat) {
+                // one 16-byte read; backwards the four dwords are taken in the opposite order with their halves
+                // exchanged, one byte permute each (the selector is uniform over the wavefront)
+                const uint4 t = *reinterpret_cast<const uint4 *>(src);
+                const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
-            for (int c = 0; c < kGran; ++c) um[c] = to_f32(src[c]);
+                for (int jw = 0; jw < 4; ++jw) {
+                    const uint32_t o = __builtin_amdgcn_perm(w[3 - jw], w[jw], u_sel);
+                    uv[2 * jw] = to_f32(in_t{(uint16_t)(o & 0xffffu)});
+                    uv[2 * jw + 1] = to_f32(in_t{(uint16_t)(o >> 16)});
+                }
+            } else {
+                float um[kGran];
 #pragma unroll
-            for (int t = 0; t < kGran; ++t) uv[gi * kGran + t] = reverse ? um[kGran - 1 - t] : um[t];
+                for (int c = 0; c < kGran; ++c) um[c] = to_f32(src[c]);
+#pragma unroll
+                for (int t = 0; t < kGran; ++t) uv[gi * kGran + t] = reverse ? um[kGran - 1 - t] : um[t];
+            }
         }
         float dl[kItems], bias_items[kItems];
 #pragma unroll
@@ -285,7 +323,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         const float s_in = fmaf(a_ex, h_carry, h_ex);
         h_carry = fmaf(a_tot, h_carry, h_tot);
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) yv[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), Dv * uv[i]);
+        for (int i = 0; i < kItems; ++i) yv[i] = Cv[i] * fmaf(ac[i], s_in, hh[i]);
     };
 
     // Plane update of one pass: every entry is reached once by the forward and once by the backward direction of its
@@ -319,7 +357,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             raw = to_f32(dl_base[e]);
             Bv = gather_elem<in_t>(B_rsrc, B_soff + i * (uint32_t)p.B_bs + jj);
             Cv = gather_elem<in_t>(C_rsrc, C_soff + i * (uint32_t)p.C_bs + jj);
-            u = to_f32(xs[lds_index<kEs>(base)]);
+            u = to_f32(xs[map_index<kEs, kFlat>(base)]);
         }
         float dl = kSoftplus ? softplus_log2(fmaf(raw, kLog2e, bias * kLog2e)) : raw + bias;
         dl = valid ? dl : 0.0f;
@@ -329,7 +367,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         float a_ex, h_ex, a_tot, h_tot;
         wave_scan_pairs(a, b, a_ex, h_ex, a_tot, h_tot);
         const float h = fmaf(a, fmaf(a_ex, h_carry, h_ex), b);
-        const float y = fmaf(Cv, h, Dv * u);
+        const float y = Cv * h;
         float *dst = plane + lds_index<4>(base);
         if (!reverse && valid) *dst += y;
         __syncthreads();
@@ -337,8 +375,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
         __syncthreads();
     };
 
-    auto run_passes = [&](bool rev) {
-        const bool reverse = rev;
+    {
         float h_carry = 0.0f;
         for (int pass0 = 0; pass0 < n_pass; pass0 += kCoreBurst) {
 #pragma unroll
@@ -347,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
                 if (pass < n_pass) {                 // uniform over the workgroup: every wavefront meets every barrier
                     float yv[kItems];
                     GroupSlot slot[kGroups];
-                    compute(rev, pass, regs[q], h_carry, yv, slot);
+                    compute(reverse, pass, regs[q], h_carry, yv, slot);
                     if (!reverse) update_plane(false, yv, slot);
                     __syncthreads();
                     if (reverse) update_plane(true, yv, slot);
@@ -357,12 +394,42 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             }
         }
         if (short_tail) short_pass(reverse, h_carry);
-    };
-    // the direction is uniform per wavefront; both branches meet the same barriers
-    run_passes(dir >= 2);
+    }
 
-    // ---- merge: out[r] = A[r] + B[t(r)] ---------------------------------------------------------------------------
+    // ---- merge: out[r] = (A[r] + B[t(r)]) + (D0 + D1 + D2 + D3) * x[r] ---------------------------------------------
+    float Dsum = 0.0f;
+    if (p.Dv) Dsum = (p.Dv[d] + p.Dv[2 * p.D + (int)d]) + (p.Dv[p.D + (int)d] + p.Dv[3 * p.D + (int)d]);
     float *yo = reinterpret_cast<float *>(p.y);
+    if (p.tile_merge) {
+        // H and W multiples of 4, y 16-byte aligned (host-checked): one 4 x 4 tile of a map per thread.  Its rows are
+        // four consecutive entries of plane A each, its columns four consecutive entries of plane B each -- the
+        // transposition is a renaming of registers -- and every row leaves as one 16-byte store.
+        const int n_tiles = nb * (int)divTiles.d;
+        for (int q = threadIdx.x; q < n_tiles; q += kBlock) {
+            uint32_t img, rest, hb, wb;
+            divmod((uint32_t)q, divTiles, img, rest);
+            divmod(rest, divWt, hb, wb);
+            const int in_img = (int)hb * 4 * p.W + (int)wb * 4;
+            const int r0 = (int)img * L + in_img;
+            const int t0 = (int)img * L + (int)wb * 4 * H + (int)hb * 4;
+            float a[4][4], b[4][4], x[4][4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float *pa = planeA + lds_index<4>(r0 + k * p.W);      // no pad word inside an aligned group of 4
+                const float *pb = planeB + lds_index<4>(t0 + k * H);
+                const in_t *px = xR + map_index<kEs, kFlat>(r0 + k * p.W);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) { a[k][c] = pa[c]; b[k][c] = pb[c]; x[k][c] = to_f32(px[c]); }
+            }
+            float *dst = yo + ((size_t)(b0 + img) * p.D + d) * L + in_img;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                *reinterpret_cast<float4 *>(dst + k * p.W) =
+                    make_float4(fmaf(Dsum, x[k][0], a[k][0] + b[0][k]), fmaf(Dsum, x[k][1], a[k][1] + b[1][k]),
+                                fmaf(Dsum, x[k][2], a[k][2] + b[2][k]), fmaf(Dsum, x[k][3], a[k][3] + b[3][k]));
+        }
+        return;
+    }
     if (kGran >= 4 && p.vec_out && p.W >= 4) {
         // four consecutive positions per lane (L is a multiple of kGran, so they share an image and, with W >= 4, span
         // at most two rows): one 16-byte store
@@ -377,11 +444,13 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
                 divmod((uint32_t)idx, divL, i, r);
                 divmod(r, divW, h, w);
                 const float *pa = planeA + lds_index<4>(idx);               // no pad word inside an aligned group of 4
+                const in_t *px = xR + map_index<kEs, kFlat>(idx);
                 const int n_first = p.W - (int)w;
                 const int t0 = (int)(i * L + w * H + h), t1 = (int)(i * L + h + 1) - n_first * H;
                 float o[4];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) o[c] = pa[c] + planeB[lds_index<4>((c < n_first ? t0 : t1) + c * H)];
+                for (int c = 0; c < 4; ++c)
+                    o[c] = fmaf(Dsum, to_f32(px[c]), pa[c] + planeB[lds_index<4>((c < n_first ? t0 : t1) + c * H)]);
                 v[u] = make_float4(o[0], o[1], o[2], o[3]);
                 off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
             }
@@ -400,7 +469,8 @@ __global__ __launch_bounds__(kBlock) void ss2d_core_kernel(const CoreArgs p, Fas
             uint32_t i, r, h, w;
             divmod((uint32_t)idx, divL, i, r);
             divmod(r, divW, h, w);
-            v[u] = planeA[lds_index<4>(idx)] + planeB[lds_index<4>((int)(i * L + w * H + h))];
+            v[u] = fmaf(Dsum, to_f32(xR[map_index<kEs, kFlat>(idx)]),
+                        planeA[lds_index<4>(idx)] + planeB[lds_index<4>((int)(i * L + w * H + h))]);
             off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
         }
 #pragma unroll
@@ -417,6 +487,15 @@ static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b;
 template <typename in_t>
 static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t L = a.L;
+    // Granularity of the B / C gathers and of the walk: the largest of 8, 4, 1 positions that divides L and every B / C
+    // stride and for which the B / C bases are aligned.
+    int64_t g = core_gcd(L, kItems);
+    const int64_t strides[] = {a.B_ks, a.B_bs, a.C_ks, a.C_bs};
+    for (int64_t s : strides) g = core_gcd(g, s == 0 ? g : s);
+    const uintptr_t bases = reinterpret_cast<uintptr_t>(a.Bm) | reinterpret_cast<uintptr_t>(a.Cm);
+    while (g > 1 && (bases % (uintptr_t)(g * sizeof(in_t))) != 0) g /= 2;
+    if (g == 2) g = 1;
+    const bool flat = sizeof(in_t) == 2 && g == kItems;       // core_flat_maps
     // Images per workgroup.  A workgroup walks its CB images as one stream in passes of 512 positions, so the last
     // pass of a tile is partly empty (a remainder of up to 64 positions costs little, see short_pass); CB is chosen to
     // minimise the passes of the whole batch among the tile sizes whose LDS arrays still let six workgroups share a
@@ -424,7 +503,8 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     // on a 16-byte boundary when CB*L is a multiple of 8 elements.
     auto lds_bytes = [&](int64_t cb) {
         const int n = (int)(cb * L);
-        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)core_map_extent<(int)sizeof(in_t)>(n) * sizeof(in_t);
+        const int map_ext = flat ? core_map_extent<(int)sizeof(in_t), true>(n) : core_map_extent<(int)sizeof(in_t), false>(n);
+        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)map_ext * sizeof(in_t);
     };
     const int64_t align_rows = 8 / core_gcd(L, 8);
     auto passes = [&](int64_t images) {                       // cost of a tile in tenths of a full pass
@@ -449,20 +529,19 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     a.vec_ok = (reinterpret_cast<uintptr_t>(a.delta) % 16 == 0) && a.dl_ks % vec == 0 && a.dl_ds % vec == 0 &&
                (CB >= a.B || (CB * a.dl_bs) % vec == 0);
     a.vec_out = reinterpret_cast<uintptr_t>(a.y) % 16 == 0;   // 16-byte stores of the result (rows are multiples of 4 then)
-    int64_t g = core_gcd(L, kItems);
-    const int64_t strides[] = {a.B_ks, a.B_bs, a.C_ks, a.C_bs};
-    for (int64_t s : strides) g = core_gcd(g, s == 0 ? g : s);
-    const uintptr_t bases = reinterpret_cast<uintptr_t>(a.Bm) | reinterpret_cast<uintptr_t>(a.Cm);
-    while (g > 1 && (bases % (uintptr_t)(g * sizeof(in_t))) != 0) g /= 2;
-    if (g == 2) g = 1;
+    // 4 x 4 tiles of a map per thread for the staging of 16-bit maps (8-byte loads) and for the merge (16-byte stores)
+    const bool tiled = a.H % 4 == 0 && a.W % 4 == 0;
+    a.stage_tiles = flat && tiled && reinterpret_cast<uintptr_t>(a.x) % 8 == 0;
+    a.tile_merge = tiled && a.vec_out;
     const int64_t tiles = (a.B + CB - 1) / CB;
     const int64_t n_wg = tiles * a.D;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dD = make_fastdiv((uint32_t)a.D);
+    const FastDiv dT = make_fastdiv((uint32_t)(tiled ? (a.H / 4) * (a.W / 4) : 1)), dWt = make_fastdiv((uint32_t)(tiled ? a.W / 4 : 1));
 #define SS2D_CORE_LAUNCH(SP, G)                                                                                                     \
     do {                                                                                                                            \
-        if (a.vec_ok) hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD); \
-        else hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD);       \
+        if (a.vec_ok) hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt); \
+        else hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt);       \
     } while (0)
     if (a.softplus) {
         if (g == 8) SS2D_CORE_LAUNCH(true, 8); else if (g == 4) SS2D_CORE_LAUNCH(true, 4); else SS2D_CORE_LAUNCH(true, 1);
@@ -499,7 +578,7 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     const int64_t B_span = (3 * a.B_ks + (int64_t)(a.B - 1) * a.B_bs + L) * eb, C_span = (3 * a.C_ks + (int64_t)(a.B - 1) * a.C_bs + L) * eb;
     if (B_span >= 0x7fffffffll || C_span >= 0x7fffffffll) return SS2D_ENOTSUP;
     a.B_span_bytes = (uint32_t)B_span; a.C_span_bytes = (uint32_t)C_span;
-    a.CB = 1; a.vec_ok = 0; a.vec_out = 0;
+    a.CB = 1; a.vec_ok = 0; a.vec_out = 0; a.stage_tiles = 0; a.tile_merge = 0;
 
     hipStream_t s = (hipStream_t)stream;
     // 7 x 7 and 14 x 14 maps in the batch-innermost layout: one map row per lane, everything in registers
