@@ -14,10 +14,12 @@
 //     by a DPP scan over the lane group (forward for directions 0 / 1, in reverse lane order for 2 / 3), and the state
 //     entering the lane is pushed through its items.  A map's first item is forced to a = 0, which stops anything
 //     arriving from the neighbouring group;
-//   * u comes from two register copies of the map (its row, and its column obtained through one LDS transposition);
-//     the outputs of directions 0 + 2 accumulate in registers indexed by column, those of 1 + 3 in registers indexed by
-//     row; one more LDS transposition brings the second set into row layout and out = (y0 + y2) + (y1 + y3) leaves
-//     as plain row stores -- the association order of cross_merge_fwd (classification/models/csm_triton.py:61-62).
+//   * u comes from two register copies of the map as loaded (its row, 4-byte loads, and its column, 2-byte loads the
+//     first-level cache serves); the outputs of directions 1 + 3 accumulate in registers indexed by row and go through
+//     one LDS transposition (over delta tiles that are no longer needed) into row layout, those of 0 + 2 accumulate in
+//     registers indexed by column, and out = (y0 + y2) + (y1 + y3) + (D0 + D1 + D2 + D3) x leaves as plain row
+//     stores -- the association order of cross_merge_fwd (classification/models/csm_triton.py:61-62), the skip term,
+//     the same multiple of x in all four directions, added once.
 // No stream position, image boundary or LDS address is computed at run time.
 #include "scan_common.h"
 
@@ -64,6 +66,15 @@ template <typename in_t, int kS> struct Run {
             for (int j = 0; j < kS; ++j) w[j] = tile[elem_off + j];
         }
     }
+    __device__ __forceinline__ void pack(const uint16_t (&e)[kS]) {
+        if constexpr (kPacked) {
+#pragma unroll
+            for (int k = 0; k < kS / 2; ++k) w[k] = (uint32_t)e[2 * k] | ((uint32_t)e[2 * k + 1] << 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kS; ++j) w[j] = e[j];
+        }
+    }
     __device__ __forceinline__ float item(int j) const {
         if constexpr (kPacked) return (j & 1) ? unpack_hi<in_t>(w[j / 2]) : unpack_lo<in_t>(w[j / 2]);
         else return to_f32(in_t{(uint16_t)w[j]});
@@ -72,9 +83,9 @@ template <typename in_t, int kS> struct Run {
 
 constexpr int kSmallChans = kWavesPerWg;     // channels per workgroup: one per wavefront, all on the same images
 
-// Registers are capped so that as many workgroups share a CU as its LDS tiles allow (3 for 14 x 14, 5-6 for 7 x 7).
+// Registers are capped so that as many workgroups share a CU as its LDS tiles allow (4 for 14 x 14, 5-6 for 7 x 7).
 template <typename in_t, int kS, bool kSoftplus>
-__global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kernel(const CoreArgs p, int chan_quads, FastDiv div_quads) {
+__global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kernel(const CoreArgs p, int chan_quads, FastDiv div_quads) {
     constexpr int kLanes = kS <= 8 ? 8 : 16;                 // lanes per map
     constexpr int kMaps = kWave / kLanes;                    // maps per wavefront
     constexpr int kL = kS * kS;
@@ -87,11 +98,11 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
     // Everything a workgroup reads is fetched before its arithmetic starts (one memory latency per workgroup; the
     // registers that carry the loads are free again when the per-map arrays come alive):
     //   shared by the four wavefronts (same images): the B and C tiles of the four directions   [dir][B|C][tile]
-    //   per wavefront (its channel): the four delta tiles, and one fp32 tile that first holds the x maps (16-bit) for
-    //   the row -> column transposition and at the end the (y1 + y3) sums for the column -> row transposition
+    //   per wavefront (its channel): the four delta tiles, in the order of use 1, 3, 0, 2; once directions 1 and 3 are
+    //   done, the room of their two tiles holds the fp32 tile of the (y1 + y3) sums for the column -> row transposition
     __shared__ __align__(16) uint16_t s_bc[8 * kTileElems];
     __shared__ __align__(16) uint16_t s_dl[kWavesPerWg * 4 * kTileElems];
-    __shared__ __align__(16) float s_tr[kWavesPerWg * kTileElems];
+    static_assert(2 * kTileElems * sizeof(uint16_t) == kTileElems * sizeof(float), "the fp32 tile fits two delta tiles");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -107,7 +118,8 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
     const int gc = min(g, nb - 1), ic = min(i, kS - 1);      // clamped: every lane addresses real memory
 
     uint16_t *tile_dl = s_dl + wave * 4 * kTileElems;
-    float *tile_tr = s_tr + wave * kTileElems;
+    float *tile_tr = reinterpret_cast<float *>(tile_dl);    // over the tiles of directions 1 and 3 (slots 0 and 1)
+    constexpr int kSlot[4] = {2, 0, 3, 1};                   // direction -> slot of its delta tile
 
     // ---- fetch ------------------------------------------------------------------------------------------------------
     // delta: four tiles of this wavefront's channel, 16-byte buffer loads (range-checked: a short last tile reads zeros
@@ -146,31 +158,15 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
             r_bc[n] = make_uint4(is_c ? tc[0] : tb[0], is_c ? tc[1] : tb[1], is_c ? tc[2] : tb[2], is_c ? tc[3] : tb[3]);
         }
     }
-    // the map: this lane's row
-    float x_row[kS], x_col[kS];
+    // the map: this lane's row and this lane's column, as loaded (16-bit; widened where used)
+    Run<in_t, kS> x_row, x_col;
     {
-        const in_t *row = reinterpret_cast<const in_t *>(p.x) + ((int64_t)(b0 + gc) * p.D + d) * kL + ic * kS;
-        uint16_t *xt = reinterpret_cast<uint16_t *>(tile_tr);   // [map][row][col]
-        if constexpr (kS % 2 == 0) {
-            uint32_t w[kS / 2];
+        const in_t *map = reinterpret_cast<const in_t *>(p.x) + ((int64_t)(b0 + gc) * p.D + d) * kL;
+        x_row.read(reinterpret_cast<const uint16_t *>(map), ic * kS);
+        uint16_t e[kS];
 #pragma unroll
-            for (int k = 0; k < kS / 2; ++k) w[k] = reinterpret_cast<const uint32_t *>(row)[k];
-#pragma unroll
-            for (int k = 0; k < kS / 2; ++k) {
-                x_row[2 * k] = unpack_lo<in_t>(w[k]);
-                x_row[2 * k + 1] = unpack_hi<in_t>(w[k]);
-                if (active) reinterpret_cast<uint32_t *>(xt + gc * kL + ic * kS)[k] = w[k];
-            }
-        } else {
-            uint16_t e[kS];
-#pragma unroll
-            for (int j = 0; j < kS; ++j) e[j] = row[j].bits;
-#pragma unroll
-            for (int j = 0; j < kS; ++j) {
-                x_row[j] = to_f32(in_t{e[j]});
-                if (active) xt[gc * kL + ic * kS + j] = e[j];
-            }
-        }
+        for (int j = 0; j < kS; ++j) e[j] = map[j * kS + ic].bits;
+        x_col.pack(e);
     }
     // ---- park the streams in LDS ------------------------------------------------------------------------------------
 #pragma unroll
@@ -178,7 +174,7 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
 #pragma unroll
         for (int v = 0; v < kVecsPerLane; ++v) {
             const int vec = v * kWave + lane;
-            if (vec < kTileVecs) *reinterpret_cast<uint4 *>(tile_dl + k * kTileElems + vec * 8) = r_dl[k][v];
+            if (vec < kTileVecs) *reinterpret_cast<uint4 *>(tile_dl + kSlot[k] * kTileElems + vec * 8) = r_dl[k][v];
         }
 #pragma unroll
     for (int n = 0; n < kBcPerThread; ++n) {
@@ -187,16 +183,10 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
     }
     __syncthreads();                                         // the only workgroup barrier: B / C tiles are in place
     if (!chan_ok) return;
-    {
-        // ... and (through the x tile) this lane's column
-        const uint16_t *xt = reinterpret_cast<const uint16_t *>(tile_tr);
-#pragma unroll
-        for (int j = 0; j < kS; ++j) x_col[j] = to_f32(in_t{xt[gc * kL + j * kS + ic]});
-    }
 
-    float acc_rm[kS], acc_cm[kS];                            // y0 + y2 by column of row i;  y1 + y3 by row of column i
+    float acc[kS];                                           // y1 + y3 by row of column i, then y0 + y2 by column of row i
 #pragma unroll
-    for (int j = 0; j < kS; ++j) { acc_rm[j] = 0.0f; acc_cm[j] = 0.0f; }
+    for (int j = 0; j < kS; ++j) acc[j] = 0.0f;
 
     auto direction = [&](auto dir_tag) {
         constexpr int kDir = decltype(dir_tag)::value;
@@ -205,20 +195,19 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
         // met from its far end -- item j of the run is column (row) kS-1-j
         const int run = gc * kL + (kRev ? kS - 1 - ic : ic) * kS;
         Run<in_t, kS> raw, Bv, Cv;
-        raw.read(tile_dl + kDir * kTileElems, run);
+        raw.read(tile_dl + kSlot[kDir] * kTileElems, run);
         Bv.read(s_bc + (2 * kDir) * kTileElems, run);
         Cv.read(s_bc + (2 * kDir + 1) * kTileElems, run);
 
         const int kd = kDir * p.D + d;
         const float A2 = p.A[kd] * kLog2e;
-        const float Dk = p.Dv ? p.Dv[kd] : 0.0f;
         const float bias = p.bias ? p.bias[kd] : 0.0f;
         const bool first = kRev ? i == kS - 1 : i == 0;      // the lane that starts the map in this direction's order
         float ac[kS], hh[kS];
 #pragma unroll
         for (int j = 0; j < kS; ++j) {
             const int m = kRev ? kS - 1 - j : j;             // column (directions 0 / 2) or row (1 / 3) of item j
-            const float u = kCol ? x_col[m] : x_row[m];
+            const float u = kCol ? x_col.item(m) : x_row.item(m);
             float dl;
             if constexpr (kSoftplus) dl = softplus_log2(fmaf(raw.item(j), kLog2e, bias * kLog2e));
             else dl = raw.item(j) + bias;
@@ -234,27 +223,28 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 3) void ss2d_core_small_kerne
 #pragma unroll
         for (int j = 0; j < kS; ++j) {
             const int m = kRev ? kS - 1 - j : j;
-            const float u = kCol ? x_col[m] : x_row[m];
-            const float y = fmaf(Cv.item(j), fmaf(ac[j], h_in, hh[j]), Dk * u);
-            if constexpr (kCol) acc_cm[m] += y; else acc_rm[m] += y;
+            acc[m] += Cv.item(j) * fmaf(ac[j], h_in, hh[j]);
         }
     };
-    // (y0 + y2) and (y1 + y3): the first addition into a zero is exact, the second rounds once
-    direction(std::integral_constant<int, 0>{});
-    direction(std::integral_constant<int, 2>{});
+    // (y1 + y3), then (y0 + y2): the first addition into a zero is exact, the second rounds once
     direction(std::integral_constant<int, 1>{});
     direction(std::integral_constant<int, 3>{});
-
-    // ---- merge: bring (y1 + y3) from column layout to row layout through LDS, add, store the row --------------------
-    wave_lds_sync();                                         // every lane has read its column of the x tile
+    // bring (y1 + y3) from column layout to row layout through LDS: this lane is column i, element (row j, col i)
+    wave_lds_sync();                                         // every lane has read its runs of the delta tiles 1 and 3
     if (active) {                                            // (idle lanes address the last row / map: they must not write)
 #pragma unroll
-        for (int j = 0; j < kS; ++j) tile_tr[gc * kL + j * kS + ic] = acc_cm[j];   // this lane is column i: element (row j, col i)
+        for (int j = 0; j < kS; ++j) { tile_tr[gc * kL + j * kS + ic] = acc[j]; acc[j] = 0.0f; }
     }
+    direction(std::integral_constant<int, 0>{});
+    direction(std::integral_constant<int, 2>{});
+
+    // ---- merge: add the transposed sums and the skip term, store the row ---------------------------------------------
+    float Dsum = 0.0f;
+    if (p.Dv) Dsum = (p.Dv[d] + p.Dv[2 * p.D + d]) + (p.Dv[p.D + d] + p.Dv[3 * p.D + d]);
     wave_lds_sync();
     float out[kS];
 #pragma unroll
-    for (int j = 0; j < kS; ++j) out[j] = acc_rm[j] + tile_tr[gc * kL + ic * kS + j];
+    for (int j = 0; j < kS; ++j) out[j] = fmaf(Dsum, x_row.item(j), acc[j] + tile_tr[gc * kL + ic * kS + j]);
     if (active) {
         float *yo = reinterpret_cast<float *>(p.y) + ((int64_t)(b0 + g) * p.D + d) * kL + i * kS;
         if constexpr (kS % 2 == 0) {
