@@ -162,18 +162,22 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xb), 0, H * W * D * 2, 0x00020000);
     const int n_in = (rows + 2) * Wp;
     constexpr int kLoadsInFlight = 6;
+    uint32_t step_r, step_c;                                     // (row, column) of a padded-tile element advance by this per load
+    divmod((uint32_t)(kBlock / 4), divWp, step_r, step_c);
     for (int e0 = threadIdx.x / 4; e0 < n_in; e0 += kLoadsInFlight * (kBlock / 4)) {
         uint4 v[kLoadsInFlight];
+        uint32_t rr, cc;
+        divmod((uint32_t)e0, divWp, rr, cc);
 #pragma unroll
         for (int u = 0; u < kLoadsInFlight; ++u) {
             const int e = e0 + u * (kBlock / 4);
-            uint32_t rr, cc;
-            divmod((uint32_t)e, divWp, rr, cc);
             const int h = h0 - 1 + (int)rr, w = (int)cc - 1;
             const bool inside = e < n_in && h >= 0 && h < H && w >= 0 && w < W && c0 < D;
             const uint32_t off = inside ? (uint32_t)((h * W + w) * D + c0) * 2u : 0x7ffffff0u;
             const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
             v[u] = make_uint4(t[0], t[1], t[2], t[3]);
+            rr += step_r; cc += step_c;
+            if (cc >= (uint32_t)Wp) { cc -= (uint32_t)Wp; rr += 1; }
         }
 #pragma unroll
         for (int u = 0; u < kLoadsInFlight; ++u) {
@@ -194,13 +198,17 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             const uint4 v = reinterpret_cast<const uint4 *>(wsrc)[k];
             wraw[4 * k] = v.x; wraw[4 * k + 1] = v.y; wraw[4 * k + 2] = v.z; wraw[4 * k + 3] = v.w;
         }
-        // element e = ci * 9 + t sits in half (e & 1) of dword e / 2
-        auto elem = [&](int e) -> uint32_t { return (e & 1) ? (wraw[e / 2] >> 16) : (wraw[e / 2] & 0xffffu); };
+        // element e = ci * 9 + t sits in half (e & 1) of dword e / 2: a pair of taps starting at an even element IS a
+        // dword of the weights as loaded, one starting at an odd element straddles two (one funnel shift)
+        auto pair_at = [&](int e) -> uint32_t {
+            return (e & 1) ? __builtin_amdgcn_alignbit(wraw[e / 2 + 1], wraw[e / 2], 16) : wraw[e / 2];
+        };
 #pragma unroll
         for (int ci = 0; ci < 8; ++ci) {
 #pragma unroll
-            for (int tp = 0; tp < 4; ++tp) wp2[ci][tp] = elem(ci * 9 + 2 * tp) | (elem(ci * 9 + 2 * tp + 1) << 16);
-            wp2[ci][4] = elem(ci * 9 + 8);
+            for (int tp = 0; tp < 4; ++tp) wp2[ci][tp] = pair_at(ci * 9 + 2 * tp);
+            const int e8 = ci * 9 + 8;
+            wp2[ci][4] = (e8 & 1) ? (wraw[e8 / 2] >> 16) : (wraw[e8 / 2] & 0xffffu);
         }
 #pragma unroll
         for (int ci = 0; ci < 8; ++ci) bv[ci] = 0.0f;
@@ -213,6 +221,11 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     for (int pidx = threadIdx.x / 4; pidx < n_out; pidx += kBlock / 4) {
         uint32_t ph, pw;
         divmod((uint32_t)pidx, divW, ph, pw);
+        // Column of this position in the rows of the output tile: the rows of channel group cv are rotated by 16 * cv
+        // elements, so that the four groups of a wavefront write into different banks (their rows start a multiple
+        // of 32 banks apart).
+        int col = pidx + 16 * cv;
+        col = col >= out_pitch ? col - out_pitch : col;
         // nine taps as four pairs and a single: the two taps of a pair are brought side by side per channel (one byte
         // permute per channel pair and tap pair) and multiplied-accumulated by one dot instruction per channel
         uint4 tap[9];
@@ -246,8 +259,8 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
         for (int ci = 0; ci < 8; ci += 2) {
             uint32_t o = pack2_from_f32<T>(acc[ci], acc[ci + 1]);                                  // conv output as stored
             if (kSilu) o = pack2_from_f32<T>(silu_fast(unpack_lo<T>(o)), silu_fast(unpack_hi<T>(o)));
-            out_tile[(cv * 8 + ci) * out_pitch + pidx] = (uint16_t)(o & 0xffffu);
-            out_tile[(cv * 8 + ci + 1) * out_pitch + pidx] = (uint16_t)(o >> 16);
+            out_tile[(cv * 8 + ci) * out_pitch + col] = (uint16_t)(o & 0xffffu);
+            out_tile[(cv * 8 + ci + 1) * out_pitch + col] = (uint16_t)(o >> 16);
         }
     }
     __syncthreads();
@@ -256,17 +269,25 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     const int L = H * W;
     const int pieces = (n_out + 7) / 8;
     const bool vec = ((h0 * W) % 8 == 0) && (L % 8 == 0);
-    for (int e = threadIdx.x; e < kDwCh * pieces; e += kBlock) {
-        const int c = e / pieces, piece = e - c * pieces;
-        const int cg = c_base + c;
-        if (cg < D) {
-            T *yo = y + ((size_t)b * D + cg) * L + (size_t)h0 * W + piece * 8;
-            const uint16_t *src = out_tile + c * out_pitch + piece * 8;
-            if (vec && piece * 8 + 8 <= n_out) {
-                *reinterpret_cast<uint4 *>(yo) = *reinterpret_cast<const uint4 *>(src);
-            } else {
-                for (int i = 0; i < 8 && piece * 8 + i < n_out; ++i) yo[i] = T{src[i]};
+    // a group of 8, 16 or 32 lanes per channel (the smallest that covers the tile), a lane per piece of 8 positions: no
+    // division, and short tiles keep most lanes busy (tiles hold at most 256 positions)
+    const int lg = pieces <= 8 ? 3 : pieces <= 16 ? 4 : 5;
+    const int piece = threadIdx.x & ((1 << lg) - 1), c_first = threadIdx.x >> lg, c_step = kBlock >> lg;
+    if (piece < pieces) {
+        T *yo = y + ((size_t)b * D + c_base + c_first) * L + (size_t)h0 * W + piece * 8;
+        const bool whole = vec && piece * 8 + 8 <= n_out;
+        for (int c = c_first; c < kDwCh; c += c_step) {
+            if (c_base + c < D) {
+                int col = piece * 8 + 16 * (c / 8);                  // the row's rotation (see above); pieces stay whole
+                col = col >= out_pitch ? col - out_pitch : col;
+                const uint16_t *src = out_tile + c * out_pitch + col;
+                if (whole) {
+                    *reinterpret_cast<uint4 *>(yo) = *reinterpret_cast<const uint4 *>(src);
+                } else {
+                    for (int i = 0; i < 8 && piece * 8 + i < n_out; ++i) yo[i] = T{src[i]};
+                }
             }
+            yo += (size_t)c_step * L;
         }
     }
 }
@@ -314,7 +335,7 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             // TH rows per workgroup: about 224 positions, LDS within 64 KiB
             int TH = 224 / W;
             TH = TH < 1 ? 1 : (TH > H ? H : TH);
-            const int out_pitch = ((TH * W + 7) / 8) * 8 + 8;
+            const int out_pitch = ((TH * W + 15) / 16) * 16;          // a multiple of 16 elements: rows rotate by 16, 32, 48
             const size_t smem = ((size_t)(TH + 2) * (W + 2) * kDwCh + (size_t)kDwCh * out_pitch) * sizeof(uint16_t);
             const int row_tiles = (H + TH - 1) / TH, ch_tiles = (D + kDwCh - 1) / kDwCh;
             const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
