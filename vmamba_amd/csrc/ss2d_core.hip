@@ -17,12 +17,19 @@
 //     magnitude slower than plain LDS traffic on this chip, so the updates are plain read-add-write sequences kept
 //     apart by construction: the four wavefronts advance pass by pass, in each pass the forward directions update
 //     the planes, a barrier, then the backward directions, a barrier;
-//   * finally out[r] = A[r] + B[t(r)] is written once.
+//   * finally out[r] = (A[r] + B[t(r)]) + (D0 + D1 + D2 + D3) * x[r] is written once: the skip term D_k * u is the same
+//     multiple of x[r] in all four directions, so it is added once here instead of once per direction and item.
 // HBM traffic per element: x (s_in) + 4 delta (4 s_in) + out (s_out) = 14 bytes instead of 62.
 //
 // LDS banks: a lane owns 8 consecutive positions, so for a fixed item the 64 lanes touch addresses 8 apart, which
-// would fold onto 4 of the 32 banks.  All four LDS arrays therefore skip one 4-byte word after every 32 words
-// (lds_index): lanes 0..31 of one access then fall into 32 different banks.
+// would fold onto 4 of the 32 banks.  The fp32 planes therefore skip one 4-byte word after every 32 words
+// (lds_index): lanes 0..31 of one access then fall into 32 different banks.  The maps are padded the same way only
+// where they are read element by element; 16-bit maps walked in aligned blocks of 8 are read 16 bytes per lane,
+// consecutive lanes consecutive addresses, and are plain arrays (map_index).
+//
+// Staging and merge work on 4 x 4 tiles of a map, one per thread, when H and W are multiples of 4: rows are 8-byte
+// (staging) or 16-byte (merge) accesses on the row-major side, columns the same on the column-major side, and the
+// transposition between them happens in registers.
 //
 // The CB images of a workgroup are walked as one stream per direction (restart by a = 0 at each image start, as
 // in the flat scan kernel), which needs their delta rows adjacent in memory: delta is therefore taken with
