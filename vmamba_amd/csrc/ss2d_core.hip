@@ -63,31 +63,42 @@ template <int kBytes, bool kFlat> __host__ __device__ __forceinline__ constexpr 
     return kFlat ? core_zero_block(n) + kItems : lds_extent<kBytes>(core_zero_block(n) + kItems);
 }
 template <typename in_t, int kGran> constexpr bool core_flat_maps() { return sizeof(in_t) == 2 && kGran == kItems; }
+// Positions per lane and pass: 8, or 16 (two blocks of 8, 1024 positions per pass; 16-bit maps walked in blocks only).
+// With 16 the lane-local scan runs over 16 items and the wavefront scan, the plane bookkeeping and the loop are paid once
+// per 1024 positions instead of once per 512; it needs more registers (five wavefronts per SIMD instead of six) and
+// longer tiles, so the host picks it where a tile's LDS arrays keep a CU below six workgroups anyway.
+template <bool kWide> constexpr int core_items() { return kWide ? 2 * kItems : kItems; }
 
 // Wavefronts per SIMD the register allocation aims at: six for the 16-bit walks in blocks (what their LDS arrays allow;
 // a few values that only live before and after the pass loop are then parked in scratch memory), four otherwise.
-template <typename in_t, int kGran> constexpr int core_min_waves() { return sizeof(in_t) == 2 && kGran >= 4 ? 6 : 4; }
+template <typename in_t, int kGran, bool kWide> constexpr int core_min_waves() { return sizeof(in_t) == 2 && kGran >= 4 && !kWide ? 6 : 4; }
 
 constexpr int kCoreBurst = 2;     // passes whose delta / B / C loads are in flight per wavefront
 
 // What one pass of one lane loads from memory, as it arrives.
-template <typename in_t, int kGran>
+template <typename in_t, int kGran, bool kWide>
 struct CorePassLoads {
-    static constexpr int kGroups = kItems / kGran;
+    static constexpr int kIt = core_items<kWide>();
+    static constexpr int kGroups = kIt / kGran;
+    static constexpr int kBlocks = kIt / kItems;
     static constexpr int kWords = gather_words<in_t, kGran>();
-    Raw8<in_t> dl;
+    Raw8<in_t> dl[kBlocks];
     uint32_t b[kGroups][kWords], c[kGroups][kWords];
     uint32_t img, j0;     // first element of the image (its index times L) and position in it of the lane's first item
 };
 
-template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta>
-__global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD, FastDiv divTiles,
+template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta, bool kWide>
+__global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD, FastDiv divTiles,
                                                            FastDiv divWt) {
     extern __shared__ __align__(16) float core_smem[];
     constexpr int kEs = (int)sizeof(in_t);
-    constexpr int kGroups = kItems / kGran;
     constexpr bool kFlat = core_flat_maps<in_t, kGran>();
-    using Loads = CorePassLoads<in_t, kGran>;
+    static_assert(!kWide || core_flat_maps<in_t, kGran>(), "16 positions per lane: 16-bit maps walked in blocks of 8 only");
+    constexpr int kIt = core_items<kWide>();             // positions per lane and pass
+    constexpr int kBlocks = kIt / kItems;
+    constexpr int kGroups = kIt / kGran;
+    constexpr int kPassLen = kWave * kIt;                // positions per pass
+    using Loads = CorePassLoads<in_t, kGran, kWide>;
     const int L = p.L, H = p.H;
     const int n_max = p.CB * L;
     const int plane_ext = lds_extent<4>(n_max), map_ext = core_map_extent<kEs, kFlat>(n_max);
@@ -121,32 +132,35 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
     // B / C rows of consecutive images adjacent in memory (what one x_proj GEMM per direction writes): a lane's offset
     // into them is its stream position
     const bool bc_dense = p.B_bs == L && p.C_bs == L;
-    // passes of 512 positions; a remainder of at most 64 positions is walked one position per lane instead
-    const int tail_len = n_el % kPass;
+    // passes of 512 or 1024 positions; a remainder of at most 64 positions is walked one position per lane instead
+    const int tail_len = n_el % kPassLen;
     const bool short_tail = tail_len > 0 && tail_len <= kWave;
-    const int n_pass = short_tail ? n_el / kPass : (n_el + kPass - 1) / kPass;
+    const int n_pass = short_tail ? n_el / kPassLen : (n_el + kPassLen - 1) / kPassLen;
 
     // Image and position of this lane's first item in the pass issued next: passes are issued strictly in order, so
     // the pair just advances by 512 positions each time (no division in the loop).
     uint32_t next_img, next_j, step_img, step_j;
-    divmod((uint32_t)(lane * kItems), divL, next_img, next_j);
-    divmod((uint32_t)kPass, divL, step_img, step_j);
+    divmod((uint32_t)(lane * kIt), divL, next_img, next_j);
+    divmod((uint32_t)kPassLen, divL, step_img, step_j);
     next_img *= (uint32_t)L; step_img *= (uint32_t)L;
     auto issue = [&](int pass, Loads &r) {
-        const int e0 = pass * kPass + lane * kItems;
-        if constexpr (kVecDelta) {
-            // the stream starts 16-byte aligned (host-checked); the descriptor's range check returns 0 for the dwords
-            // past its end.  What those items hold is immaterial: they follow every valid item of the stream, their u
-            // is 0 and their outputs are never stored.
-            const int byte_off = e0 * kEs;
-            const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off, 0, 0);
-            r.dl.w[0] = t0[0]; r.dl.w[1] = t0[1]; r.dl.w[2] = t0[2]; r.dl.w[3] = t0[3];
-            if constexpr (kEs == 4) {
-                const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off + 16, 0, 0);
-                r.dl.w[4] = t1[0]; r.dl.w[5] = t1[1]; r.dl.w[6] = t1[2]; r.dl.w[7] = t1[3];
+        const int e0 = pass * kPassLen + lane * kIt;
+#pragma unroll
+        for (int blk = 0; blk < kBlocks; ++blk) {
+            if constexpr (kVecDelta) {
+                // the stream starts 16-byte aligned (host-checked); the descriptor's range check returns 0 for the dwords
+                // past its end.  What those items hold is immaterial: they follow every valid item of the stream, their u
+                // is 0 and their outputs are never stored.
+                const int byte_off = (e0 + blk * kItems) * kEs;
+                const auto t0 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off, 0, 0);
+                r.dl[blk].w[0] = t0[0]; r.dl[blk].w[1] = t0[1]; r.dl[blk].w[2] = t0[2]; r.dl[blk].w[3] = t0[3];
+                if constexpr (kEs == 4) {
+                    const auto t1 = __builtin_amdgcn_raw_buffer_load_b128(dl_rsrc, byte_off + 16, 0, 0);
+                    r.dl[blk].w[4] = t1[0]; r.dl[blk].w[5] = t1[1]; r.dl[blk].w[6] = t1[2]; r.dl[blk].w[7] = t1[3];
+                }
+            } else {
+                r.dl[blk] = load_raw<in_t, false>(dl_base, e0 + blk * kItems, n_el, delta_fill<kSoftplus>());
             }
-        } else {
-            r.dl = load_raw<in_t, false>(dl_base, e0, n_el, delta_fill<kSoftplus>());
         }
         r.img = next_img; r.j0 = next_j;
         next_img += step_img; next_j += step_j;
@@ -161,12 +175,12 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
         }
         uint32_t i0, rem;
         divmod(r.img, divL, i0, rem);
-        const int k = kGran == kItems ? kItems : min(kItems, L - (int)r.j0);   // items before the next image starts
+        const int k = kGran == kIt ? kIt : min(kIt, L - (int)r.j0);   // items before the next image starts
         const uint32_t B_a = i0 * (uint32_t)p.B_bs + r.j0, C_a = i0 * (uint32_t)p.C_bs + r.j0;   // image i0
         const uint32_t B_b = B_a + (uint32_t)p.B_bs - (uint32_t)(r.j0 + k), C_b = C_a + (uint32_t)p.C_bs - (uint32_t)(r.j0 + k);
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
-            const bool in_a = kGran == kItems ? true : gi * kGran < k;
+            const bool in_a = kGran == kIt ? true : gi * kGran < k;
             // image i0: position j0 + gi*kGran; image i0 + 1: position gi*kGran - k
             gather_group_raw<in_t, kGran>(B_rsrc, (in_a ? B_a : B_b) + gi * kGran, B_soff, r.b[gi]);
             gather_group_raw<in_t, kGran>(C_rsrc, (in_a ? C_a : C_b) + gi * kGran, C_soff, r.c[gi]);
@@ -260,19 +274,28 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
         bool valid;        // inside the stream
     };
 
-    // One pass: C * h of its 8 items in yv (scan order) and the plane slots of its groups.  The skip term D * u is the
+    // One pass: C * h of its items in yv (scan order) and the plane slots of its groups.  The skip term D * u is the
     // same multiple of x[r] in all four directions and is added once, in the merge.
-    auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kItems], GroupSlot (&slot)[kGroups]) {
-        const int e0 = pass * kPass + lane * kItems;
+    auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kIt], GroupSlot (&slot)[kGroups]) {
+        const int e0 = pass * kPassLen + lane * kIt;
         const int j0 = (int)r.j0;
-        const int k = kGran == kItems ? kItems : min(kItems, L - j0);
+        const int k = kGran == kIt ? kIt : min(kIt, L - j0);
         const int img_base = (int)r.img;
-        float raw[kItems], Bv[kItems], Cv[kItems], uv[kItems];
-        unpack_raw<in_t>(r.dl, raw);
+        float dl[kIt], Bv[kIt], Cv[kIt], uv[kIt];
+#pragma unroll
+        for (int blk = 0; blk < kBlocks; ++blk) {
+            float raw8[kItems], bias8[kItems], dl8[kItems];
+            unpack_raw<in_t>(r.dl[blk], raw8);
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) bias8[i] = bias;
+            delta_transform<kSoftplus>(raw8, bias8, dl8);
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) dl[blk * kItems + i] = dl8[i];
+        }
         bool first[kGroups];
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
-            const bool in_a = kGran == kItems ? true : gi * kGran < k;
+            const bool in_a = kGran == kIt ? true : gi * kGran < k;
             const int jg = in_a ? j0 + gi * kGran : gi * kGran - k;          // position of the group in its image
             const int img_off = in_a ? img_base : img_base + L;              // img * L
             first[gi] = jg == 0;
@@ -298,8 +321,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
 #pragma unroll
                 for (int jw = 0; jw < 4; ++jw) {
                     const uint32_t o = __builtin_amdgcn_perm(w[3 - jw], w[jw], u_sel);
-                    uv[2 * jw] = to_f32(in_t{(uint16_t)(o & 0xffffu)});
-                    uv[2 * jw + 1] = to_f32(in_t{(uint16_t)(o >> 16)});
+                    uv[gi * kGran + 2 * jw] = to_f32(in_t{(uint16_t)(o & 0xffffu)});
+                    uv[gi * kGran + 2 * jw + 1] = to_f32(in_t{(uint16_t)(o >> 16)});
                 }
             } else {
                 float um[kGran];
@@ -309,13 +332,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
                 for (int t = 0; t < kGran; ++t) uv[gi * kGran + t] = reverse ? um[kGran - 1 - t] : um[t];
             }
         }
-        float dl[kItems], bias_items[kItems];
+        float ac[kIt], hh[kIt];
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) bias_items[i] = bias;
-        delta_transform<kSoftplus>(raw, bias_items, dl);
-        float ac[kItems], hh[kItems];
-#pragma unroll
-        for (int i = 0; i < kItems; ++i) {
+        for (int i = 0; i < kIt; ++i) {
             // past the end of the stream delta was filled so that dl = 0 (softplus) or is zeroed here; u is 0 there and
             // B finite (the buffer load returns 0 out of range), so the pair is the identity (1, 0)
             if constexpr (!kSoftplus) dl[i] = slot[i / kGran].valid ? dl[i] : 0.0f;
@@ -326,18 +345,18 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
             hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
         }
         float a_ex, h_ex, a_tot, h_tot;
-        wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+        wave_scan_pairs(ac[kIt - 1], hh[kIt - 1], a_ex, h_ex, a_tot, h_tot);
         const float s_in = fmaf(a_ex, h_carry, h_ex);
         h_carry = fmaf(a_tot, h_carry, h_tot);
 #pragma unroll
-        for (int i = 0; i < kItems; ++i) yv[i] = Cv[i] * fmaf(ac[i], s_in, hh[i]);
+        for (int i = 0; i < kIt; ++i) yv[i] = Cv[i] * fmaf(ac[i], s_in, hh[i]);
     };
 
     // Plane update of one pass: every entry is reached once by the forward and once by the backward direction of its
     // plane; both add to the zero-initialised entry, so it ends as fl(y_fwd + y_bwd) whatever the order.  Only when the
     // two meet in the same pass could the read-add-write sequences overlap: the barrier between the two halves of a
     // pass keeps them apart.
-    auto update_plane = [&](bool reverse, const float (&yv)[kItems], const GroupSlot (&slot)[kGroups]) {
+    auto update_plane = [&](bool reverse, const float (&yv)[kIt], const GroupSlot (&slot)[kGroups]) {
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             if (slot[gi].valid) {
@@ -351,10 +370,10 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
         }
     };
 
-    // The short last pass: lane l holds stream position 512 * n_pass + l.  Same arithmetic and the same two-barrier
+    // The short last pass: lane l holds stream position kPassLen * n_pass + l.  Same arithmetic and the same two-barrier
     // plane update as a full pass, one item per lane.
     auto short_pass = [&](bool reverse, float h_carry) {
-        const int e = n_pass * kPass + lane;
+        const int e = n_pass * kPassLen + lane;
         const bool valid = e < n_el;
         uint32_t i, jj;
         divmod((uint32_t)min(e, n_el - 1), divL, i, jj);
@@ -389,7 +408,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran>())) void ss2d_
             for (int q = 0; q < kCoreBurst; ++q) {
                 const int pass = pass0 + q;
                 if (pass < n_pass) {                 // uniform over the workgroup: every wavefront meets every barrier
-                    float yv[kItems];
+                    float yv[kIt];
                     GroupSlot slot[kGroups];
                     compute(reverse, pass, regs[q], h_carry, yv, slot);
                     if (!reverse) update_plane(false, yv, slot);
@@ -491,6 +510,13 @@ constexpr size_t kCoreSixPerCu = 26 * 1024;     // a sixth of the 160 KB of LDS 
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
 
+// LDS bytes of a tile of n positions: two fp32 planes and two maps.
+template <typename in_t> static size_t lds_bytes_of(int64_t n64, bool flat) {
+    const int n = (int)n64;
+    const int map_ext = flat ? core_map_extent<(int)sizeof(in_t), true>(n) : core_map_extent<(int)sizeof(in_t), false>(n);
+    return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)map_ext * sizeof(in_t);
+}
+
 template <typename in_t>
 static int launch_core(CoreArgs a, hipStream_t stream) {
     const int64_t L = a.L;
@@ -503,29 +529,30 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     while (g > 1 && (bases % (uintptr_t)(g * sizeof(in_t))) != 0) g /= 2;
     if (g == 2) g = 1;
     const bool flat = sizeof(in_t) == 2 && g == kItems;       // core_flat_maps
+    // 16 positions per lane and pass where one image alone takes more LDS than a sixth of a CU (the tile cannot be
+    // shortened, six workgroups per CU are out of reach anyway); else 8, with tiles that let six workgroups share a CU
+    const bool wide = flat && a.dl_bs == L && lds_bytes_of<in_t>(L, true) > kCoreSixPerCu;
+    const int64_t pass_len = wide ? 2 * kPass : kPass;         // core_items * 64
+    const size_t lds_cap = wide ? 40 * 1024 : kCoreSixPerCu;
     // Images per workgroup.  A workgroup walks its CB images as one stream in passes of 512 positions, so the last
     // pass of a tile is partly empty (a remainder of up to 64 positions costs little, see short_pass); CB is chosen to
     // minimise the passes of the whole batch among the tile sizes whose LDS arrays still let six workgroups share a
     // CU (~2200 positions; measured: more resident workgroups beat longer tiles).  A workgroup's first delta row sits
     // on a 16-byte boundary when CB*L is a multiple of 8 elements.
-    auto lds_bytes = [&](int64_t cb) {
-        const int n = (int)(cb * L);
-        const int map_ext = flat ? core_map_extent<(int)sizeof(in_t), true>(n) : core_map_extent<(int)sizeof(in_t), false>(n);
-        return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)map_ext * sizeof(in_t);
-    };
+    auto lds_bytes = [&](int64_t cb) { return lds_bytes_of<in_t>(cb * L, flat); };
     const int64_t align_rows = 8 / core_gcd(L, 8);
     auto passes = [&](int64_t images) {                       // cost of a tile in tenths of a full pass
-        const int64_t n = images * L, rem = n % kPass;
-        return 10 * (n / kPass) + (rem == 0 ? 0 : rem <= kWave ? 3 : 10);
+        const int64_t n = images * L, rem = n % pass_len;
+        return 10 * (n / pass_len) + (rem == 0 ? 0 : rem <= kWave ? 3 : 10);
     };
     int64_t CB = 1;
     if (a.dl_bs == L) {                                       // adjacent delta rows need the batch-innermost layout
         int64_t best = -1;
-        for (int64_t cb = align_rows; cb < a.B && lds_bytes(cb) <= kCoreSixPerCu; cb += align_rows) {
+        for (int64_t cb = align_rows; cb < a.B && lds_bytes(cb) <= lds_cap; cb += align_rows) {
             const int64_t cost = (a.B / cb) * passes(cb) + passes(a.B % cb);
             if (best < 0 || cost <= best) { best = cost; CB = cb; }
         }
-        if (lds_bytes(a.B) <= kCoreSixPerCu && (best < 0 || passes(a.B) <= best)) CB = a.B;   // a single tile starts at image 0
+        if (lds_bytes(a.B) <= lds_cap && (best < 0 || passes(a.B) <= best)) CB = a.B;   // a single tile starts at image 0
     }
     const size_t smem = lds_bytes(CB);
     if (smem > kCoreMaxLds) return SS2D_ENOTSUP;
@@ -545,16 +572,21 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dD = make_fastdiv((uint32_t)a.D);
     const FastDiv dT = make_fastdiv((uint32_t)(tiled ? (a.H / 4) * (a.W / 4) : 1)), dWt = make_fastdiv((uint32_t)(tiled ? a.W / 4 : 1));
+#define SS2D_CORE_LAUNCH_W(SP, G, V, W16)                                                                                         \
+    hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, V, W16>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt)
 #define SS2D_CORE_LAUNCH(SP, G)                                                                                                     \
     do {                                                                                                                            \
-        if (a.vec_ok) hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt); \
-        else hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt);       \
+        if constexpr (G == kItems && sizeof(in_t) == 2) {                                                                          \
+            if (wide) { if (a.vec_ok) SS2D_CORE_LAUNCH_W(SP, G, true, true); else SS2D_CORE_LAUNCH_W(SP, G, false, true); break; } \
+        }                                                                                                                           \
+        if (a.vec_ok) SS2D_CORE_LAUNCH_W(SP, G, true, false); else SS2D_CORE_LAUNCH_W(SP, G, false, false);                         \
     } while (0)
     if (a.softplus) {
         if (g == 8) SS2D_CORE_LAUNCH(true, 8); else if (g == 4) SS2D_CORE_LAUNCH(true, 4); else SS2D_CORE_LAUNCH(true, 1);
     } else {
         if (g == 8) SS2D_CORE_LAUNCH(false, 8); else if (g == 4) SS2D_CORE_LAUNCH(false, 4); else SS2D_CORE_LAUNCH(false, 1);
     }
+#undef SS2D_CORE_LAUNCH_W
 #undef SS2D_CORE_LAUNCH
     return launch_status();
 }
