@@ -159,6 +159,50 @@ def test_scan_channel_per_lane_optional_arguments_and_delta_groups(has_D, has_bi
     assert torch.allclose(got, want, **TOL32)
 
 
+# Shapes that select scan_small_kernel (rows of 49 / 196 positions, one state, 16-bit inputs: one segment of a row per
+# lane, 8 / 4 rows per wavefront).  A single wavefront's worth of rows, whole workgroups, a last workgroup with idle
+# wavefronts, several groups, several images.
+SMALL_GRID = [
+    (1, 4, 1, 1, 196), (3, 8, 2, 1, 196), (1, 12, 3, 1, 196), (2, 40, 2, 1, 196), (1, 64, 4, 1, 196),
+    (1, 8, 1, 1, 49), (2, 16, 2, 1, 49), (3, 24, 1, 1, 49), (1, 72, 3, 1, 49), (2, 128, 4, 1, 49),
+]
+
+
+@pytest.mark.parametrize("batch,dim,G,N,L", SMALL_GRID)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scan_short_row_kernel_matches_oracle(batch, dim, G, N, L, dtype):
+    _announce("scan-small", batch, dim, G, N, L, dtype)
+    args = make_inputs(41, batch, dim, G, N, L, dtype)
+    want = orc.selective_scan(*args, True, out_float=True)
+    got, _ = run_gpu(*args, True, True, want_x=False)
+    assert torch.allclose(got, want, **TOL32), f"max abs err {(got - want).abs().max().item()}"
+    # the same rows with the chunk states requested go through the wavefront-scan kernel: two kernels, one answer
+    got_x, _ = run_gpu(*args, True, True, want_x=True)
+    assert torch.allclose(got_x, want, **TOL32)
+    # SS2D-style constants (A = -1, D = 1, dt bias), output in the input dtype
+    args = make_inputs(42, batch, dim, G, N, L, dtype, ss2d_like=True)
+    want = orc.selective_scan(*args, True, out_float=False)
+    got, _ = run_gpu(*args, True, False, want_x=False)
+    assert got.dtype == dtype and torch.allclose(got.float(), want.float(), **TOL16)
+
+
+@pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False)])
+@pytest.mark.parametrize("L", [49, 196])
+def test_scan_short_row_kernel_optional_arguments_and_views(has_D, has_bias, softplus, L):
+    _announce("scan-small-opt", has_D, has_bias, softplus, L)
+    u, delta, A, B, C, D, bias = make_inputs(43, 2, 32, 2, 1, L, torch.bfloat16)
+    args = (u, delta, A, B, C, D if has_D else None, bias if has_bias else None)
+    want = orc.selective_scan(*args, softplus, out_float=True)
+    got, _ = run_gpu(*args, softplus, True, want_x=False)
+    assert torch.allclose(got, want, **TOL32), f"max abs err {(got - want).abs().max().item()}"
+    # B and C as strided views of one projection tensor (what SS2D.project hands over)
+    proj = torch.randn(2, 2, 5, L, generator=torch.Generator().manual_seed(44)).to(torch.bfloat16)
+    Bv, Cv = proj[:, :, 3:4], proj[:, :, 4:5]
+    want = orc.selective_scan(u, delta, A, Bv.contiguous(), Cv.contiguous(), D, bias, True, out_float=True)
+    got, _ = run_gpu(u, delta, A, Bv, Cv, D, bias, True, True, want_x=False)
+    assert torch.allclose(got, want, **TOL32)
+
+
 @pytest.mark.parametrize("batch,dim,G,N,L", [(2, 8, 4, 1, 3136), (1, 8, 4, 16, 784), (2, 16, 4, 1, 49), (1, 4, 4, 1, 333)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_scan_ss2d_init_recipe(batch, dim, G, N, L, dtype):

@@ -23,6 +23,7 @@ struct ScanArgs {
     int32_t batch, dim, L, N, dim_per_group, dim_per_delta, n_chunks, softplus;
     int64_t u_bs, u_ds, dl_bs, dl_ds, A_ds, A_ns, B_bs, B_gs, B_ns, C_bs, C_gs, C_ns, o_bs, o_ds;
     int32_t rows;
+    int32_t vec_out_ok;                    // scan_small.hip: the output base is 16-byte aligned
     uint32_t B_span_bytes, C_span_bytes;   // extent of B / C reachable through the strides (buffer-descriptor kernels)
 };
 
@@ -42,6 +43,10 @@ struct CoreArgs {
     int64_t B_ks, B_bs, C_ks, C_bs;     // B / C strides over direction and batch (elements)
     uint32_t B_span_bytes, C_span_bytes;
 };
+
+// scan_small.hip: the stand-alone scan for rows of 49 or 196 positions and one state, one segment of a row per lane.
+bool scan_small_eligible(const ScanArgs &a, int in_dtype, const void *u, const void *delta, const void *out);
+int launch_scan_small(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream);
 
 // ss2d_core_small.hip: the row-per-lane kernel for small square maps.
 bool core_small_eligible(const CoreArgs &a, int in_dtype);
@@ -320,5 +325,66 @@ __device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32
     gather_group_raw<T, kGran>(rsrc, elem_offset, uniform_elem_offset, w);
     unpack_group<T, kGran>(w, v);
 }
+
+// ---- short rows: one segment of a row per lane (ss2d_core_small.hip, scan_small.hip) --------------------------------
+// Inclusive scan of (a, h) pairs over the 16-lane DPP row, in lane order or in reverse lane order; returns the
+// EXCLUSIVE h (the state entering this lane; 0 for the first lane of the row).  Lanes without a source keep their value.
+template <bool kReverse>
+__device__ __forceinline__ float row_scan_state_in(float a, float h) {
+    float hx = 0.0f;
+#define SS2D_ROW_STEP(CTRL)                                         \
+    "v_fmac_f32_dpp %1, %1, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t" \
+    "v_mul_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"  \
+    "s_nop 0\n\t"
+    if constexpr (!kReverse) {
+        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shr:1") SS2D_ROW_STEP("row_shr:2") SS2D_ROW_STEP("row_shr:4") SS2D_ROW_STEP("row_shr:8")
+            "s_nop 0\n\t"
+            "v_mov_b32_dpp %2, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0"
+            : "+v"(a), "+v"(h), "+v"(hx));
+    } else {
+        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shl:1") SS2D_ROW_STEP("row_shl:2") SS2D_ROW_STEP("row_shl:4") SS2D_ROW_STEP("row_shl:8")
+            "s_nop 0\n\t"
+            "v_mov_b32_dpp %2, %1 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 0"
+            : "+v"(a), "+v"(h), "+v"(hx));
+    }
+#undef SS2D_ROW_STEP
+    return hx;
+}
+
+// kS consecutive 16-bit elements of an LDS tile, packed two to a register as they sit there; item() widens element j.
+// Even kS: the run starts at an even element offset (4-byte reads).  Odd kS: it may start anywhere -- the dwords that
+// cover it are read and funnel-shifted into place (one more LDS element than the run is touched when it starts at an
+// even offset: tiles keep a few elements of slack behind them).
+template <typename in_t, int kS> struct Run {
+    static constexpr int kWords = (kS + 1) / 2;
+    uint32_t w[kWords];
+    __device__ __forceinline__ void read(const uint16_t *tile, int elem_off) {
+        if constexpr (kS % 2 == 0) {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(tile + elem_off);
+#pragma unroll
+            for (int k = 0; k < kWords; ++k) w[k] = src[k];
+        } else {
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(tile + (elem_off & ~1));
+            const uint32_t shift = (uint32_t)(elem_off & 1) * 16u;
+            uint32_t r[kWords];
+#pragma unroll
+            for (int k = 0; k < kWords; ++k) r[k] = src[k];
+#pragma unroll
+            for (int k = 0; k + 1 < kWords; ++k) w[k] = __builtin_amdgcn_alignbit(r[k + 1], r[k], shift);
+            w[kWords - 1] = r[kWords - 1] >> shift;
+        }
+    }
+    __device__ __forceinline__ void pack(const uint16_t (&e)[kS]) {
+#pragma unroll
+        for (int k = 0; k < kS / 2; ++k) w[k] = (uint32_t)e[2 * k] | ((uint32_t)e[2 * k + 1] << 16);
+        if constexpr (kS % 2 != 0) w[kWords - 1] = e[kS - 1];
+    }
+    __device__ __forceinline__ float item(int j) const {
+        return (j & 1) ? unpack_hi<in_t>(w[j / 2]) : unpack_lo<in_t>(w[j / 2]);
+    }
+};
+constexpr int kRunSlack = 8;     // 16-bit elements kept free behind an LDS array whose last run may be read one element long
 
 }  // namespace ss2d

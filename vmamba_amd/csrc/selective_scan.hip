@@ -571,6 +571,8 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     const int64_t row_slots = ((int64_t)q->seqlen + kPass - 1) / kPass * kPass;
     const bool flat = flat_eligible(a, q) && (!vec || 10 * (int64_t)q->seqlen < 7 * row_slots);
     hipStream_t s = (hipStream_t)stream;
+    // rows of 49 / 196 positions, one state, rows adjacent in memory: one segment of a row per lane
+    if (scan_small_eligible(a, q->in_dtype, q->u, q->delta, q->out)) return launch_scan_small(a, q->in_dtype, q->out_dtype, s);
     // several states per channel and enough channels per group to fill wavefronts: one channel per lane
     if (vec && scan_chan_eligible(a)) return launch_scan_chan(a, q->in_dtype, q->out_dtype, s);
     if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, flat, s);

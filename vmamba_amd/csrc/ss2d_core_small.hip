@@ -25,62 +25,6 @@
 
 namespace ss2d {
 
-// Inclusive scan of (a, h) pairs over the 16-lane DPP row, in lane order or in reverse lane order; returns the
-// EXCLUSIVE h (the state entering this lane; 0 for the first lane of the row).  Lanes without a source keep their value.
-template <bool kReverse>
-__device__ __forceinline__ float row_scan_state_in(float a, float h) {
-    float hx = 0.0f;
-#define SS2D_ROW_STEP(CTRL)                                         \
-    "v_fmac_f32_dpp %1, %1, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t" \
-    "v_mul_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"  \
-    "s_nop 0\n\t"
-    if constexpr (!kReverse) {
-        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shr:1") SS2D_ROW_STEP("row_shr:2") SS2D_ROW_STEP("row_shr:4") SS2D_ROW_STEP("row_shr:8")
-            "s_nop 0\n\t"
-            "v_mov_b32_dpp %2, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
-            "s_nop 0"
-            : "+v"(a), "+v"(h), "+v"(hx));
-    } else {
-        asm("s_nop 1\n\t" SS2D_ROW_STEP("row_shl:1") SS2D_ROW_STEP("row_shl:2") SS2D_ROW_STEP("row_shl:4") SS2D_ROW_STEP("row_shl:8")
-            "s_nop 0\n\t"
-            "v_mov_b32_dpp %2, %1 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
-            "s_nop 0"
-            : "+v"(a), "+v"(h), "+v"(hx));
-    }
-#undef SS2D_ROW_STEP
-    return hx;
-}
-
-// kS consecutive 16-bit elements of an LDS tile as they sit there: dwords of two elements for even kS (element offsets
-// are even then: 4-byte reads), one element per register for odd kS.  item() widens element j.
-template <typename in_t, int kS> struct Run {
-    static constexpr bool kPacked = kS % 2 == 0;
-    uint32_t w[kPacked ? kS / 2 : kS];
-    __device__ __forceinline__ void read(const uint16_t *tile, int elem_off) {
-        if constexpr (kPacked) {
-            const uint32_t *src = reinterpret_cast<const uint32_t *>(tile + elem_off);
-#pragma unroll
-            for (int k = 0; k < kS / 2; ++k) w[k] = src[k];
-        } else {
-#pragma unroll
-            for (int j = 0; j < kS; ++j) w[j] = tile[elem_off + j];
-        }
-    }
-    __device__ __forceinline__ void pack(const uint16_t (&e)[kS]) {
-        if constexpr (kPacked) {
-#pragma unroll
-            for (int k = 0; k < kS / 2; ++k) w[k] = (uint32_t)e[2 * k] | ((uint32_t)e[2 * k + 1] << 16);
-        } else {
-#pragma unroll
-            for (int j = 0; j < kS; ++j) w[j] = e[j];
-        }
-    }
-    __device__ __forceinline__ float item(int j) const {
-        if constexpr (kPacked) return (j & 1) ? unpack_hi<in_t>(w[j / 2]) : unpack_lo<in_t>(w[j / 2]);
-        else return to_f32(in_t{(uint16_t)w[j]});
-    }
-};
-
 constexpr int kSmallChans = kWavesPerWg;     // channels per workgroup: one per wavefront, all on the same images
 
 // Registers are capped so that as many workgroups share a CU as its LDS tiles allow (4 for 14 x 14, 5-6 for 7 x 7).
@@ -100,8 +44,8 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
     //   shared by the four wavefronts (same images): the B and C tiles of the four directions   [dir][B|C][tile]
     //   per wavefront (its channel): the four delta tiles, in the order of use 1, 3, 0, 2; once directions 1 and 3 are
     //   done, the room of their two tiles holds the fp32 tile of the (y1 + y3) sums for the column -> row transposition
-    __shared__ __align__(16) uint16_t s_bc[8 * kTileElems];
-    __shared__ __align__(16) uint16_t s_dl[kWavesPerWg * 4 * kTileElems];
+    __shared__ __align__(16) uint16_t s_bc[8 * kTileElems + kRunSlack];
+    __shared__ __align__(16) uint16_t s_dl[kWavesPerWg * 4 * kTileElems + kRunSlack];
     static_assert(2 * kTileElems * sizeof(uint16_t) == kTileElems * sizeof(float), "the fp32 tile fits two delta tiles");
 
     const int lane = threadIdx.x & (kWave - 1);
