@@ -111,7 +111,11 @@ def test_layer_norm_rows_without_affine_and_known_answers():
 
 # B, C, H, W
 CF = [(2, 96, 56, 56), (2, 48, 5, 7), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (1, 1000, 3, 3), (2, 7, 9, 4), (1, 96, 1, 1),
-      (1, 1300, 3, 5), (1, 97, 8, 9), (2, 200, 3, 70), (1, 500, 6, 6), (2, 768, 6, 6), (3, 40, 2, 2), (1, 136, 4, 9)]
+      (1, 1300, 3, 5), (1, 97, 8, 9), (2, 200, 3, 70), (1, 500, 6, 6), (2, 768, 6, 6), (3, 40, 2, 2), (1, 136, 4, 9),
+      # short images, one workgroup per image or per share of one: odd maps (rows that are not 16-byte aligned), a last
+      # lane group that holds fewer channels, maps of two and of one position, shares of unequal size
+      (3, 40, 5, 5), (2, 24, 3, 3), (2, 16, 1, 2), (2, 100, 4, 4), (5, 104, 13, 4), (2, 8, 1, 1), (3, 72, 31, 1), (2, 20, 3, 3),
+      (2, 384, 10, 10), (1, 192, 31, 33)]
 
 
 @pytest.mark.parametrize("B,C,H,W", CF)
@@ -128,6 +132,21 @@ def test_layer_norm_channel_first(B, C, H, W, in_dt, w_dt, out_dt, out_cl):
     got = layer_norm_cf_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_channel_last=out_cl, out_dtype=out_dt).cpu()
     assert got.dtype == want.dtype and got.shape == want.shape
     assert torch.allclose(got.float(), want.float(), **_tol(out_dt))
+
+
+@pytest.mark.parametrize("B,C,H,W", [(128, 192, 28, 28), (128, 384, 14, 14), (128, 768, 7, 7), (64, 384, 14, 14), (300, 768, 7, 7)])
+def test_layer_norm_channel_first_benchmark_batches(B, C, H, W):
+    """The out_norm shapes of the 224 x 224 model at the benchmark's batch (the split of an image over workgroups
+    depends on the batch): fp32 scan output in, bf16 channel-last rows out, every image against the oracle."""
+    print("CASE ln-cf-batch", B, C, H, W, flush=True)
+    g = torch.Generator().manual_seed(44)
+    x = torch.randn(B, C, H, W, generator=g) * 1.5 + 0.2
+    w, b = (torch.randn(C, generator=g) + 1).bfloat16(), torch.randn(C, generator=g).bfloat16()
+    want = torch_ref.layer_norm_cf(x, w, b, 1e-5, True, torch.bfloat16)
+    got = layer_norm_cf_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_channel_last=True, out_dtype=torch.bfloat16).cpu()
+    assert got.shape == want.shape and torch.allclose(got.float(), want.float(), **_tol(torch.bfloat16))
+    got_cf = layer_norm_cf_hip(_dev(x), _dev(w), _dev(b), 1e-5, out_channel_last=False, out_dtype=torch.bfloat16).cpu()
+    assert torch.equal(got_cf.permute(0, 2, 3, 1), got)
 
 
 def test_modules_share_state_dict_with_torch():

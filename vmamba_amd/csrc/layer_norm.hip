@@ -430,6 +430,199 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
     }
 }
 
+// Image variant for fp32 channel-first input of SHORT images (7 x 7 ... 28 x 28 maps): the tile kernels above cut an
+// image into pieces of 16 or 32 positions, i.e. 64- or 128-byte runs per channel row, and on short rows that is what
+// they are bound by.  Here a workgroup of up to 1024 threads takes a whole image, or a 1/T share of its positions, and
+// reads it as 16-byte vectors of ONE flat stream:
+//   * kCh = 1 (L a multiple of 4): a unit is one channel row, Q = L/4 vectors; the workgroup takes Qn consecutive
+//     vectors of every row;
+//   * kCh = 4 (any other L, C a multiple of 4): a unit is four consecutive channel rows = L vectors that start on a
+//     16-byte boundary although the rows do not; element j of vector q is (channel e / L, position e % L), e = 4q+j.
+// Thread (q, g) holds vector q of units g*kU .. g*kU+kU-1; which (channel offset, position) its four elements are
+// does not depend on the unit, so a lane adds its units up in registers, the partial sums of the groups meet in LDS
+// (in a fixed order: results do not depend on timing), and mean and 1/std come back per position.  Variance from
+// centred values, as everywhere in this file.  Channel-first output leaves as it came; channel-last output is turned
+// round through an LDS tile [position][channel] whose pitch is an odd number of dwords.
+constexpr int kLnImgBlock = 1024;
+constexpr int kLnImgStat = 256;                      // positions per workgroup at most
+
+template <typename w_t, typename out_t, bool kOutChannelLast, int kCh, int kU>
+__global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const float *__restrict__ x, const w_t *__restrict__ weight,
+                                                                          const w_t *__restrict__ bias, out_t *__restrict__ y, int C,
+                                                                          int L, int T, int Qn, int G, int pitch_dw, float eps) {
+    static_assert(kCh == 1 || kCh == 4, "a unit is one channel row or four");
+    static_assert(kU % 2 == 0, "channel pairs share a dword of the output tile");
+    extern __shared__ __align__(16) unsigned char lni_smem[];
+    float *red = reinterpret_cast<float *>(lni_smem);                          // [thread][4]
+    float *stat = red + 4 * kLnImgBlock;                                       // [2][kLnImgStat]
+    float *wb = stat + 2 * kLnImgStat;                                         // [2][C] weight, bias
+    uint32_t *tile = reinterpret_cast<uint32_t *>(wb + 2 * C);                 // [position][pitch_dw]
+    const int Q = kCh * L / 4, n_units = C / kCh;
+    const int b = blockIdx.x / T, q0 = ((int)blockIdx.x - b * T) * Qn;
+    const int Qt = min(Qn, Q - q0);
+    const int t = threadIdx.x, g = t / Qn, q = t - g * Qn;
+    const bool lane_on = g < G && q < Qt;
+    const int Lt = kCh == 1 ? 4 * Qt : L;                                      // positions of this workgroup
+    int lj[4], cc[4];                                                          // element j: position (tile-relative), channel offset
+    if constexpr (kCh == 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { lj[j] = 4 * q + j; cc[j] = 0; }
+    } else {
+        const int e0 = min(4 * q, kCh * L - 4);                                // idle lanes: any vector of the unit
+        cc[0] = e0 / L; lj[0] = e0 - cc[0] * L;
+#pragma unroll
+        for (int j = 1; j < 4; ++j) {
+            const bool wrap = lj[j - 1] + 1 == L;
+            lj[j] = wrap ? 0 : lj[j - 1] + 1;
+            cc[j] = wrap ? cc[j - 1] + 1 : cc[j - 1];
+        }
+    }
+    const int n_valid = lane_on ? min(max(n_units - g * kU, 0), kU) : 0;       // units this lane really holds
+    const float *xb = x + (size_t)b * C * L;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(xb), 0, C * L * 4, 0x00020000);
+
+    float v[kU][4];
+    float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int n = 0; n < kU; ++n) {
+        const int unit = g * kU + n;
+        // idle lanes and units past the last point past the end of the buffer, where the hardware returns 0
+        const uint32_t off = n < n_valid ? (uint32_t)(unit * Q + q0 + q) * 16u : 0x7ffffff0u;
+        const auto r = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { v[n][j] = bits_to_f32(r[j]); s[j] += v[n][j]; }
+    }
+    // weight and bias wait in LDS (read after the barriers of the two reductions)
+    for (int c = t; c < C; c += (int)blockDim.x) {
+        wb[c] = weight ? to_f32(weight[c]) : 1.0f;
+        wb[C + c] = bias ? to_f32(bias[c]) : 0.0f;
+    }
+    // per-position totals over groups (and, kCh = 4, over the four channel offsets), always in the same order
+    auto totals = [&](const float (&acc)[4], int which, auto finish) {
+        *reinterpret_cast<float4 *>(red + 4 * t) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (t < Lt) {
+            float tot = 0.0f;
+#pragma unroll 4
+            for (int gg = 0; gg < G; ++gg)
+#pragma unroll
+                for (int c = 0; c < kCh; ++c) tot += red[gg * Qn * 4 + c * L + t];
+            stat[which * kLnImgStat + t] = finish(tot);
+        }
+        __syncthreads();
+    };
+    const float inv_c = 1.0f / (float)C;
+    totals(s, 0, [&](float tot) { return tot * inv_c; });
+    float mean[4], qq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mean[j] = stat[lj[j]];
+#pragma unroll
+    for (int n = 0; n < kU; ++n) {
+        if (n < n_valid) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float d = v[n][j] - mean[j];
+                qq[j] = fmaf(d, d, qq[j]);
+            }
+        }
+    }
+    totals(qq, 1, [&](float tot) { return rsqrtf(tot * inv_c + eps); });
+    float rstd[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rstd[j] = stat[kLnImgStat + lj[j]];
+
+    // normalised values, in place.  A unit's weight and bias are one value (kCh = 1) or four, of which a lane's
+    // four consecutive elements meet at most two neighbours.
+    const int cc_lo = cc[0], cc_hi = min(cc[0] + 1, kCh - 1);
+#pragma unroll
+    for (int n = 0; n < kU; ++n) {
+        const int unit = min(g * kU + n, n_units - 1);
+        const float w_lo = wb[unit * kCh + cc_lo], b_lo = wb[C + unit * kCh + cc_lo];
+        float w_hi = w_lo, b_hi = b_lo;
+        if constexpr (kCh > 1) {
+            w_hi = wb[unit * kCh + cc_hi];
+            b_hi = wb[C + unit * kCh + cc_hi];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float wv = cc[j] == cc_lo ? w_lo : w_hi, bv = cc[j] == cc_lo ? b_lo : b_hi;
+            v[n][j] = fmaf((v[n][j] - mean[j]) * rstd[j], wv, bv);
+        }
+    }
+
+    if constexpr (!kOutChannelLast) {
+        out_t *yb = y + (size_t)b * C * L;
+#pragma unroll
+        for (int n = 0; n < kU; ++n) {
+            const int unit = g * kU + n;
+            if (n < n_valid) {
+                out_t *dst = yb + ((size_t)unit * Q + q0 + q) * 4;
+                if constexpr (sizeof(out_t) == 4) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v[n][0], v[n][1], v[n][2], v[n][3]);
+                } else {
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(pack2_from_f32<out_t>(v[n][0], v[n][1]), pack2_from_f32<out_t>(v[n][2], v[n][3]));
+                }
+            }
+        }
+    } else {
+        // element j of unit n sits at row lj[j], column (g * kU + n) * kCh + cc[j]: per-lane bases, constant steps
+        if constexpr (sizeof(out_t) == 4) {
+            int base[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) base[j] = lj[j] * pitch_dw + g * kU * kCh + cc[j];
+#pragma unroll
+            for (int n = 0; n < kU; ++n) {
+                if (n < n_valid) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) tile[base[j] + n * kCh] = __builtin_bit_cast(uint32_t, v[n][j]);
+                }
+            }
+        } else if constexpr (kCh == 1) {
+            // a lane's channels are consecutive and start on an even one: pairs go out as dwords (C is even,
+            // host-checked: a pair is inside or outside)
+            int base[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) base[j] = lj[j] * pitch_dw + g * (kU / 2);
+#pragma unroll
+            for (int n = 0; n < kU; n += 2) {
+                if (n < n_valid) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) tile[base[j] + n / 2] = pack2_from_f32<out_t>(v[n][j], v[n + 1][j]);
+                }
+            }
+        } else {
+            uint16_t *tile16 = reinterpret_cast<uint16_t *>(tile);
+            int base[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) base[j] = lj[j] * pitch_dw * 2 + g * kU * kCh + cc[j];
+#pragma unroll
+            for (int n = 0; n < kU; n += 2) {
+                if (n < n_valid) {                     // the units of a lane come in pairs (C / 4 even: host-checked)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t two = pack2_from_f32<out_t>(v[n][j], v[n + 1][j]);
+                        tile16[base[j] + n * kCh] = (uint16_t)(two & 0xffffu);
+                        tile16[base[j] + (n + 1) * kCh] = (uint16_t)(two >> 16);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // rows of C channels, 16 bytes per lane (C * sizeof(out_t) is a multiple of 16: host-checked)
+        const int pieces = C * (int)sizeof(out_t) / 16;
+        const int l0 = kCh == 1 ? 4 * q0 : 0;
+        uint4 *yb = reinterpret_cast<uint4 *>(y + ((size_t)b * L + l0) * C);
+        int r = t / pieces, pc = t - r * pieces;
+        const int step_r = (int)blockDim.x / pieces, step_p = (int)blockDim.x - step_r * pieces;
+        while (r < Lt) {
+            const uint32_t *src = tile + r * pitch_dw + pc * 4;
+            yb[(size_t)r * pieces + pc] = make_uint4(src[0], src[1], src[2], src[3]);
+            r += step_r; pc += step_p;
+            if (pc >= pieces) { pc -= pieces; ++r; }
+        }
+    }
+}
+
 // ---- host side ----------------------------------------------------------------------------------
 static bool ln_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -531,10 +724,74 @@ static int launch_ln_cf_quad(const void *x, const void *w, const void *b, void *
     return launch_status();
 }
 
+// The image variant's split of an image and its launch; false when the shape is not one it covers.
+struct LnImagePlan { int kch, ku, T, Qn, G, threads, pitch_dw; size_t smem; };
+static bool ln_image_plan(int B, int C, int L, size_t out_size, bool out_channel_last, LnImagePlan &p) {
+    if (L > 1024 || (int64_t)C * L * 4 >= 0x7ffffff0ll) return false;
+    p.kch = L % 4 == 0 ? 1 : 4;
+    if (C % (2 * p.kch) != 0) return false;                     // a lane's channels (kCh = 1) or units (kCh = 4) come in pairs
+    if (out_channel_last && (C * out_size) % 16 != 0) return false;
+    const int Q = p.kch * L / 4, n_units = C / p.kch;
+    p.pitch_dw = (int)(out_size == 4 ? C : C / 2) | 1;
+    if (p.kch == 4 && L < 2) return false;                     // four elements of a vector would meet more than two channels
+    // The fewest workgroups per image that fit (threads, LDS), then finer splits: down to runs of 384 bytes per
+    // channel row in any case (smaller tiles let two workgroups share a CU and overlap their phases), and down to
+    // 192 bytes while there are fewer workgroups than CUs.
+    const int t_max = p.kch == 1 ? Q : 1;
+    bool found = false;
+    for (int T = 1; T <= t_max; ++T) {
+        const int Qn = (Q + T - 1) / T;
+        if ((Qn - 1) * T >= Q) continue;                       // an empty last share: the split of a smaller T
+        if (found && (Qn < 12 || (Qn < 24 && (int64_t)B * p.T >= 256))) break;
+        const int positions = p.kch == 1 ? 4 * Qn : L;
+        if (positions > kLnImgStat) continue;
+        const size_t smem = (size_t)4 * kLnImgBlock * 4 + 2 * kLnImgStat * 4 + (size_t)2 * C * 4 +
+                            (out_channel_last ? (size_t)positions * p.pitch_dw * 4 : 0);
+        if (smem > 100 * 1024) continue;
+        for (int ku : {8, 10}) {
+            const int G = (n_units + ku - 1) / ku;
+            if ((int64_t)G * Qn > kLnImgBlock) continue;
+            p.ku = ku; p.T = T; p.Qn = Qn; p.G = G; p.threads = ((G * Qn + kWave - 1) / kWave) * kWave; p.smem = smem;
+            found = true;
+            break;
+        }
+    }
+    return found;
+}
+
+template <typename w_t, typename out_t>
+static int launch_ln_cf_image(const LnImagePlan &p, const void *x, const void *w, const void *b, void *y, int B, int C, int L,
+                              float eps, int out_channel_last, hipStream_t stream) {
+    const int64_t n_wg = (int64_t)B * p.T;
+    if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+#define SS2D_LN_IMAGE(CL, KCH, KU)                                                                                              \
+    {                                                                                                                            \
+        auto kern = layer_norm_cf_image_kernel<w_t, out_t, CL, KCH, KU>;                                                         \
+        if (p.smem > 64 * 1024 &&                                                                                                \
+            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.smem) != hipSuccess) \
+            return SS2D_ELAUNCH;                                                                                                 \
+        hipLaunchKernelGGL(kern, dim3((uint32_t)n_wg), dim3(p.threads), p.smem, stream, (const float *)x, (const w_t *)w,        \
+                           (const w_t *)b, (out_t *)y, C, L, p.T, p.Qn, p.G, p.pitch_dw, eps);                                   \
+    }
+    if (out_channel_last) {
+        if (p.kch == 1) { if (p.ku == 8) SS2D_LN_IMAGE(true, 1, 8) else SS2D_LN_IMAGE(true, 1, 10) }
+        else { if (p.ku == 8) SS2D_LN_IMAGE(true, 4, 8) else SS2D_LN_IMAGE(true, 4, 10) }
+    } else {
+        if (p.kch == 1) { if (p.ku == 8) SS2D_LN_IMAGE(false, 1, 8) else SS2D_LN_IMAGE(false, 1, 10) }
+        else { if (p.ku == 8) SS2D_LN_IMAGE(false, 4, 8) else SS2D_LN_IMAGE(false, 4, 10) }
+    }
+#undef SS2D_LN_IMAGE
+    return launch_status();
+}
+
 template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
                         int out_channel_last, hipStream_t stream) {
     if constexpr (sizeof(in_t) == 4) {
+        // short images: a whole image, or an even share of one, per workgroup
+        LnImagePlan plan;
+        if (L <= 1024 && ln_aligned16(x) && ln_aligned16(y) && ln_image_plan(B, C, L, sizeof(out_t), out_channel_last != 0, plan))
+            return launch_ln_cf_image<w_t, out_t>(plan, x, w, b, y, B, C, L, eps, out_channel_last, stream);
         // fp32 input, quads of positions: 16-byte loads (and 16-byte channel-last stores)
         const bool quad_ok = L % 4 == 0 && ln_aligned16(x) && (int64_t)C * L * 4 < 0x7ffffff0ll && (int64_t)B * ((L + 15) / 16) <= 0x7fffffff &&
                              (out_channel_last ? (C % (16 / (int)sizeof(out_t)) == 0 && ln_aligned16(y)) : ln_aligned16(y));
