@@ -140,7 +140,8 @@ template <typename T, bool kSilu>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restrict__ x, const T *__restrict__ weight,
                                                                 const T *__restrict__ bias, T *__restrict__ y, int D,
                                                                 int H, int W, int TH, int row_tiles, int ch_tiles,
-                                                                int out_pitch, FastDiv divW, FastDiv divWp) {
+                                                                int out_pitch, int flat_out, FastDiv divW, FastDiv divWp,
+                                                                FastDiv divL) {
     extern __shared__ __align__(16) uint16_t dw_smem[];
     const int Wp = W + 2;
     uint16_t *in_tile = dw_smem;                                 // [TH + 2][W + 2][32]
@@ -154,6 +155,23 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     const int c_base = (int)ct * kDwCh;
     const int cv = threadIdx.x % 4;
     const int c0 = c_base + cv * 8;                              // this lane's 8 channels, in every phase
+
+    // The 72 weights of the 8 channels (9 consecutive 16-byte vectors) and the bias: requested first, so that their
+    // latency passes under the tile's loads.
+    const int cw = min(c0, D - 8);                               // keep the loads in range; lanes with c0 >= D store nothing
+    uint32_t wraw[36];
+    {
+        const uint16_t *wsrc = reinterpret_cast<const uint16_t *>(weight + (size_t)cw * 9);
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            const uint4 v = reinterpret_cast<const uint4 *>(wsrc)[k];
+            wraw[4 * k] = v.x; wraw[4 * k + 1] = v.y; wraw[4 * k + 2] = v.z; wraw[4 * k + 3] = v.w;
+        }
+    }
+    float bv[8];
+#pragma unroll
+    for (int ci = 0; ci < 8; ++ci) bv[ci] = 0.0f;
+    if (bias) unpack8<T>(*reinterpret_cast<const uint4 *>(bias + cw), bv);
 
     // ---- input rows h0-1 .. h0+rows into LDS; outside the image (and channels >= D) zeros.  The image sits behind a
     // buffer descriptor and pieces outside it are pointed past its end, where the hardware returns 0: the loads
@@ -185,19 +203,10 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             if (e < n_in) *reinterpret_cast<uint4 *>(in_tile + (size_t)e * kDwCh + cv * 8) = v[u];
         }
     }
-    // The 72 weights of the 8 channels (9 consecutive 16-byte vectors), regrouped for the dot instruction: per channel
-    // four dwords holding taps (0,1) (2,3) (4,5) (6,7) and one holding (tap 8, zero).
+    // The weights regrouped for the dot instruction: per channel four dwords holding taps (0,1) (2,3) (4,5) (6,7) and
+    // one holding (tap 8, zero).
     uint32_t wp2[8][5];
-    float bv[8];
     {
-        const int cw = min(c0, D - 8);                           // keep the loads in range; lanes with c0 >= D store nothing
-        const uint16_t *wsrc = reinterpret_cast<const uint16_t *>(weight + (size_t)cw * 9);
-        uint32_t wraw[36];
-#pragma unroll
-        for (int k = 0; k < 9; ++k) {
-            const uint4 v = reinterpret_cast<const uint4 *>(wsrc)[k];
-            wraw[4 * k] = v.x; wraw[4 * k + 1] = v.y; wraw[4 * k + 2] = v.z; wraw[4 * k + 3] = v.w;
-        }
         // element e = ci * 9 + t sits in half (e & 1) of dword e / 2: a pair of taps starting at an even element IS a
         // dword of the weights as loaded, one starting at an odd element straddles two (one funnel shift)
         auto pair_at = [&](int e) -> uint32_t {
@@ -210,9 +219,6 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             const int e8 = ci * 9 + 8;
             wp2[ci][4] = (e8 & 1) ? (wraw[e8 / 2] >> 16) : (wraw[e8 / 2] & 0xffffu);
         }
-#pragma unroll
-        for (int ci = 0; ci < 8; ++ci) bv[ci] = 0.0f;
-        if (bias) unpack8<T>(*reinterpret_cast<const uint4 *>(bias + cw), bv);
     }
     __syncthreads();
 
@@ -267,6 +273,26 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
 
     // ---- write back: the tile's positions are contiguous per channel in (B, D, H, W)
     const int L = H * W;
+    if (flat_out) {
+        // A whole image per workgroup: its 32 channel rows are ONE contiguous block of y that starts on a 16-byte
+        // boundary whatever L is (32 * L elements).  16 bytes per lane over the block; a piece may run from one
+        // channel row into the next, so its elements are picked out of the tile one by one.
+        uint4 *dst = reinterpret_cast<uint4 *>(y + ((size_t)b * D + c_base) * L);
+        for (int pc = threadIdx.x; pc < kDwCh * L / 8; pc += kBlock) {
+            uint32_t c, pos;
+            divmod((uint32_t)pc * 8u, divL, c, pos);
+            uint32_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int col = (int)pos + 16 * (int)(c / 8);
+                col = col >= out_pitch ? col - out_pitch : col;
+                e[i] = out_tile[c * out_pitch + col];
+                if (++pos == (uint32_t)L) { pos = 0; ++c; }
+            }
+            dst[pc] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+        }
+        return;
+    }
     const int pieces = (n_out + 7) / 8;
     const bool vec = ((h0 * W) % 8 == 0) && (L % 8 == 0);
     // a group of 8, 16 or 32 lanes per channel (the smallest that covers the tile), a lane per piece of 8 positions: no
@@ -339,15 +365,19 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             const size_t smem = ((size_t)(TH + 2) * (W + 2) * kDwCh + (size_t)kDwCh * out_pitch) * sizeof(uint16_t);
             const int row_tiles = (H + TH - 1) / TH, ch_tiles = (D + kDwCh - 1) / kDwCh;
             const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
+            // whole images whose rows do not take 16-byte stores: the tile leaves as one flat block
+            const int flat_out = row_tiles == 1 && D % kDwCh == 0 && L % 8 != 0;
             if (smem <= 64 * 1024 && n_wg <= 0x7fffffff && (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
                 if (apply_silu) {
                     hipLaunchKernelGGL((dwconv3x3_rows_kernel<T, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream,
                                        (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles,
-                                       out_pitch, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)));
+                                       out_pitch, flat_out, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)),
+                                       make_fastdiv((uint32_t)L));
                 } else {
                     hipLaunchKernelGGL((dwconv3x3_rows_kernel<T, false>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream,
                                        (const T *)x, (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles,
-                                       out_pitch, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)));
+                                       out_pitch, flat_out, make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)(W + 2)),
+                                       make_fastdiv((uint32_t)L));
                 }
                 return launch_status();
             }
