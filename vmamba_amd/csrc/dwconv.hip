@@ -155,6 +155,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     const int c_base = (int)ct * kDwCh;
     const int cv = threadIdx.x % 4;
     const int c0 = c_base + cv * 8;                              // this lane's 8 channels, in every phase
+    const int rot = flat_out ? 0 : 16;                           // rotation of the output tile's rows per channel group
 
     // The 72 weights of the 8 channels (9 consecutive 16-byte vectors) and the bias: requested first, so that their
     // latency passes under the tile's loads.
@@ -203,9 +204,10 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             if (e < n_in) *reinterpret_cast<uint4 *>(in_tile + (size_t)e * kDwCh + cv * 8) = v[u];
         }
     }
-    // The weights regrouped for the dot instruction: per channel four dwords holding taps (0,1) (2,3) (4,5) (6,7) and
-    // one holding (tap 8, zero).
-    uint32_t wp2[8][5];
+    // The weights regrouped for the dot instruction: per channel four dwords holding taps (0,1) (2,3) (4,5) (6,7);
+    // tap 8 as fp32.
+    uint32_t wp2[8][4];
+    float w8[8];
     {
         // element e = ci * 9 + t sits in half (e & 1) of dword e / 2: a pair of taps starting at an even element IS a
         // dword of the weights as loaded, one starting at an odd element straddles two (one funnel shift)
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
 #pragma unroll
             for (int tp = 0; tp < 4; ++tp) wp2[ci][tp] = pair_at(ci * 9 + 2 * tp);
             const int e8 = ci * 9 + 8;
-            wp2[ci][4] = (e8 & 1) ? (wraw[e8 / 2] >> 16) : (wraw[e8 / 2] & 0xffffu);
+            w8[ci] = (e8 & 1) ? unpack_hi<T>(wraw[e8 / 2]) : unpack_lo<T>(wraw[e8 / 2]);
         }
     }
     __syncthreads();
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
         // Column of this position in the rows of the output tile: the rows of channel group cv are rotated by 16 * cv
         // elements, so that the four groups of a wavefront write into different banks (their rows start a multiple
         // of 32 banks apart).
-        int col = pidx + 16 * cv;
+        int col = pidx + rot * cv;
         col = col >= out_pitch ? col - out_pitch : col;
         // nine taps as four pairs and a single: the two taps of a pair are brought side by side per channel (one byte
         // permute per channel pair and tap pair) and multiplied-accumulated by one dot instruction per channel
@@ -240,9 +242,16 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw)
                 tap[kh * 3 + kw] = *reinterpret_cast<const uint4 *>(in_tile + ((size_t)(ph + kh) * Wp + pw + kw) * kDwCh + cv * 8);
+        // tap 8 is single: one fused multiply-add on the widened value starts each accumulator from the bias
         float acc[8];
+        {
+            const uint32_t a[4] = {tap[8].x, tap[8].y, tap[8].z, tap[8].w};
 #pragma unroll
-        for (int ci = 0; ci < 8; ++ci) acc[ci] = bv[ci];
+            for (int cp = 0; cp < 4; ++cp) {
+                acc[2 * cp] = fmaf(unpack_lo<T>(a[cp]), w8[2 * cp], bv[2 * cp]);
+                acc[2 * cp + 1] = fmaf(unpack_hi<T>(a[cp]), w8[2 * cp + 1], bv[2 * cp + 1]);
+            }
+        }
 #pragma unroll
         for (int tp = 0; tp < 4; ++tp) {
             const uint32_t a[4] = {tap[2 * tp].x, tap[2 * tp].y, tap[2 * tp].z, tap[2 * tp].w};
@@ -251,14 +260,6 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
             for (int cp = 0; cp < 4; ++cp) {
                 acc[2 * cp] = dot2_acc(T{}, pair_lo(a[cp], b[cp]), wp2[2 * cp][tp], acc[2 * cp]);
                 acc[2 * cp + 1] = dot2_acc(T{}, pair_hi(a[cp], b[cp]), wp2[2 * cp + 1][tp], acc[2 * cp + 1]);
-            }
-        }
-        {
-            const uint32_t a[4] = {tap[8].x, tap[8].y, tap[8].z, tap[8].w};
-#pragma unroll
-            for (int cp = 0; cp < 4; ++cp) {
-                acc[2 * cp] = dot2_acc(T{}, a[cp] & 0xffffu, wp2[2 * cp][4], acc[2 * cp]);
-                acc[2 * cp + 1] = dot2_acc(T{}, a[cp] >> 16, wp2[2 * cp + 1][4], acc[2 * cp + 1]);
             }
         }
 #pragma unroll
@@ -281,14 +282,12 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
         for (int pc = threadIdx.x; pc < kDwCh * L / 8; pc += kBlock) {
             uint32_t c, pos;
             divmod((uint32_t)pc * 8u, divL, c, pos);
+            // L >= 8 (host-checked): at most one row boundary inside a piece
+            const int n_first = min(8, L - (int)pos);
+            const uint16_t *row0 = out_tile + c * out_pitch + pos, *row1 = out_tile + (c + 1) * out_pitch - n_first;
             uint32_t e[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                int col = (int)pos + 16 * (int)(c / 8);
-                col = col >= out_pitch ? col - out_pitch : col;
-                e[i] = out_tile[c * out_pitch + col];
-                if (++pos == (uint32_t)L) { pos = 0; ++c; }
-            }
+            for (int i = 0; i < 8; ++i) e[i] = (i < n_first ? row0 : row1)[i];
             dst[pc] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
         }
         return;
@@ -361,12 +360,15 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             // TH rows per workgroup: about 224 positions, LDS within 64 KiB
             int TH = 224 / W;
             TH = TH < 1 ? 1 : (TH > H ? H : TH);
-            const int out_pitch = ((TH * W + 15) / 16) * 16;          // a multiple of 16 elements: rows rotate by 16, 32, 48
-            const size_t smem = ((size_t)(TH + 2) * (W + 2) * kDwCh + (size_t)kDwCh * out_pitch) * sizeof(uint16_t);
+            int out_pitch = ((TH * W + 15) / 16) * 16;                // a multiple of 16 elements: rows rotate by 16, 32, 48
             const int row_tiles = (H + TH - 1) / TH, ch_tiles = (D + kDwCh - 1) / kDwCh;
             const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
             // whole images whose rows do not take 16-byte stores: the tile leaves as one flat block
-            const int flat_out = row_tiles == 1 && D % kDwCh == 0 && L % 8 != 0;
+            const int flat_out = row_tiles == 1 && D % kDwCh == 0 && L % 8 != 0 && L >= 8;
+            // (its output tile is read element by element, so the rows need no 16-byte alignment: a pitch of 2 mod 16
+            // elements puts the rows of the four channel groups of a wavefront 8 banks apart without any rotation)
+            if (flat_out) out_pitch = (int)((L + 13) / 16) * 16 + 2;
+            const size_t smem = ((size_t)(TH + 2) * (W + 2) * kDwCh + (size_t)kDwCh * out_pitch) * sizeof(uint16_t);
             if (smem <= 64 * 1024 && n_wg <= 0x7fffffff && (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
                 if (apply_silu) {
                     hipLaunchKernelGGL((dwconv3x3_rows_kernel<T, true>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream,
