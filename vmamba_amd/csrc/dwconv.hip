@@ -317,6 +317,174 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
     }
 }
 
+// Plane variant of the channel-last kernel: the layout change happens on the way INTO LDS instead of on the way out.
+// A workgroup owns TH full rows x kCh channels (32 or 64, i.e. runs of 64 or 128 bytes per position).  The input rows
+// (with halo) are fetched as 16-byte channel vectors, two neighbouring positions per lane, and written into one LDS plane
+// per channel as dwords holding TWO NEIGHBOURING POSITIONS of that channel (one byte permute per channel and pair):
+// a plane is the zero-padded image rows of one channel, [TH + 2][pitch], padded column 0 = image column -1.
+// In the compute phase a lane owns one channel and segments of 8 consecutive outputs of a row.  With the taps of a
+// row in dwords D_i = (p[8s + 2i], p[8s + 2i + 1]) an output needs two dot instructions per filter row and no data
+// movement at all:
+//   even output 2i:  (p[2i], p[2i+1]) . (k0, k1) + (p[2i+2], p[2i+3]) . (k2, 0)  = D_i . P0 + D_i+1 . P1
+//   odd output 2i+1: (p[2i], p[2i+1]) . (0, k0)  + (p[2i+2], p[2i+3]) . (k1, k2) = D_i . P2 + D_i+1 . P3
+// (v_dot2c_f32_bf16 / v_dot2_f32_f16, fp32 accumulation), against nine instructions per output and channel pair for
+// taps that sit in different dwords.  A lane's 8 outputs are 16 contiguous bytes of the channel-first result: they
+// are stored straight from registers (W a multiple of 4), or -- whole images whose rows are not 8-byte aligned --
+// parked in LDS as the 64 * L (32 * L) contiguous elements they are in memory and stored 16 bytes per lane.
+constexpr int kDwpMaxIt = 8;         // segments per lane at most
+
+template <typename T, bool kSilu, int kCh>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__restrict__ x, const T *__restrict__ weight,
+                                                                  const T *__restrict__ bias, T *__restrict__ y, int D, int H,
+                                                                  int W, int TH, int row_tiles, int ch_tiles, int pitch,
+                                                                  int plane_dw, int nseg, int n_it, int flat_out,
+                                                                  FastDiv divHalf, FastDiv divNseg) {
+    constexpr int kLpc = kBlock / kCh;                           // lanes per channel in the compute phase
+    constexpr int kCv = kCh / 8;                                 // 16-byte channel vectors per position
+    constexpr int kPer = kBlock / kCv;                           // position pairs per staging pass
+    constexpr int kInFlight = 3;                                 // pairs (two loads each) a lane requests together
+    extern __shared__ __align__(16) uint32_t dwp_smem[];         // [kCh][plane_dw]
+    uint32_t wg = blockIdx.x;
+    const uint32_t ct = wg % ch_tiles; wg /= ch_tiles;
+    const uint32_t rt = wg % row_tiles;
+    const uint32_t b = wg / row_tiles;
+    const int h0 = (int)rt * TH;
+    const int rows = min(TH, H - h0);
+    const int c_base = (int)ct * kCh;
+    const int L = H * W, half = pitch / 2;
+
+    // compute-phase identity: channel and segment slot; its nine weights and bias, requested first
+    const int cl = threadIdx.x / kLpc, slot = threadIdx.x % kLpc;
+    const int c = c_base + cl;
+    uint32_t wr[9];
+    {
+        const uint16_t *wsrc = reinterpret_cast<const uint16_t *>(weight + (size_t)c * 9);
+#pragma unroll
+        for (int k = 0; k < 9; ++k) wr[k] = wsrc[k];
+    }
+    const float bv = bias ? to_f32(bias[c]) : 0.0f;
+
+    // ---- staging: rows h0-1 .. h0+rows of kCh channels into the planes, zeros outside the image
+    {
+        const int cv = threadIdx.x % kCv;
+        const int c0 = c_base + cv * 8;
+        const T *xb = x + (size_t)b * H * W * D;
+        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xb), 0, H * W * D * 2, 0x00020000);
+        const int n_items = (rows + 2) * half;
+        uint32_t *plane0 = dwp_smem + (cv * 8) * plane_dw;
+        for (int q0 = threadIdx.x / kCv; q0 < n_items; q0 += kInFlight * kPer) {
+            uint4 va[kInFlight], vb[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const int q = q0 + u * kPer;
+                uint32_t rr, pp;
+                divmod((uint32_t)q, divHalf, rr, pp);
+                const int h = h0 - 1 + (int)rr, w0 = 2 * (int)pp - 1, w1 = 2 * (int)pp;
+                const bool row_ok = q < n_items && h >= 0 && h < H;
+                const uint32_t off_a = (row_ok && w0 >= 0 && w0 < W) ? (uint32_t)((h * W + w0) * D + c0) * 2u : 0x7ffffff0u;
+                const uint32_t off_b = (row_ok && w1 < W) ? (uint32_t)((h * W + w1) * D + c0) * 2u : 0x7ffffff0u;
+                const auto ta = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off_a, 0, 0);
+                const auto tb = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off_b, 0, 0);
+                va[u] = make_uint4(ta[0], ta[1], ta[2], ta[3]);
+                vb[u] = make_uint4(tb[0], tb[1], tb[2], tb[3]);
+            }
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const int q = q0 + u * kPer;
+                if (q < n_items) {
+                    const uint32_t a[4] = {va[u].x, va[u].y, va[u].z, va[u].w}, bb[4] = {vb[u].x, vb[u].y, vb[u].z, vb[u].w};
+                    uint32_t *dst = plane0 + q;                  // rr * half + pp = q
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        dst[(2 * i) * plane_dw] = pair_lo(a[i], bb[i]);
+                        dst[(2 * i + 1) * plane_dw] = pair_hi(a[i], bb[i]);
+                    }
+                }
+            }
+        }
+    }
+    // weight pairs per filter row
+    uint32_t P0[3], P1[3], P2[3], P3[3];
+#pragma unroll
+    for (int kr = 0; kr < 3; ++kr) {
+        P0[kr] = wr[3 * kr] | (wr[3 * kr + 1] << 16);
+        P1[kr] = wr[3 * kr + 2];
+        P2[kr] = wr[3 * kr] << 16;
+        P3[kr] = wr[3 * kr + 1] | (wr[3 * kr + 2] << 16);
+    }
+    __syncthreads();
+
+    const uint32_t *plane = dwp_smem + cl * plane_dw;
+    const int n_seg = rows * nseg;
+    T *yc = y + ((size_t)b * D + c) * L + (size_t)h0 * W;
+    uint32_t keep[kDwpMaxIt][4];
+#pragma unroll
+    for (int it = 0; it < kDwpMaxIt; ++it) {
+        if (it < n_it) {                                          // uniform
+            const int sg = slot + kLpc * it;
+            uint32_t r, seg;
+            divmod((uint32_t)min(sg, n_seg - 1), divNseg, r, seg);
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = bv;
+#pragma unroll
+            for (int kr = 0; kr < 3; ++kr) {
+                const uint32_t *row = plane + (r + kr) * half + seg * 4;
+                const uint2 d01 = *reinterpret_cast<const uint2 *>(row), d23 = *reinterpret_cast<const uint2 *>(row + 2);
+                const uint32_t d[5] = {d01.x, d01.y, d23.x, d23.y, row[4]};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[2 * i] = dot2_acc(T{}, d[i], P0[kr], acc[2 * i]);
+                    acc[2 * i] = dot2_acc(T{}, d[i + 1], P1[kr], acc[2 * i]);
+                    acc[2 * i + 1] = dot2_acc(T{}, d[i], P2[kr], acc[2 * i + 1]);
+                    acc[2 * i + 1] = dot2_acc(T{}, d[i + 1], P3[kr], acc[2 * i + 1]);
+                }
+            }
+            uint32_t o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                o[i] = pack2_from_f32<T>(acc[2 * i], acc[2 * i + 1]);                                   // conv output as stored
+                if (kSilu) o[i] = pack2_from_f32<T>(silu_fast(unpack_lo<T>(o[i])), silu_fast(unpack_hi<T>(o[i])));
+            }
+            if (flat_out) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) keep[it][i] = o[i];
+            } else if (sg < n_seg) {
+                T *dst = yc + r * W + seg * 8;
+                if (W % 8 == 0) {
+                    *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
+                } else {                                          // W % 4 == 0: 8-byte rows, a last segment of 4
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(o[0], o[1]);
+                    if ((int)seg * 8 + 8 <= W) *reinterpret_cast<uint2 *>(dst + 4) = make_uint2(o[2], o[3]);
+                }
+            }
+        }
+    }
+    if (!flat_out) return;
+
+    // ---- whole image: the results of the kCh channels are one contiguous block of y; park them in LDS as they lie in
+    // memory (the planes are no longer needed) and store 16 bytes per lane
+    __syncthreads();
+    uint16_t *flat = reinterpret_cast<uint16_t *>(dwp_smem);      // [kCh][L]
+#pragma unroll
+    for (int it = 0; it < kDwpMaxIt; ++it) {
+        const int sg = slot + kLpc * it;
+        if (it < n_it && sg < n_seg) {
+            uint32_t r, seg;
+            divmod((uint32_t)sg, divNseg, r, seg);
+            uint16_t *dst = flat + cl * L + r * W + seg * 8;
+            const int nv = min(8, W - (int)seg * 8);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (j < nv) dst[j] = (uint16_t)((j & 1) ? keep[it][j / 2] >> 16 : keep[it][j / 2] & 0xffffu);
+        }
+    }
+    __syncthreads();
+    uint4 *dst = reinterpret_cast<uint4 *>(y + ((size_t)b * D + c_base) * L);
+    const uint4 *src = reinterpret_cast<const uint4 *>(flat);
+    for (int pc = threadIdx.x; pc < kCh * L / 8; pc += kBlock) dst[pc] = src[pc];
+}
+
 // Generic variant: any element type, either input layout, one output element per lane (lanes along W).
 template <typename T, bool kInChannelLast, bool kSilu>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_generic_kernel(const T *__restrict__ x, const T *__restrict__ weight,
@@ -356,6 +524,30 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
     const int64_t L = (int64_t)H * W;
     auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     if constexpr (sizeof(T) == 2) {
+        // plane variant: channel tiles of 64 (or 32), full rows, outputs that leave as whole 8- or 16-byte pieces
+        if (in_channel_last && D % 32 == 0 && W <= 120 && al16(x) && al16(y) && (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
+            const int kch = D % 64 == 0 ? 64 : 32, lpc = kBlock / kch;
+            const int nseg = (W + 7) / 8, pitch = 8 * nseg + 4;
+            int TH = (7 * lpc) / nseg;
+            TH = TH > H ? H : TH;
+            const int row_tiles = TH >= 1 ? (H + TH - 1) / TH : 0, ch_tiles = D / kch;
+            const int flat_out = W % 4 != 0;
+            const int n_it = TH >= 1 ? (TH * nseg + lpc - 1) / lpc : 0;
+            int plane_dw = (TH + 2) * pitch / 2;
+            plane_dw += (2 - plane_dw % 8 + 8) % 8;                // = 2 mod 8 dwords: the planes of a lane's 8 channels 16 banks apart
+            const size_t smem = (size_t)kch * plane_dw * 4;
+            const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
+            if (TH >= 1 && n_it <= kDwpMaxIt && (!flat_out || row_tiles == 1) && smem <= 64 * 1024 && n_wg <= 0x7fffffff) {
+#define SS2D_DW_PLANES(SILU, KCH)                                                                                              \
+    hipLaunchKernelGGL((dwconv3x3_planes_kernel<T, SILU, KCH>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x,  \
+                       (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles, pitch, plane_dw, nseg, n_it,     \
+                       flat_out, make_fastdiv((uint32_t)(pitch / 2)), make_fastdiv((uint32_t)nseg))
+                if (kch == 64) { if (apply_silu) SS2D_DW_PLANES(true, 64); else SS2D_DW_PLANES(false, 64); }
+                else { if (apply_silu) SS2D_DW_PLANES(true, 32); else SS2D_DW_PLANES(false, 32); }
+#undef SS2D_DW_PLANES
+                return launch_status();
+            }
+        }
         if (in_channel_last && D % 8 == 0 && W <= kDwMaxW && al16(x) && al16(w) && al16(y) && (!bias || al16(bias))) {
             // TH rows per workgroup: about 224 positions, LDS within 64 KiB
             int TH = 224 / W;
