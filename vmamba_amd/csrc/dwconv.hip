@@ -332,6 +332,10 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_rows_kernel(const T *__restr
 // are stored straight from registers (W a multiple of 4), or -- whole images whose rows are not 8-byte aligned --
 // parked in LDS as the 64 * L (32 * L) contiguous elements they are in memory and stored 16 bytes per lane.
 constexpr int kDwpMaxIt = 8;         // segments per lane at most
+// Dword offset of channel plane c: planes are plane_dw apart, moved up by one where that leaves them on an even dword
+// (the 8-byte reads of the compute phase).  plane_dw = 2 mod 8 for 32-channel tiles, 1 mod 8 for 64-channel tiles:
+// the 4 (8) channel vectors that a wavefront writes together then land 16 (8) banks apart.
+__device__ __forceinline__ int plane_at(int c, int plane_dw) { const int o = c * plane_dw; return o + (o & 1); }
 
 template <typename T, bool kSilu, int kCh>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__restrict__ x, const T *__restrict__ weight,
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
         const T *xb = x + (size_t)b * H * W * D;
         const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xb), 0, H * W * D * 2, 0x00020000);
         const int n_items = (rows + 2) * half;
-        uint32_t *plane0 = dwp_smem + (cv * 8) * plane_dw;
+        uint32_t *plane0 = dwp_smem;
         for (int q0 = threadIdx.x / kCv; q0 < n_items; q0 += kInFlight * kPer) {
             uint4 va[kInFlight], vb[kInFlight];
 #pragma unroll
@@ -396,8 +400,8 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
                     uint32_t *dst = plane0 + q;                  // rr * half + pp = q
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        dst[(2 * i) * plane_dw] = pair_lo(a[i], bb[i]);
-                        dst[(2 * i + 1) * plane_dw] = pair_hi(a[i], bb[i]);
+                        dst[plane_at(cv * 8 + 2 * i, plane_dw)] = pair_lo(a[i], bb[i]);
+                        dst[plane_at(cv * 8 + 2 * i + 1, plane_dw)] = pair_hi(a[i], bb[i]);
                     }
                 }
             }
@@ -414,7 +418,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
     }
     __syncthreads();
 
-    const uint32_t *plane = dwp_smem + cl * plane_dw;
+    const uint32_t *plane = dwp_smem + plane_at(cl, plane_dw);
     const int n_seg = rows * nseg;
     T *yc = y + ((size_t)b * D + c) * L + (size_t)h0 * W;
     uint32_t keep[kDwpMaxIt][4];
@@ -474,9 +478,15 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
             divmod((uint32_t)sg, divNseg, r, seg);
             uint16_t *dst = flat + cl * L + r * W + seg * 8;
             const int nv = min(8, W - (int)seg * 8);
+            if (W % 2 == 0) {                                     // every offset and count is even: whole dwords
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (j < nv) dst[j] = (uint16_t)((j & 1) ? keep[it][j / 2] >> 16 : keep[it][j / 2] & 0xffffu);
+                for (int i = 0; i < 4; ++i)
+                    if (2 * i < nv) reinterpret_cast<uint32_t *>(dst)[i] = keep[it][i];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j < nv) dst[j] = (uint16_t)((j & 1) ? keep[it][j / 2] >> 16 : keep[it][j / 2] & 0xffffu);
+            }
         }
     }
     __syncthreads();
@@ -534,8 +544,10 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             const int flat_out = W % 4 != 0;
             const int n_it = TH >= 1 ? (TH * nseg + lpc - 1) / lpc : 0;
             int plane_dw = (TH + 2) * pitch / 2;
-            plane_dw += (2 - plane_dw % 8 + 8) % 8;                // = 2 mod 8 dwords: the planes of a lane's 8 channels 16 banks apart
-            const size_t smem = (size_t)kch * plane_dw * 4;
+            const int want = kch == 64 ? 1 : 2;                    // see plane_at
+            plane_dw += 1;                                         // room for the parity shift
+            plane_dw += (want - plane_dw % 8 + 8) % 8;
+            const size_t smem = ((size_t)kch * plane_dw + 2) * 4;
             const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
             if (TH >= 1 && n_it <= kDwpMaxIt && (!flat_out || row_tiles == 1) && smem <= 64 * 1024 && n_wg <= 0x7fffffff) {
 #define SS2D_DW_PLANES(SILU, KCH)                                                                                              \
