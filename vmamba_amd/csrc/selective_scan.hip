@@ -360,15 +360,34 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
     const int L = p.L;
 
     const int n_chunks = (L + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
+    // the next chunk's u / delta (and B / C of the first state) are requested before this chunk's arithmetic and its
+    // barriers: a wavefront always has a chunk of loads in flight (positions past the row's end come back as the fill)
+    const int pos_first = wave * kPass + lane * kItems;
+    Raw8<in_t> u_nx = load_raw<in_t, kVec>(u_row, pos_first, L);
+    Raw8<in_t> dl_nx = load_raw<in_t, kVec>(dl_row, pos_first, L, delta_fill<kSoftplus>());
+    Raw8<in_t> B_nx = load_raw<in_t, kVec>(B_row, pos_first, L), C_nx = load_raw<in_t, kVec>(C_row, pos_first, L);
     for (int chunk = 0; chunk < n_chunks; ++chunk) {
         const int par = chunk & 1;
-        const int pos = chunk * SS2D_SCAN_CHUNK + wave * kPass + lane * kItems;
+        const int pos = chunk * SS2D_SCAN_CHUNK + pos_first;
+        const Raw8<in_t> u_raw = u_nx, dl_raw = dl_nx, B_raw = B_nx, C_raw = C_nx;
+        if (chunk + 1 < n_chunks) {
+            const int pos_nx = pos + SS2D_SCAN_CHUNK;
+            u_nx = load_raw<in_t, kVec>(u_row, pos_nx, L);
+            dl_nx = load_raw<in_t, kVec>(dl_row, pos_nx, L, delta_fill<kSoftplus>());
+            B_nx = load_raw<in_t, kVec>(B_row, pos_nx, L);
+            C_nx = load_raw<in_t, kVec>(C_row, pos_nx, L);
+        }
         float dl[kItems], du[kItems], y[kItems];
-        load_delta_u<in_t, kVec, kSoftplus>(u_row, dl_row, pos, L, bias, Dv, dl, du, y);
+        prepare_delta_u<in_t, kSoftplus>(u_raw, dl_raw, L - pos, bias, Dv, dl, du, y);
         for (int n = 0; n < N; ++n) {
             float Bv[kItems], Cv[kItems];
-            load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
-            load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+            if (n == 0) {
+                unpack_raw<in_t>(B_raw, Bv);
+                unpack_raw<in_t>(C_raw, Cv);
+            } else {
+                load_items<in_t, kVec>(B_row + n * p.B_ns, pos, L, Bv);
+                load_items<in_t, kVec>(C_row + n * p.C_ns, pos, L, Cv);
+            }
             const float A_log2e = A_row[n * p.A_ns] * kLog2e;
             float ac[kItems], hh[kItems];
 #pragma unroll
