@@ -149,6 +149,27 @@ def test_layer_norm_channel_first_benchmark_batches(B, C, H, W):
     assert torch.equal(got_cf.permute(0, 2, 3, 1), got)
 
 
+@pytest.mark.parametrize("B,C,H,W", [(3, 384, 14, 14), (2, 768, 7, 7), (2, 96, 56, 56), (2, 40, 5, 5)])
+@pytest.mark.parametrize("out_cl", [False, True])
+def test_layer_norm_channel_first_without_affine_and_views(B, C, H, W, out_cl):
+    """No weight / no bias on every channel-first kernel, zero-size batches, and a non-contiguous input (made
+    contiguous by the wrapper): per-position mean 0 and variance 1 besides the oracle."""
+    g = torch.Generator().manual_seed(45)
+    x = torch.randn(B, C, H, W, generator=g) * 3 + 1
+    got = layer_norm_cf_hip(_dev(x), None, None, 1e-5, out_channel_last=out_cl).cpu()
+    want = torch_ref.layer_norm_cf(x, None, None, 1e-5, out_cl, torch.float32)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-4)
+    axis = -1 if out_cl else 1
+    assert torch.allclose(got.mean(axis), torch.zeros(()), atol=1e-5) and torch.allclose(got.var(axis, unbiased=False), torch.ones(()), atol=1e-3)
+    w = torch.randn(C, generator=g)
+    only_w = layer_norm_cf_hip(_dev(x), _dev(w), None, 1e-5, out_channel_last=out_cl).cpu()
+    assert torch.allclose(only_w, torch_ref.layer_norm_cf(x, w, None, 1e-5, out_cl, torch.float32), rtol=1e-4, atol=1e-4)
+    xt = x.transpose(2, 3)                                   # a view: (B, C, W, H), not contiguous
+    got_t = layer_norm_cf_hip(_dev(xt), None, None, 1e-5, out_channel_last=out_cl).cpu()
+    assert torch.allclose(got_t, torch_ref.layer_norm_cf(xt.contiguous(), None, None, 1e-5, out_cl, torch.float32), rtol=1e-4, atol=1e-4)
+    assert layer_norm_cf_hip(_dev(x[:0]), None, None, out_channel_last=out_cl).numel() == 0
+
+
 def test_modules_share_state_dict_with_torch():
     ln, ref = LayerNorm(24).to(DEV), torch.nn.LayerNorm(24)
     ref.weight.data.normal_(); ref.bias.data.normal_()
