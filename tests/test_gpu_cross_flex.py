@@ -83,6 +83,17 @@ def test_staged_mixed_layout_scan_equals_the_route_kernel(x_cl, obo, scans):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("B,R,S", [(2, 96, 3136), (3, 64, 64), (1, 72, 200), (2, 8, 8), (1, 136, 24), (2, 96, 49), (1, 5, 7), (2, 100, 36)])
+@pytest.mark.parametrize("dtype", [torch.int16, torch.int32, torch.int8, torch.int64])
+def test_transpose_bcl_is_a_transpose(B, R, S, dtype):
+    """(B, R, S) -> (B, S, R): extents that take the 16-byte kernel (multiples of a vector, with short last tiles) and
+    extents that take the element-wise one, every element size, bit for bit against torch."""
+    from vmamba_amd.csm import transpose_bcl_hip
+    info = torch.iinfo(dtype)
+    x = torch.randint(max(info.min, -2 ** 31), min(info.max, 2 ** 31 - 1), (B, R, S), dtype=dtype, device=DEV)
+    assert torch.equal(transpose_bcl_hip(x), x.transpose(1, 2).contiguous())
+
+
 def test_cross_merge_flex_left_to_right_order():
     y = torch.randn(2, 7, 5, 4, 6, generator=torch.Generator().manual_seed(1)).bfloat16()
     want = torch_ref.cross_merge_flex(y, False, False, False, 0, left_to_right=True)

@@ -287,6 +287,56 @@ __global__ __launch_bounds__(kBlock) void transpose_bcl_kernel(const U *__restri
     }
 }
 
+// The same for 2- and 4-byte elements when both extents are multiples of a 16-byte vector and the tensors are 16-byte
+// aligned: 16-byte loads along S, 16-byte stores along R, the turn made by reading the LDS tile down its columns one
+// element at a time (the element-wise kernel above moves 128 bytes per wavefront instruction and is bound by their
+// number).  Row pitch: an odd number of dwords, so that the 8 (16) row groups of a column read fall into different banks.
+template <typename U>
+__global__ __launch_bounds__(kBlock) void transpose_bcl_vec_kernel(const U *__restrict__ src, U *__restrict__ dst, int R, int S,
+                                                                   int r_tiles, int s_tiles) {
+    constexpr int kT = 64, kVec = 16 / (int)sizeof(U), kPpr = kT / kVec;   // pieces per tile row
+    constexpr int kPitchDw = sizeof(U) == 2 ? 33 : 65;                      // dwords per tile row
+    __shared__ uint32_t tile[kT * kPitchDw];
+    uint32_t wg = blockIdx.x;
+    const uint32_t st = wg % s_tiles; wg /= s_tiles;
+    const uint32_t rt = wg % r_tiles;
+    const uint32_t b = wg / r_tiles;
+    const int r0 = (int)rt * kT, s0 = (int)st * kT;
+    const U *sb = src + (size_t)b * R * S;
+    U *db = dst + (size_t)b * R * S;
+#pragma unroll
+    for (int p = threadIdx.x; p < kT * kPpr; p += kBlock) {
+        const int i = p / kPpr, pc = p % kPpr;
+        const int r = r0 + i, sp = s0 + pc * kVec;
+        if (r < R && sp < S) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(sb + (size_t)r * S + sp);
+            uint32_t *row = tile + i * kPitchDw + pc * 4;
+            row[0] = v.x; row[1] = v.y; row[2] = v.z; row[3] = v.w;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = threadIdx.x; p < kT * kPpr; p += kBlock) {
+        const int si = p / kPpr, rp = p % kPpr;
+        const int sp = s0 + si, r = r0 + rp * kVec;
+        if (sp < S && r < R) {
+            uint32_t w[4];
+            if constexpr (sizeof(U) == 2) {
+                const uint16_t *t16 = reinterpret_cast<const uint16_t *>(tile);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t lo = t16[(rp * 8 + 2 * k) * (2 * kPitchDw) + si], hi = t16[(rp * 8 + 2 * k + 1) * (2 * kPitchDw) + si];
+                    w[k] = lo | (hi << 16);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) w[k] = tile[(rp * 4 + k) * kPitchDw + si];
+            }
+            *reinterpret_cast<uint4 *>(db + (size_t)sp * R + r) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
 }  // namespace ss2d
 
 extern "C" int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, int elem_bytes, void *stream) {
@@ -299,6 +349,13 @@ extern "C" int ss2d_transpose_bcl(const void *x, void *y, int B, int R, int S, i
     const int64_t n_wg = (int64_t)B * r_tiles * s_tiles;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     hipStream_t s = (hipStream_t)stream;
+    const int vec = 16 / elem_bytes;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+    if ((elem_bytes == 2 || elem_bytes == 4) && R % vec == 0 && S % vec == 0 && aligned) {
+        if (elem_bytes == 2) hipLaunchKernelGGL((transpose_bcl_vec_kernel<uint16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint16_t *)x, (uint16_t *)y, R, S, r_tiles, s_tiles);
+        else hipLaunchKernelGGL((transpose_bcl_vec_kernel<uint32_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint32_t *)x, (uint32_t *)y, R, S, r_tiles, s_tiles);
+        return launch_status();
+    }
     switch (elem_bytes) {
         case 1: hipLaunchKernelGGL((transpose_bcl_kernel<uint8_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint8_t *)x, (uint8_t *)y, R, S, r_tiles, s_tiles); break;
         case 2: hipLaunchKernelGGL((transpose_bcl_kernel<uint16_t>), dim3((uint32_t)n_wg), dim3(kBlock), 0, s, (const uint16_t *)x, (uint16_t *)y, R, S, r_tiles, s_tiles); break;
