@@ -100,8 +100,25 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
     const int64_t block1 = block0 + p.blocks_per_wave < p.n_blocks ? block0 + p.blocks_per_wave : p.n_blocks;
     for (int64_t blk = block0; blk < block1; ++blk) {
         const int64_t n0 = blk * kDtBlock;
-        // ---- x rows of the block -> LDS: kPieces lanes x 16 bytes per row
-        for (int idx = lane; idx < p.R * kPieces; idx += kWave) {
+        // ---- x rows of the block -> LDS: kPieces lanes x 16 bytes per row.  With 16-byte loads all of a lane's pieces
+        // (one per 8 rows) are requested before the first is parked: one memory latency per block, not one per piece
+        if (p.vec_ok) {
+            uint4 v[kSteps];
+#pragma unroll
+            for (int it = 0; it < kSteps; ++it) {
+                const int idx = lane + kWave * it, r = idx / kPieces, c = idx % kPieces;
+                const int64_t n = n0 + 8 * c;
+                const uint32_t off = (r < p.R && n < p.N) ? (uint32_t)(r * p.x_rs + n) * 2u : kDtOutOfRange;
+                const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+                v[it] = make_uint4(t[0], t[1], t[2], t[3]);
+            }
+#pragma unroll
+            for (int it = 0; it < kSteps; ++it) {
+                const int idx = lane + kWave * it, r = idx / kPieces, c = idx % kPieces;
+                if (r < p.R) *reinterpret_cast<uint4 *>(xs + r * kDtPitch + 8 * c) = v[it];
+            }
+        }
+        for (int idx = lane; idx < (p.vec_ok ? 0 : p.R * kPieces); idx += kWave) {
             const int r = idx / kPieces, c = idx % kPieces;
             const int64_t n = n0 + 8 * c;
             uint4 v;
