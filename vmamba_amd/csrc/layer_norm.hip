@@ -47,6 +47,29 @@ template <typename T> __device__ __forceinline__ void ln_store8(T *p, const floa
     }
 }
 
+// Eight elements as loaded (one 16-byte piece for 16-bit types, two for fp32), widened when they are used.
+template <typename T> struct LnRaw { uint4 a, b; };
+template <typename T> __device__ __forceinline__ LnRaw<T> ln_load_raw(const T *p) {
+    LnRaw<T> r;
+    r.a = *reinterpret_cast<const uint4 *>(p);
+    if constexpr (sizeof(T) == 4) r.b = *reinterpret_cast<const uint4 *>(p + 4);
+    else r.b = r.a;
+    return r;
+}
+template <typename T> __device__ __forceinline__ void ln_widen(const LnRaw<T> &r, float (&v)[kLnItems]) {
+    if constexpr (sizeof(T) == 2) {
+        const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = to_f32(T{(uint16_t)(w[i] & 0xffffu)});
+            v[2 * i + 1] = to_f32(T{(uint16_t)(w[i] >> 16)});
+        }
+    } else {
+        v[0] = bits_to_f32(r.a.x); v[1] = bits_to_f32(r.a.y); v[2] = bits_to_f32(r.a.z); v[3] = bits_to_f32(r.a.w);
+        v[4] = bits_to_f32(r.b.x); v[5] = bits_to_f32(r.b.y); v[6] = bits_to_f32(r.b.z); v[7] = bits_to_f32(r.b.w);
+    }
+}
+
 template <int kGroup> __device__ __forceinline__ float group_sum(float v) {
 #pragma unroll
     for (int off = kGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kGroup);
@@ -67,62 +90,77 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__r
     const int g = threadIdx.x % kGroup;
     const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kGroup;
     const bool row_ok = row < rows;
-    const in_t *xr = x + (row_ok ? row : 0) * C;
-    float v[kChunks][kLnItems];
-    float pb[kChunks][kLnItems];
+    const int64_t row_c = row_ok ? row : rows - 1;   // lanes without a row or a chunk load real memory and drop it
+    // Everything the row needs is requested before anything is used (raw 16-byte pieces, widened later): one memory
+    // latency per workgroup instead of one per chunk and operand.
+    LnRaw<in_t> x_raw[kChunks], r_raw[kChunks];
+    LnRaw<w_t> pb_raw[kChunks], w_raw[kChunks], b_raw[kChunks];
     bool have[kChunks];
-    float s = 0.0f;
-    if (pre_bias) {                                  // requested ahead of the row so that the two loads overlap
-#pragma unroll
-        for (int j = 0; j < kChunks; ++j) {
-            const int c0 = (j * kGroup + g) * kLnItems;
-            if (c0 < C) ln_load8<w_t>(pre_bias + c0, pb[j]);
-        }
-    }
+    int c0c[kChunks];
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
         const int c0 = (j * kGroup + g) * kLnItems;
         have[j] = row_ok && c0 < C;
-        if (have[j]) {
-            ln_load8<in_t>(xr + c0, v[j]);
-            if (residual) {
-                // the row is x + residual, rounded to the tensor type as the separate add would leave it
-                float r[kLnItems];
-                ln_load8<in_t>(residual + row * C + c0, r);
+        c0c[j] = c0 < C ? c0 : C - kLnItems;
+        x_raw[j] = ln_load_raw<in_t>(x + row_c * C + c0c[j]);
+    }
+    if (residual) {
 #pragma unroll
-                for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + r[i]));
-                ln_store8<in_t>(sum_out + row * C + c0, v[j]);
-            }
-            if (pre_bias) {
-                // the row is x + pre_bias (one value per channel), rounded as the separate add would leave it
+        for (int j = 0; j < kChunks; ++j) r_raw[j] = ln_load_raw<in_t>(residual + row_c * C + c0c[j]);
+    }
+    if (pre_bias) {
 #pragma unroll
-                for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + pb[j][i]));
-            }
-        } else {
+        for (int j = 0; j < kChunks; ++j) pb_raw[j] = ln_load_raw<w_t>(pre_bias + c0c[j]);
+    }
+    if (weight) {
 #pragma unroll
-            for (int i = 0; i < kLnItems; ++i) v[j][i] = 0.0f;
+        for (int j = 0; j < kChunks; ++j) w_raw[j] = ln_load_raw<w_t>(weight + c0c[j]);
+    }
+    if (bias) {
+#pragma unroll
+        for (int j = 0; j < kChunks; ++j) b_raw[j] = ln_load_raw<w_t>(bias + c0c[j]);
+    }
+
+    float v[kChunks][kLnItems];
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+        ln_widen<in_t>(x_raw[j], v[j]);
+        if (residual) {
+            // the row is x + residual, rounded to the tensor type as the separate add would leave it
+            float r[kLnItems];
+            ln_widen<in_t>(r_raw[j], r);
+#pragma unroll
+            for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + r[i]));
+            if (have[j]) ln_store8<in_t>(sum_out + row * C + c0c[j], v[j]);
+        }
+        if (pre_bias) {
+            // the row is x + pre_bias (one value per channel), rounded as the separate add would leave it
+            float pb[kLnItems];
+            ln_widen<w_t>(pb_raw[j], pb);
+#pragma unroll
+            for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + pb[i]));
         }
 #pragma unroll
-        for (int i = 0; i < kLnItems; ++i) s += v[j][i];
+        for (int i = 0; i < kLnItems; ++i) { v[j][i] = have[j] ? v[j][i] : 0.0f; s += v[j][i]; }
     }
     const float inv_c = 1.0f / (float)C;
     const float mean = group_sum<kGroup>(s) * inv_c;
     float q = 0.0f;
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
-        if (have[j]) {
 #pragma unroll
-            for (int i = 0; i < kLnItems; ++i) { const float d = v[j][i] - mean; q = fmaf(d, d, q); }
+        for (int i = 0; i < kLnItems; ++i) {
+            const float d = v[j][i] - mean;
+            q = have[j] ? fmaf(d, d, q) : q;
         }
     }
     const float rstd = rsqrtf(group_sum<kGroup>(q) * inv_c + eps);
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
-        if (!have[j]) continue;
-        const int c0 = (j * kGroup + g) * kLnItems;
         float wv[kLnItems], bv[kLnItems], o[kLnItems];
-        if (weight) ln_load8<w_t>(weight + c0, wv);
-        if (bias) ln_load8<w_t>(bias + c0, bv);
+        if (weight) ln_widen<w_t>(w_raw[j], wv);
+        if (bias) ln_widen<w_t>(b_raw[j], bv);
 #pragma unroll
         for (int i = 0; i < kLnItems; ++i) {
             float t = (v[j][i] - mean) * rstd;
@@ -130,7 +168,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__r
             if (bias) t += bv[i];
             o[i] = t;
         }
-        ln_store8<out_t>(y + row * C + c0, o);
+        if (have[j]) ln_store8<out_t>(y + row * C + c0c[j], o);
     }
 }
 
