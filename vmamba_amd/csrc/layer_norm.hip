@@ -38,8 +38,7 @@ template <typename T> __device__ __forceinline__ void ln_store8(T *p, const floa
     if constexpr (sizeof(T) == 2) {
         uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = (uint32_t)from_f32<T>(v[2 * i]).bits | ((uint32_t)from_f32<T>(v[2 * i + 1]).bits << 16);
+        for (int i = 0; i < 4; ++i) w[i] = pack2_from_f32<T>(v[2 * i], v[2 * i + 1]);   // one conversion per pair
         *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
     } else {
         *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -67,6 +66,21 @@ template <typename T> __device__ __forceinline__ void ln_widen(const LnRaw<T> &r
     } else {
         v[0] = bits_to_f32(r.a.x); v[1] = bits_to_f32(r.a.y); v[2] = bits_to_f32(r.a.z); v[3] = bits_to_f32(r.a.w);
         v[4] = bits_to_f32(r.b.x); v[5] = bits_to_f32(r.b.y); v[6] = bits_to_f32(r.b.z); v[7] = bits_to_f32(r.b.w);
+    }
+}
+
+// v[i] = (v[i] + r[i]) rounded to T and widened again -- what a separate add in the tensor's type would leave
+template <typename T> __device__ __forceinline__ void ln_add_rounded(float (&v)[kLnItems], const float (&r)[kLnItems]) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < kLnItems; i += 2) {
+            const uint32_t two = pack2_from_f32<T>(v[i] + r[i], v[i + 1] + r[i + 1]);
+            v[i] = unpack_lo<T>(two);
+            v[i + 1] = unpack_hi<T>(two);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kLnItems; ++i) v[i] = v[i] + r[i];
     }
 }
 
@@ -130,16 +144,14 @@ __global__ __launch_bounds__(kBlock) void layer_norm_rows_kernel(const in_t *__r
             // the row is x + residual, rounded to the tensor type as the separate add would leave it
             float r[kLnItems];
             ln_widen<in_t>(r_raw[j], r);
-#pragma unroll
-            for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + r[i]));
+            ln_add_rounded<in_t>(v[j], r);
             if (have[j]) ln_store8<in_t>(sum_out + row * C + c0c[j], v[j]);
         }
         if (pre_bias) {
             // the row is x + pre_bias (one value per channel), rounded as the separate add would leave it
             float pb[kLnItems];
             ln_widen<w_t>(pb_raw[j], pb);
-#pragma unroll
-            for (int i = 0; i < kLnItems; ++i) v[j][i] = to_f32(from_f32<in_t>(v[j][i] + pb[i]));
+            ln_add_rounded<in_t>(v[j], pb);
         }
 #pragma unroll
         for (int i = 0; i < kLnItems; ++i) { v[j][i] = have[j] ? v[j][i] : 0.0f; s += v[j][i]; }
@@ -433,15 +445,14 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
             const int c = g + i * kG;
             if (valid && c < C) {
                 const float wv = weight ? to_f32(weight[c]) : 1.0f, bv = bias ? to_f32(bias[c]) : 0.0f;
-                out_t o[4];
+                float o[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = from_f32<out_t>(fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv));
+                for (int j = 0; j < 4; ++j) o[j] = fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv);
                 out_t *dst = yb + (size_t)c * L;
                 if constexpr (sizeof(out_t) == 4) {
                     *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
                 } else {
-                    *reinterpret_cast<uint2 *>(dst) = make_uint2((uint32_t)o[0].bits | ((uint32_t)o[1].bits << 16),
-                                                                 (uint32_t)o[2].bits | ((uint32_t)o[3].bits << 16));
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(pack2_from_f32<out_t>(o[0], o[1]), pack2_from_f32<out_t>(o[2], o[3]));
                 }
             }
         }
@@ -452,8 +463,21 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
             const int c = g + i * kG;
             if (c < C) {
                 const float wv = weight ? to_f32(weight[c]) : 1.0f, bv = bias ? to_f32(bias[c]) : 0.0f;
+                float o[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) ot[(4 * q + j) * Cp + c] = from_f32<out_t>(fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv));
+                for (int j = 0; j < 4; ++j) o[j] = fmaf((v[i][j] - mean[j]) * rstd[j], wv, bv);
+                if constexpr (sizeof(out_t) == 4) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ot[(4 * q + j) * Cp + c] = o[j];
+                } else {                                           // one conversion per pair of positions
+                    uint16_t *ot16 = reinterpret_cast<uint16_t *>(ot);
+#pragma unroll
+                    for (int j = 0; j < 4; j += 2) {
+                        const uint32_t two = pack2_from_f32<out_t>(o[j], o[j + 1]);
+                        ot16[(4 * q + j) * Cp + c] = (uint16_t)(two & 0xffffu);
+                        ot16[(4 * q + j + 1) * Cp + c] = (uint16_t)(two >> 16);
+                    }
+                }
             }
         }
         __syncthreads();
