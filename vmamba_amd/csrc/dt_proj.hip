@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
                     uint32_t w[8];
 #pragma unroll
                     for (int v = 0; v < 8; ++v)
-                        w[v] = (uint32_t)from_f32<T>(acc[2 * v]).bits | ((uint32_t)from_f32<T>(acc[2 * v + 1]).bits << 16);
+                        w[v] = pack2_from_f32<T>(acc[2 * v], acc[2 * v + 1]);
                     uint4 *dst = reinterpret_cast<uint4 *>(ob + j * kDtPitch + t * kDtTile + 16 * kh);
                     dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
                     dst[1] = make_uint4(w[4], w[5], w[6], w[7]);

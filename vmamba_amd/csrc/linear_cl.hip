@@ -117,8 +117,12 @@ __global__ __launch_bounds__(kBlock, 2) void linear_cl_kernel(const LinArgs p) {
                     const float g = to_f32(T{gamma_l[c]}), bt = to_f32(T{beta_l[c]});
                     const float in[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        stage[(4 * quad + e) * PS + c] = from_f32<T>(fmaf((in[e] - mean[e]) * rstd[e], g, bt)).bits;
+                    for (int e = 0; e < 4; e += 2) {                 // one conversion per pair of positions
+                        const uint32_t two = pack2_from_f32<T>(fmaf((in[e] - mean[e]) * rstd[e], g, bt),
+                                                               fmaf((in[e + 1] - mean[e + 1]) * rstd[e + 1], g, bt));
+                        stage[(4 * quad + e) * PS + c] = (uint16_t)(two & 0xffffu);
+                        stage[(4 * quad + e + 1) * PS + c] = (uint16_t)(two >> 16);
+                    }
                 }
                 wave_lds_sync();
             } else {

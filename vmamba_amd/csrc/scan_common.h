@@ -135,8 +135,7 @@ __device__ __forceinline__ void store_items(T *__restrict__ row, int pos, int L,
             if (pos < L) {
                 uint32_t w[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    w[i] = (uint32_t)from_f32<T>(v[2 * i]).bits | ((uint32_t)from_f32<T>(v[2 * i + 1]).bits << 16);
+                for (int i = 0; i < 4; ++i) w[i] = pack2_from_f32<T>(v[2 * i], v[2 * i + 1]);
                 *reinterpret_cast<uint4 *>(row + pos) = make_uint4(w[0], w[1], w[2], w[3]);
             }
         } else {
