@@ -84,9 +84,17 @@ template <typename T> __device__ __forceinline__ void ln_add_rounded(float (&v)[
     }
 }
 
+// Sum over a power-of-two group of lanes, the same value in every lane of the group.  Inside a row of 16 lanes the
+// partners come through the DPP operand of the add itself (lane ^ 1 and lane ^ 2 as quad permutations, then the mirror
+// images inside 8 and 16 lanes: a quad meets the other quad of its half, a half the other half) -- no LDS round trip;
+// wider groups finish with lane exchanges.
 template <int kGroup> __device__ __forceinline__ float group_sum(float v) {
+    if constexpr (kGroup >= 2) v += dpp_move<0xB1>(v, v);      // quad_perm [1,0,3,2]
+    if constexpr (kGroup >= 4) v += dpp_move<0x4E>(v, v);      // quad_perm [2,3,0,1]
+    if constexpr (kGroup >= 8) v += dpp_move<0x141>(v, v);     // row_half_mirror
+    if constexpr (kGroup >= 16) v += dpp_move<0x140>(v, v);    // row_mirror
 #pragma unroll
-    for (int off = kGroup / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kGroup);
+    for (int off = 16; off < kGroup; off <<= 1) v += __shfl_xor(v, off, kWave);
     return v;
 }
 
