@@ -498,7 +498,7 @@ static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
 template <typename in_t, typename out_t, bool kVec>
 static int launch_scan(const ScanArgs &a, hipStream_t stream) {
     // Few long rows: split every row over the 4 wavefronts of a workgroup.
-    const bool split_rows = a.L > SS2D_SCAN_CHUNK && a.rows < 16384;
+    const bool split_rows = a.L > SS2D_SCAN_CHUNK && a.rows < 2048;      // (3072 rows and more: a wavefront per row is faster)
     if (split_rows) {
         const size_t smem = (size_t)(2 * a.N * kWavesPerWg + 2 * a.N) * sizeof(float2);
         if (a.softplus) {
