@@ -571,13 +571,13 @@ __global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const 
     auto totals = [&](const float (&acc)[4], int which, auto finish) {
         *reinterpret_cast<float4 *>(red + 4 * t) = make_float4(acc[0], acc[1], acc[2], acc[3]);
         __syncthreads();
-        if (t < Lt) {
+        for (int l = t; l < Lt; l += (int)blockDim.x) {      // (a workgroup may have fewer threads than positions)
             float tot = 0.0f;
 #pragma unroll 4
             for (int gg = 0; gg < G; ++gg)
 #pragma unroll
-                for (int c = 0; c < kCh; ++c) tot += red[gg * Qn * 4 + c * L + t];
-            stat[which * kLnImgStat + t] = finish(tot);
+                for (int c = 0; c < kCh; ++c) tot += red[gg * Qn * 4 + c * L + l];
+            stat[which * kLnImgStat + l] = finish(tot);
         }
         __syncthreads();
     };
