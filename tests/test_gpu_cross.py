@@ -21,6 +21,9 @@ SHAPES = [
     (1, 1, 1, 1), (2, 3, 3, 5), (3, 5, 7, 7), (2, 9, 14, 14), (2, 6, 28, 28), (2, 96, 56, 56),
     (3, 5, 56, 57), (2, 7, 57, 58), (130, 3, 1, 1), (2, 3, 1, 37), (2, 3, 41, 1),
     (1, 2, 200, 130), (1, 3, 128, 128), (1, 1, 256, 256), (1, 2, 65, 300),
+    # odd maps with an even channel count (16-bit elements then travel as pairs across map boundaries): one group, several
+    # groups with a short last one, single positions
+    (2, 6, 7, 7), (3, 10, 5, 9), (1, 2, 1, 1), (2, 4, 3, 3), (2, 170, 7, 7), (1, 86, 7, 7), (2, 768, 7, 7),
 ]
 
 

@@ -110,6 +110,64 @@ __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__rest
     }
 }
 
+// 16-bit maps with an ODD number of positions (7 x 7, 5 x 9 ...): single maps start on odd element offsets, but a group
+// of an even number of maps is one block of memory that starts on a 4-byte boundary in x and in each of the four
+// outputs (C even).  The block is read, kept in LDS and written as a flat stream of 4-byte pairs: output pair q of a
+// direction is two consecutive scan positions (possibly the last of one map and the first of the next), each picked
+// from the LDS copy through the direction's route.  Half the memory instructions of the element-wise variant.
+__global__ __launch_bounds__(kBlock) void cross_scan_maps_flat_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ y,
+                                                                      int C, int H, int W, int G, int groups_per_image,
+                                                                      FastDiv divL, FastDiv divH) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    uint16_t *lds = reinterpret_cast<uint16_t *>(smem_raw);      // the g maps as they lie in memory
+    const uint32_t wg = blockIdx.x;
+    const uint32_t b = wg / (uint32_t)groups_per_image;
+    const uint32_t c0 = (wg - b * groups_per_image) * (uint32_t)G;
+    const uint32_t g = min((uint32_t)G, (uint32_t)C - c0);
+    const uint32_t L = divL.d, n = g * L, pairs = n / 2;         // an odd last element (odd g) is handled on its own
+    const size_t CL = (size_t)C * L;
+    const uint16_t *xin = x + ((size_t)b * C + c0) * L;
+    uint16_t *y0 = y + ((size_t)b * 4) * CL + (size_t)c0 * L;
+    const uint32_t *xin_p = reinterpret_cast<const uint32_t *>(xin);
+    uint32_t *lds_p = reinterpret_cast<uint32_t *>(lds), *y0_p = reinterpret_cast<uint32_t *>(y0);
+    for (uint32_t base = threadIdx.x; base < pairs; base += kBlock * kUnroll) {
+        uint32_t v[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q < pairs) v[k] = xin_p[q];
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint32_t q = base + k * kBlock;
+            if (q < pairs) { y0_p[q] = v[k]; lds_p[q] = v[k]; }
+        }
+    }
+    if ((n & 1u) && threadIdx.x == 0) { const uint16_t v = xin[n - 1]; y0[n - 1] = v; lds[n - 1] = v; }
+    __syncthreads();
+    // source element (inside the block) of scan position t of map m, per direction
+    auto src1 = [&](uint32_t m, uint32_t t) { uint32_t w, h; divmod(t, divH, w, h); return m * L + h * (uint32_t)W + w; };
+    uint16_t *y1 = y0 + CL, *y2 = y1 + CL, *y3 = y2 + CL;
+    for (uint32_t q = threadIdx.x; q < pairs; q += kBlock) {
+        uint32_t m0, t0;
+        divmod(2 * q, divL, m0, t0);
+        const bool wrap = t0 + 1 == L;
+        const uint32_t m1 = wrap ? m0 + 1 : m0, t1 = wrap ? 0 : t0 + 1;
+        const uint32_t a1 = lds[src1(m0, t0)], b1 = lds[src1(m1, t1)];
+        const uint32_t a2 = lds[m0 * L + (L - 1 - t0)], b2 = lds[m1 * L + (L - 1 - t1)];
+        const uint32_t a3 = lds[src1(m0, L - 1 - t0)], b3 = lds[src1(m1, L - 1 - t1)];
+        reinterpret_cast<uint32_t *>(y1)[q] = a1 | (b1 << 16);
+        reinterpret_cast<uint32_t *>(y2)[q] = a2 | (b2 << 16);
+        reinterpret_cast<uint32_t *>(y3)[q] = a3 | (b3 << 16);
+    }
+    if ((n & 1u) && threadIdx.x == 0) {
+        const uint32_t m = g - 1, t = L - 1;
+        y1[n - 1] = lds[src1(m, t)];
+        y2[n - 1] = lds[m * L];
+        y3[n - 1] = lds[src1(m, 0)];
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void cross_scan_tile_kernel(const T *__restrict__ x, T *__restrict__ y, int C,
                                                                  int H, int W, int tiles_h, int tiles_w) {
@@ -168,6 +226,21 @@ static int launch_cross_scan(const void *x, void *y, int B, int C, int H, int W,
         bool pairs = false;
         if constexpr (sizeof(T) == 2) {
             pairs = (L % 2 == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 4 == 0);
+        }
+        if constexpr (sizeof(T) == 2) {
+            // odd maps: an even number of maps per workgroup is a 4-byte aligned block on both sides
+            const bool aligned4 = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 4 == 0;
+            if (L % 2 == 1 && C % 2 == 0 && aligned4 && G >= 2) {
+                const int Gf = G & ~1;
+                const int groups_f = (C + Gf - 1) / Gf;
+                const int64_t n_wg_f = (int64_t)B * groups_f;
+                if (n_wg_f <= 0x7fffffff) {
+                    hipLaunchKernelGGL(cross_scan_maps_flat_kernel, dim3((uint32_t)n_wg_f), dim3(kBlock), (size_t)(Gf * L * 2 + 4), stream,
+                                       (const uint16_t *)x, (uint16_t *)y, C, H, W, Gf, groups_f, make_fastdiv((uint32_t)L),
+                                       make_fastdiv((uint32_t)H));
+                    return launch_status();
+                }
+            }
         }
         if (pairs) {
             if constexpr (sizeof(T) == 2) {
