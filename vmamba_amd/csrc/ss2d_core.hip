@@ -699,6 +699,48 @@ __global__ __launch_bounds__(kBlock) void cross_scan_1b1_wave_kernel(const T *__
     }
 }
 
+// One workgroup per map, 16-bit maps with an even number of positions on 4-byte boundaries: two positions per lane and
+// memory instruction (see the wavefront variant below).
+__global__ __launch_bounds__(kBlock) void cross_scan_1b1_pairs_kernel(const uint16_t *__restrict__ x, uint16_t *__restrict__ y, int H,
+                                                                      int W, int Wp, int64_t y_bs, int64_t y_ks, int64_t y_cs,
+                                                                      FastDiv divC, FastDiv divW, FastDiv divH) {
+    extern __shared__ __align__(16) unsigned char map_smem[];
+    uint16_t *tile = reinterpret_cast<uint16_t *>(map_smem);
+    uint32_t bk, c;
+    divmod(blockIdx.x, divC, bk, c);
+    const uint32_t b = bk / 4, k = bk % 4;
+    const int L = H * W, P = L / 2;
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(x + (size_t)blockIdx.x * L);
+    uint32_t *dst = reinterpret_cast<uint32_t *>(y + (int64_t)b * y_bs + (int64_t)k * y_ks + (int64_t)c * y_cs);
+    if ((k & 1u) == 0) {
+        for (int q = threadIdx.x; q < P; q += kBlock) {
+            const uint32_t v = src[k == 0 ? q : P - 1 - q];
+            dst[q] = k == 0 ? v : (v >> 16) | (v << 16);
+        }
+        return;
+    }
+    for (int q = threadIdx.x; q < P; q += kBlock) {
+        const uint32_t v = src[q];
+        uint32_t h, w;
+        divmod((uint32_t)(2 * q), divW, h, w);
+        tile[h * Wp + w] = (uint16_t)(v & 0xffffu);
+        if (++w == (uint32_t)W) { w = 0; ++h; }
+        tile[h * Wp + w] = (uint16_t)(v >> 16);
+    }
+    __syncthreads();
+    for (int q = threadIdx.x; q < P; q += kBlock) {
+        uint32_t e[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int j = 2 * q + i;
+            uint32_t w, h;
+            divmod((uint32_t)(k == 1 ? j : L - 1 - j), divH, w, h);
+            e[i] = tile[h * Wp + w];
+        }
+        dst[q] = e[0] | (e[1] << 16);
+    }
+}
+
 // The same for 16-bit maps with an even number of positions whose rows start on 4-byte boundaries on both sides: two
 // positions per lane and memory instruction (the reversed routes swap the halves; the transposing routes pick the two
 // elements from the LDS copy).
@@ -772,6 +814,16 @@ static int launch_cross_scan_1b1(const void *x, void *y, int B, int C, int H, in
         return launch_status();
     }
     const int use_lds = smem <= 48 * 1024;
+    if constexpr (sizeof(T) == 2) {
+        const bool even = ((int64_t)H * W) % 2 == 0 && y_bs % 2 == 0 && y_ks % 2 == 0 && y_cs % 2 == 0 &&
+                          (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 4 == 0;
+        if (even && use_lds) {
+            hipLaunchKernelGGL(cross_scan_1b1_pairs_kernel, dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const uint16_t *)x,
+                               (uint16_t *)y, H, W, Wp, y_bs, y_ks, y_cs, make_fastdiv((uint32_t)C), make_fastdiv((uint32_t)W),
+                               make_fastdiv((uint32_t)H));
+            return launch_status();
+        }
+    }
     if (!use_lds) smem = 0;
     hipLaunchKernelGGL((cross_scan_1b1_kernel<T>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x, (T *)y, H, W, Wp,
                        use_lds, y_bs, y_ks, y_cs, make_fastdiv((uint32_t)C), make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)H));
