@@ -14,7 +14,9 @@ SHAPES = [(2, 96, 56, 56), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (
           (2, 12, 5, 6), (1, 7, 4, 4), (1, 32, 1, 70), (1, 16, 2, 200), (1, 64, 20, 128),
           # channel tiles of 64 / 32 with row tiles and a short last one, rows of 16- and 8-byte pieces, odd whole images,
           # a map too tall for one tile whose rows take no 8-byte stores (the older row-tile kernel), the widest rows
-          (2, 64, 30, 56), (1, 32, 37, 28), (2, 128, 5, 9), (1, 64, 100, 14), (1, 32, 3, 120), (1, 160, 9, 12), (3, 64, 8, 8)]
+          (2, 64, 30, 56), (1, 32, 37, 28), (2, 128, 5, 9), (1, 64, 100, 14), (1, 32, 3, 120), (1, 160, 9, 12), (3, 64, 8, 8),
+          # tiles of at most 32 positions with several channel groups (the rotation of the output rows wraps)
+          (3, 40, 4, 2), (2, 24, 4, 4), (1, 48, 5, 6), (2, 16, 3, 3), (1, 72, 2, 9)]
 
 
 def _tol(dtype):

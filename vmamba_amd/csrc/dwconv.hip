@@ -565,6 +565,7 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             int TH = 224 / W;
             TH = TH < 1 ? 1 : (TH > H ? H : TH);
             int out_pitch = ((TH * W + 15) / 16) * 16;                // a multiple of 16 elements: rows rotate by 16, 32, 48
+            if (out_pitch < 48) out_pitch = 48;                       // ... and a rotated column wraps around at most once
             const int row_tiles = (H + TH - 1) / TH, ch_tiles = (D + kDwCh - 1) / kDwCh;
             const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
             // whole images whose rows do not take 16-byte stores: the tile leaves as one flat block
