@@ -407,6 +407,9 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--image-size", type=int, default=224,
+                    help="side of the square input images; 224 is the metric's workload, other sizes are side runs named in "
+                         "config.workload (benchmark config 4: --batch 4 --image-size 1024 --sub-batches 1)")
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
@@ -457,7 +460,7 @@ def main():
         # conv weights in channels-last memory format (same values, same state_dict): the stem / downsample convs then
         # run NHWC kernels and the permutes around them are views instead of copies
         model = model.to(memory_format=torch.channels_last)
-    x = torch.randn(args.batch, 3, 224, 224, device=dev).bfloat16()
+    x = torch.randn(args.batch, 3, args.image_size, args.image_size, device=dev).bfloat16()
 
     def time_steps(step, warmup, steps):
         """The reference's protocol (classification/main.py:346-363): warm-up, synchronise, time `steps` launches
@@ -610,7 +613,7 @@ def main():
                 x32 = x.float()
                 model32(x32)
                 t32 = time_steps(lambda: model32(x32), 3, 10) / 10
-                extra["fp32"] = dict(workload=f"VMamba-T forward, batch {args.batch} @224^2, fp32 activations and weights (the reference "
+                extra["fp32"] = dict(workload=f"VMamba-T forward, batch {args.batch} @{args.image_size}^2, fp32 activations and weights (the reference "
                                               f"harness's precision, no AMP), eager launches, {gemm_mode.split(' picked')[0]} as met",
                                      ms_per_step=t32 * 1e3, img_per_s=args.batch / t32)
                 log("fp32:", extra["fp32"])
@@ -651,7 +654,7 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"launch": launch, "sub_batches": sub_batches if launch == "concurrent" else 1,
-                   "workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @224x224, "
+                   "workload": f"VMamba-T (vmamba_tiny_s1l8 shape, random init) forward, batch {args.batch} @{args.image_size}x{args.image_size}, "
                                f"bf16 activations/weights, fp32 scan state, {args.layout} blocks, {launch_text}, {gemm_mode}; "
                                f"SS2D core, LayerNorm, depthwise conv, patch-embedding stem, narrow-stage MLP and projections on HIP kernels"},
         "ms_per_step_eager": ms_of("eager"), "ms_per_step_one_graph": ms_of("one_graph"),

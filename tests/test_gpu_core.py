@@ -262,7 +262,8 @@ def test_core_rejections():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8, torch.float64], ids=str)
 @pytest.mark.parametrize("shape", [(2, 3, 56, 56), (3, 5, 7, 9), (1, 2, 1, 17), (2, 1, 13, 1), (1, 1, 130, 100),
-                                   (2, 6, 14, 14), (3, 2, 4, 6), (2, 3, 2, 1), (1, 5, 3, 10), (2, 2, 30, 27)],
+                                   (2, 6, 14, 14), (3, 2, 4, 6), (2, 3, 2, 1), (1, 5, 3, 10), (2, 2, 30, 27),
+                                   (1, 2, 256, 256), (2, 1, 130, 197), (1, 1, 65, 400)],      # maps walked in 64 x 64 tiles
                          ids=lambda s: "x".join(map(str, s)))
 def test_cross_scan_1b1_bit_exact(shape, dtype):
     _announce("cross_scan_1b1", shape, dtype)

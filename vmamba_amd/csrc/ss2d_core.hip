@@ -664,6 +664,47 @@ __global__ __launch_bounds__(kBlock) void cross_scan_1b1_kernel(const T *__restr
     }
 }
 
+// Large maps: one workgroup per 64 x 64 tile of a map.  Rows are read along W; the row-major directions store them as
+// they are (forwards or mirrored), the column-major ones read the tile back down its columns from LDS (pitch 65) and
+// store along H, so both sides of every direction are contiguous per wavefront.
+constexpr int k1b1Tile = 64;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cross_scan_1b1_tile_kernel(const T *__restrict__ x, T *__restrict__ y, int H, int W,
+                                                                     int tiles_h, int tiles_w, int64_t y_bs, int64_t y_ks,
+                                                                     int64_t y_cs, FastDiv divC) {
+    __shared__ T tile[k1b1Tile * (k1b1Tile + 1)];
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    uint32_t wg = blockIdx.x;
+    const uint32_t tw = wg % (uint32_t)tiles_w; wg /= (uint32_t)tiles_w;
+    const uint32_t th = wg % (uint32_t)tiles_h; wg /= (uint32_t)tiles_h;      // wg: the map (b, k, c)
+    uint32_t bk, c;
+    divmod(wg, divC, bk, c);
+    const uint32_t b = bk / 4, k = bk % 4;
+    const size_t L = (size_t)H * W;
+    const T *src = x + (size_t)wg * L;
+    T *dst = y + (int64_t)b * y_bs + (int64_t)k * y_ks + (int64_t)c * y_cs;
+    const uint32_t h0 = th * k1b1Tile, w0 = tw * k1b1Tile;
+    const bool column_major = (k & 1u) != 0, mirrored = k >= 2;
+    for (uint32_t rr = wave; rr < (uint32_t)k1b1Tile; rr += kBlock / kWave) {
+        const uint32_t h = h0 + rr, w = w0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t r = (size_t)h * W + w;
+            const T v = src[r];
+            if (column_major) tile[rr * (k1b1Tile + 1) + lane] = v;
+            else dst[mirrored ? L - 1 - r : r] = v;
+        }
+    }
+    if (!column_major) return;                 // uniform over the workgroup
+    __syncthreads();
+    for (uint32_t cc = wave; cc < (uint32_t)k1b1Tile; cc += kBlock / kWave) {
+        const uint32_t w = w0 + cc, h = h0 + lane;
+        if (h < (uint32_t)H && w < (uint32_t)W) {
+            const size_t t = (size_t)w * H + h;
+            dst[mirrored ? L - 1 - t : t] = tile[lane * (k1b1Tile + 1) + cc];
+        }
+    }
+}
+
 // Short maps (L <= 1024): one WAVEFRONT per map, four maps per workgroup, each with a private LDS tile -- a whole
 // workgroup per 49- or 196-element map leaves most of its lanes idle and the launch is then bound by workgroup count.
 template <typename T>
@@ -813,7 +854,9 @@ static int launch_cross_scan_1b1(const void *x, void *y, int B, int C, int H, in
                            make_fastdiv((uint32_t)H));
         return launch_status();
     }
-    const int use_lds = smem <= 48 * 1024;
+    // maps too large for one workgroup's LDS, or few large maps (a workgroup per map would leave most of the chip idle)
+    const bool by_tiles = smem > 48 * 1024 || ((int64_t)H * W >= 8192 && n_wg < 2048);
+    const int use_lds = !by_tiles;
     if constexpr (sizeof(T) == 2) {
         const bool even = ((int64_t)H * W) % 2 == 0 && y_bs % 2 == 0 && y_ks % 2 == 0 && y_cs % 2 == 0 &&
                           (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 4 == 0;
@@ -824,7 +867,16 @@ static int launch_cross_scan_1b1(const void *x, void *y, int B, int C, int H, in
             return launch_status();
         }
     }
-    if (!use_lds) smem = 0;
+    if (!use_lds) {
+        const int tiles_h = (H + k1b1Tile - 1) / k1b1Tile, tiles_w = (W + k1b1Tile - 1) / k1b1Tile;
+        const int64_t n_tiles = n_wg * tiles_h * tiles_w;
+        if (n_tiles <= 0x7fffffff) {
+            hipLaunchKernelGGL((cross_scan_1b1_tile_kernel<T>), dim3((uint32_t)n_tiles), dim3(kBlock), 0, stream, (const T *)x, (T *)y,
+                               H, W, tiles_h, tiles_w, y_bs, y_ks, y_cs, make_fastdiv((uint32_t)C));
+            return launch_status();
+        }
+        smem = 0;
+    }
     hipLaunchKernelGGL((cross_scan_1b1_kernel<T>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x, (T *)y, H, W, Wp,
                        use_lds, y_bs, y_ks, y_cs, make_fastdiv((uint32_t)C), make_fastdiv((uint32_t)W), make_fastdiv((uint32_t)H));
     return launch_status();
