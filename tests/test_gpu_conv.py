@@ -16,7 +16,9 @@ SHAPES = [(2, 96, 56, 56), (3, 192, 28, 28), (2, 384, 14, 14), (2, 768, 7, 7), (
           # a map too tall for one tile whose rows take no 8-byte stores (the older row-tile kernel), the widest rows
           (2, 64, 30, 56), (1, 32, 37, 28), (2, 128, 5, 9), (1, 64, 100, 14), (1, 32, 3, 120), (1, 160, 9, 12), (3, 64, 8, 8),
           # tiles of at most 32 positions with several channel groups (the rotation of the output rows wraps)
-          (3, 40, 4, 2), (2, 24, 4, 4), (1, 48, 5, 6), (2, 16, 3, 3), (1, 72, 2, 9)]
+          (3, 40, 4, 2), (2, 24, 4, 4), (1, 48, 5, 6), (2, 16, 3, 3), (1, 72, 2, 9),
+          # wide images in column tiles of 8 / 4 / 5 / 4 segments (and 17 segments, which no tile width divides)
+          (1, 32, 20, 256), (2, 64, 9, 128), (1, 32, 33, 200), (1, 64, 5, 192), (1, 96, 16, 136)]
 
 
 def _tol(dtype):

@@ -340,9 +340,9 @@ __device__ __forceinline__ int plane_at(int c, int plane_dw) { const int o = c *
 template <typename T, bool kSilu, int kCh>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__restrict__ x, const T *__restrict__ weight,
                                                                   const T *__restrict__ bias, T *__restrict__ y, int D, int H,
-                                                                  int W, int TH, int row_tiles, int ch_tiles, int pitch,
-                                                                  int plane_dw, int nseg, int n_it, int flat_out,
-                                                                  FastDiv divHalf, FastDiv divNseg) {
+                                                                  int W, int TH, int row_tiles, int ch_tiles, int col_tiles,
+                                                                  int TW, int pitch, int plane_dw, int nseg, int n_it,
+                                                                  int flat_out, FastDiv divHalf, FastDiv divNseg) {
     constexpr int kLpc = kBlock / kCh;                           // lanes per channel in the compute phase
     constexpr int kCv = kCh / 8;                                 // 16-byte channel vectors per position
     constexpr int kPer = kBlock / kCv;                           // position pairs per staging pass
@@ -350,10 +350,12 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
     extern __shared__ __align__(16) uint32_t dwp_smem[];         // [kCh][plane_dw]
     uint32_t wg = blockIdx.x;
     const uint32_t ct = wg % ch_tiles; wg /= ch_tiles;
+    const uint32_t cx = wg % col_tiles; wg /= col_tiles;         // wide images: tiles of TW columns (col_tiles = 1 otherwise)
     const uint32_t rt = wg % row_tiles;
     const uint32_t b = wg / row_tiles;
     const int h0 = (int)rt * TH;
     const int rows = min(TH, H - h0);
+    const int wb = (int)cx * TW;                                 // first image column of the tile
     const int c_base = (int)ct * kCh;
     const int L = H * W, half = pitch / 2;
 
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
                 const int q = q0 + u * kPer;
                 uint32_t rr, pp;
                 divmod((uint32_t)q, divHalf, rr, pp);
-                const int h = h0 - 1 + (int)rr, w0 = 2 * (int)pp - 1, w1 = 2 * (int)pp;
+                const int h = h0 - 1 + (int)rr, w0 = wb + 2 * (int)pp - 1, w1 = wb + 2 * (int)pp;
                 const bool row_ok = q < n_items && h >= 0 && h < H;
                 const uint32_t off_a = (row_ok && w0 >= 0 && w0 < W) ? (uint32_t)((h * W + w0) * D + c0) * 2u : 0x7ffffff0u;
                 const uint32_t off_b = (row_ok && w1 < W) ? (uint32_t)((h * W + w1) * D + c0) * 2u : 0x7ffffff0u;
@@ -454,7 +456,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
 #pragma unroll
                 for (int i = 0; i < 4; ++i) keep[it][i] = o[i];
             } else if (sg < n_seg) {
-                T *dst = yc + r * W + seg * 8;
+                T *dst = yc + r * W + wb + seg * 8;
                 if (W % 8 == 0) {
                     *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
                 } else {                                          // W % 4 == 0: 8-byte rows, a last segment of 4
@@ -535,9 +537,16 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
     auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     if constexpr (sizeof(T) == 2) {
         // plane variant: channel tiles of 64 (or 32), full rows, outputs that leave as whole 8- or 16-byte pieces
-        if (in_channel_last && D % 32 == 0 && W <= 120 && al16(x) && al16(y) && (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
+        // images wider than 120 columns: column tiles of lpc, ..., 4 whole segments, if such a width divides W
+        int seg_t = 0;
+        if (W > 120 && W % 8 == 0)
+            for (int n = kBlock / (D % 64 == 0 ? 64 : 32); n >= 4 && seg_t == 0; --n)
+                if ((W / 8) % n == 0) seg_t = n;
+        if (in_channel_last && D % 32 == 0 && (W <= 120 || seg_t > 0) && al16(x) && al16(y) &&
+            (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
             const int kch = D % 64 == 0 ? 64 : 32, lpc = kBlock / kch;
-            const int nseg = (W + 7) / 8, pitch = 8 * nseg + 4;
+            const int TW = seg_t > 0 ? 8 * seg_t : W, col_tiles = seg_t > 0 ? W / TW : 1;
+            const int nseg = (TW + 7) / 8, pitch = 8 * nseg + 4;
             int TH = (7 * lpc) / nseg;
             TH = TH > H ? H : TH;
             const int row_tiles = TH >= 1 ? (H + TH - 1) / TH : 0, ch_tiles = D / kch;
@@ -548,12 +557,12 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
             plane_dw += 1;                                         // room for the parity shift
             plane_dw += (want - plane_dw % 8 + 8) % 8;
             const size_t smem = ((size_t)kch * plane_dw + 2) * 4;
-            const int64_t n_wg = (int64_t)B * row_tiles * ch_tiles;
+            const int64_t n_wg = (int64_t)B * row_tiles * col_tiles * ch_tiles;
             if (TH >= 1 && n_it <= kDwpMaxIt && (!flat_out || row_tiles == 1) && smem <= 64 * 1024 && n_wg <= 0x7fffffff) {
 #define SS2D_DW_PLANES(SILU, KCH)                                                                                              \
     hipLaunchKernelGGL((dwconv3x3_planes_kernel<T, SILU, KCH>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x,  \
-                       (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles, pitch, plane_dw, nseg, n_it,     \
-                       flat_out, make_fastdiv((uint32_t)(pitch / 2)), make_fastdiv((uint32_t)nseg))
+                       (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles, col_tiles, TW, pitch, plane_dw,  \
+                       nseg, n_it, flat_out, make_fastdiv((uint32_t)(pitch / 2)), make_fastdiv((uint32_t)nseg))
                 if (kch == 64) { if (apply_silu) SS2D_DW_PLANES(true, 64); else SS2D_DW_PLANES(false, 64); }
                 else { if (apply_silu) SS2D_DW_PLANES(true, 32); else SS2D_DW_PLANES(false, 32); }
 #undef SS2D_DW_PLANES
