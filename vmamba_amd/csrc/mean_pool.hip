@@ -25,13 +25,26 @@ __global__ __launch_bounds__(kBlock) void mean_pool_cl_kernel(const T *__restric
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
     if (c0 < C) {
         const T *xb = x + (size_t)b * L * C + c0;
-        for (int l = slice; l < L; l += kPoolSlices) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(xb + (size_t)l * C);
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        // eight positions requested together (long maps would otherwise pay one memory latency per position), added
+        // in position order
+        constexpr int kAhead = 8;
+        for (int l0 = slice; l0 < L; l0 += kAhead * kPoolSlices) {
+            uint4 v[kAhead];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[2 * i] += unpack_lo<T>(w[i]);
-                acc[2 * i + 1] += unpack_hi<T>(w[i]);
+            for (int u = 0; u < kAhead; ++u) {
+                const int l = min(l0 + u * kPoolSlices, L - 1);
+                v[u] = *reinterpret_cast<const uint4 *>(xb + (size_t)l * C);
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                if (l0 + u * kPoolSlices < L) {
+                    const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[2 * i] += unpack_lo<T>(w[i]);
+                        acc[2 * i + 1] += unpack_hi<T>(w[i]);
+                    }
+                }
             }
         }
     }
