@@ -497,6 +497,85 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
     for (int pc = threadIdx.x; pc < kCh * L / 8; pc += kBlock) dst[pc] = src[pc];
 }
 
+// fp32, channel-last input: the 16-bit tap-by-tap kernel's scheme with four channels per 16-byte vector.  A workgroup
+// owns 32 consecutive positions x 32 channels; a lane convolves 4 channels at one position from nine 16-byte loads
+// (the eight lanes of a position read 128 contiguous bytes; neighbouring positions re-use the lines out of L1 / L2),
+// parks its results in LDS and the tile leaves transposed, 16 bytes per lane along the positions.  Same arithmetic as the
+// generic kernel below: taps accumulated in (kh, kw) order with fused multiply-adds, bias added last, exact SiLU.
+constexpr int kDwfPos = 32, kDwfCh = 32, kDwfPitch = kDwfPos + 4;
+template <bool kSilu>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_f32_kernel(const float *__restrict__ x, const float *__restrict__ weight,
+                                                                     const float *__restrict__ bias, float *__restrict__ y, int D,
+                                                                     int H, int W, int pos_tiles, int ch_tiles, FastDiv divW) {
+    __shared__ __align__(16) float tile[kDwfCh * kDwfPitch];
+    uint32_t wg = blockIdx.x;
+    const uint32_t ct = wg % ch_tiles; wg /= ch_tiles;
+    const uint32_t pt = wg % pos_tiles;
+    const uint32_t b = wg / pos_tiles;
+    const int L = H * W;
+    const int r0 = (int)pt * kDwfPos;
+    const int p = threadIdx.x / 8, cv = threadIdx.x % 8;
+    const int c0 = (int)ct * kDwfCh + cv * 4;           // this lane's 4 channels
+    const int r = r0 + p;
+    if (r < L && c0 < D) {
+        uint32_t h, w;
+        divmod((uint32_t)r, divW, h, w);
+        float wt[36];                                   // [channel][tap]: 9 consecutive 16-byte vectors
+        {
+            const float4 *wp = reinterpret_cast<const float4 *>(weight + (size_t)c0 * 9);
+#pragma unroll
+            for (int k = 0; k < 9; ++k) {
+                const float4 t = wp[k];
+                wt[4 * k] = t.x; wt[4 * k + 1] = t.y; wt[4 * k + 2] = t.z; wt[4 * k + 3] = t.w;
+            }
+        }
+        const float *xb = x + (size_t)b * L * D;
+        float4 tap[9];
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int hh = (int)h + kh - 1, ww = (int)w + kw - 1;
+                const bool in = hh >= 0 && hh < H && ww >= 0 && ww < W;
+                // out-of-image taps read this position's own vector (a valid address) and are left out of the sum
+                const size_t off = in ? ((size_t)hh * W + ww) * D + c0 : ((size_t)h * W + w) * D + c0;
+                tap[kh * 3 + kw] = *reinterpret_cast<const float4 *>(xb + off);
+            }
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int hh = (int)h + kh - 1, ww = (int)w + kw - 1;
+                if (hh >= 0 && hh < H && ww >= 0 && ww < W) {
+                    const float xv[4] = {tap[kh * 3 + kw].x, tap[kh * 3 + kw].y, tap[kh * 3 + kw].z, tap[kh * 3 + kw].w};
+#pragma unroll
+                    for (int ci = 0; ci < 4; ++ci) acc[ci] = fmaf(wt[ci * 9 + kh * 3 + kw], xv[ci], acc[ci]);
+                }
+            }
+        if (bias) {
+            const float4 bv = *reinterpret_cast<const float4 *>(bias + c0);
+            acc[0] += bv.x; acc[1] += bv.y; acc[2] += bv.z; acc[3] += bv.w;
+        }
+#pragma unroll
+        for (int ci = 0; ci < 4; ++ci) tile[(cv * 4 + ci) * kDwfPitch + p] = kSilu ? silu_f32(acc[ci]) : acc[ci];
+    }
+    __syncthreads();
+    // write back: lane -> (channel = tid / 8, four consecutive positions)
+    const int c = threadIdx.x / 8, chunk = threadIdx.x % 8;
+    const int cg = (int)ct * kDwfCh + c;
+    const int rr = r0 + chunk * 4;
+    if (cg < D && rr < L) {
+        float *yo = y + ((size_t)b * D + cg) * L + rr;
+        const float *src = tile + c * kDwfPitch + chunk * 4;
+        if (rr + 4 <= L && (L % 4) == 0) {
+            *reinterpret_cast<float4 *>(yo) = *reinterpret_cast<const float4 *>(src);
+        } else {
+            for (int i = 0; i < 4 && rr + i < L; ++i) yo[i] = src[i];
+        }
+    }
+}
+
 // Generic variant: any element type, either input layout, one output element per lane (lanes along W).
 template <typename T, bool kInChannelLast, bool kSilu>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_generic_kernel(const T *__restrict__ x, const T *__restrict__ weight,
@@ -612,6 +691,24 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
                                    make_fastdiv((uint32_t)W));
             }
             return launch_status();
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        if (in_channel_last && D % 4 == 0 && al16(x) && al16(w) && al16(y) && (!bias || al16(bias))) {
+            const int pos_tiles = (int)((L + kDwfPos - 1) / kDwfPos), ch_tiles = (D + kDwfCh - 1) / kDwfCh;
+            const int64_t n_tiles = (int64_t)B * pos_tiles * ch_tiles;
+            if (n_tiles <= 0x7fffffff) {
+                if (apply_silu) {
+                    hipLaunchKernelGGL((dwconv3x3_cl2cf_f32_kernel<true>), dim3((uint32_t)n_tiles), dim3(kBlock), 0, stream,
+                                       (const float *)x, (const float *)w, (const float *)bias, (float *)y, D, H, W, pos_tiles,
+                                       ch_tiles, make_fastdiv((uint32_t)W));
+                } else {
+                    hipLaunchKernelGGL((dwconv3x3_cl2cf_f32_kernel<false>), dim3((uint32_t)n_tiles), dim3(kBlock), 0, stream,
+                                       (const float *)x, (const float *)w, (const float *)bias, (float *)y, D, H, W, pos_tiles,
+                                       ch_tiles, make_fastdiv((uint32_t)W));
+                }
+                return launch_status();
+            }
         }
     }
     const int64_t total = (int64_t)B * D * L;
