@@ -612,9 +612,12 @@ def main():
                 model32 = model.float()
                 x32 = x.float()
                 model32(x32)
+                t_tune = time.perf_counter()
+                tune(model32, x32)
+                log(f"fp32 GEMM tuning forward: {time.perf_counter() - t_tune:.1f} s")
                 t32 = time_steps(lambda: model32(x32), 3, 10) / 10
                 extra["fp32"] = dict(workload=f"VMamba-T forward, batch {args.batch} @{args.image_size}^2, fp32 activations and weights (the reference "
-                                              f"harness's precision, no AMP), eager launches, {gemm_mode.split(' picked')[0]} as met",
+                                              f"harness's precision, no AMP), eager launches, {gemm_mode}",
                                      ms_per_step=t32 * 1e3, img_per_s=args.batch / t32)
                 log("fp32:", extra["fp32"])
                 del x32, model32
