@@ -157,6 +157,29 @@ def test_vmamba_tiny_bf16_1024px_batch4():
     assert (got[True] - got[False]).abs().max().item() <= 2e-2 * scale
 
 
+@pytest.mark.parametrize("dims,ratio,d_state,size", [((128, 256, 512, 1024), 2.0, 1, 224), ((96, 192, 384, 768), 2.0, 1, 128),
+                                                     ((64, 128, 256, 512), 1.0, 4, 96)])
+def test_other_model_widths_match_reference_core(dims, ratio, d_state, size):
+    """The widths of the reference's larger models (ssm_ratio 2: up to 2048 inner channels, dt ranks up to 64) and a
+    several-state variant, one block per stage, bf16 channel-last: logits against the all-torch fp32 CPU model that
+    holds the same bf16-rounded weights."""
+    from oracle.ss2d_core_ref import TorchLayers
+    print("CASE vssm-widths", dims, ratio, d_state, size, flush=True)
+    torch.manual_seed(21)
+    cfg = dict(depths=(1, 1, 1, 1), dims=dims, d_state=d_state, ssm_ratio=ratio, num_classes=40)
+    ref = VSSM(**cfg, channel_first=True, ss2d_cls=RefSS2D, layers=TorchLayers).eval().bfloat16().float()
+    hip = VSSM(**cfg, channel_first=False).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip = hip.bfloat16().to(DEV)
+    x = torch.randn(2, 3, size, size, generator=torch.Generator().manual_seed(22)).bfloat16()
+    with torch.no_grad():
+        want = ref(x.float())
+        got = hip(x.to(DEV)).float().cpu()
+    scale = want.abs().max().item()
+    assert got.shape == (2, 40)
+    assert (got - want).abs().max().item() <= 2e-2 * scale
+
+
 def test_small_vssm_trains_on_the_gpu():
     """One training step: gradients of a small model on the GPU (HIP scan / cross-scan / cross-merge backward, torch
     autograd for the rest) against the all-torch CPU model with the same weights."""

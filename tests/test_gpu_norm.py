@@ -117,7 +117,10 @@ CF = [(2, 96, 56, 56), (2, 48, 5, 7), (3, 192, 28, 28), (2, 384, 14, 14), (2, 76
       (3, 40, 5, 5), (2, 24, 3, 3), (2, 16, 1, 2), (2, 100, 4, 4), (5, 104, 13, 4), (2, 8, 1, 1), (3, 72, 31, 1), (2, 20, 3, 3),
       (2, 384, 10, 10), (1, 192, 31, 33),
       # few channels on many positions: a workgroup with fewer threads than positions
-      (1, 16, 6, 12), (2, 8, 8, 8), (1, 24, 9, 20), (3, 8, 16, 16)]
+      (1, 16, 6, 12), (2, 8, 8, 8), (1, 24, 9, 20), (3, 8, 16, 16),
+      # rows wider than the register variants hold: the LDS-tile kernel with 8 and with 4 positions per workgroup (the
+      # 2048 inner channels of the widest reference model; a tile beyond 64 KB of LDS)
+      (2, 1600, 3, 3), (2, 2048, 7, 7), (1, 4000, 2, 5)]
 
 
 @pytest.mark.parametrize("B,C,H,W", CF)

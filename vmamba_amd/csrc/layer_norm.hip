@@ -744,12 +744,21 @@ static int launch_ln_cf_tile(const void *x, const void *w, const void *b, void *
     const int64_t n_wg = (int64_t)B * tiles;
     const size_t smem = (size_t)C * (kCfTile + 1) * sizeof(float);
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
+    // tiles beyond the default 64 KB of dynamic LDS are requested explicitly (a CU has 160 KB)
+    auto raise_limit = [&](const void *kern) {
+        return smem <= 64 * 1024 ||
+               hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+    };
     if (out_channel_last) {
-        hipLaunchKernelGGL((layer_norm_cf_kernel<in_t, w_t, out_t, true, kCfTile>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
-                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, eps);
+        auto kern = layer_norm_cf_kernel<in_t, w_t, out_t, true, kCfTile>;
+        if (!raise_limit(reinterpret_cast<const void *>(kern))) return SS2D_ELAUNCH;
+        hipLaunchKernelGGL(kern, dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const in_t *)x, (const w_t *)w, (const w_t *)b,
+                           (out_t *)y, C, L, tiles, eps);
     } else {
-        hipLaunchKernelGGL((layer_norm_cf_kernel<in_t, w_t, out_t, false, kCfTile>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
-                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, eps);
+        auto kern = layer_norm_cf_kernel<in_t, w_t, out_t, false, kCfTile>;
+        if (!raise_limit(reinterpret_cast<const void *>(kern))) return SS2D_ELAUNCH;
+        hipLaunchKernelGGL(kern, dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const in_t *)x, (const w_t *)w, (const w_t *)b,
+                           (out_t *)y, C, L, tiles, eps);
     }
     return launch_status();
 }
@@ -877,9 +886,12 @@ static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, in
     if (C <= 384) return launch_ln_cf_reg<in_t, w_t, out_t, 32, 8, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     if (C <= 768) return launch_ln_cf_reg<in_t, w_t, out_t, 16, 16, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     if (C <= 1536) return launch_ln_cf_reg<in_t, w_t, out_t, 8, 32, 48>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
-    constexpr size_t kBudget = 48 * 1024;      // very wide rows: the LDS-tile kernel
-    if ((size_t)C * 9 * sizeof(float) <= kBudget)
+    // very wide rows: the LDS-tile kernel, 8 positions per workgroup while that fits 48 KB, else 4 (up to 7800 channels
+    // in 156 KB of LDS)
+    if ((size_t)C * 9 * sizeof(float) <= 48 * 1024)
         return launch_ln_cf_tile<in_t, w_t, out_t, 8>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    if ((size_t)C * 5 * sizeof(float) <= 156 * 1024)
+        return launch_ln_cf_tile<in_t, w_t, out_t, 4>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
     return SS2D_ENOTSUP;
 }
 
