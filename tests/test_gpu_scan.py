@@ -296,13 +296,16 @@ def test_scan_errors_from_host_api():
     assert torch.equal(leaf.grad, torch.zeros_like(leaf))
 
 
-@pytest.mark.parametrize("cfg", ["stage1", "stage2", "stage3", "stage4", "n16", "hires"])
+@pytest.mark.parametrize("cfg", ["stage1", "stage2", "stage3", "stage4", "n16", "hires", "rows57x58", "rows75x75"])
 def test_full_size_properties(cfg):
     """the benchmark configurations at full size: exact scaling linearity in u, exact skip path with B=0, and a
     slice of rows against the oracle."""
     _announce("scan-full", cfg)
     batch, Dn, L, N = dict(stage1=(128, 96, 3136, 1), stage2=(128, 192, 784, 1), stage3=(128, 384, 196, 1),
-                           stage4=(128, 768, 49, 1), n16=(64, 192, 3136, 16), hires=(4, 96, 65536, 1))[cfg]
+                           stage4=(128, 768, 49, 1), n16=(64, 192, 3136, 16), hires=(4, 96, 65536, 1),
+                           # many long rows that do not start on 16-byte boundaries (the reference's 57 x 58 check size,
+                           # an odd map): walked eight rows to a wavefront as one aligned stream
+                           rows57x58=(48, 96, 3306, 1), rows75x75=(24, 192, 5625, 1))[cfg]
     K = 4
     g = torch.Generator(device=DEV).manual_seed(28)
     rn = lambda *s: torch.randn(*s, generator=g, device=DEV)
