@@ -198,14 +198,20 @@ class SS2D(nn.Module):
         K, L, R = self.k_group, H * W, self.dt_rank
         C = R + 2
         proj = torch.bmm(consts["Wx_all"], x.view(B, D, L))                                   # (B, K*C, L)
-        x_dbl = proj.new_empty((K, C, B, L))
-        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl.permute(2, 0, 1, 3))
-        dts = x_dbl[:, :R].reshape(K, R, B * L)
+        # Rows of B*L positions start on 16-byte boundaries only if B*L is a multiple of the 16-byte vector: maps with
+        # an odd (or 2, 4 mod 8) number of positions get room for a few images more, which nothing reads back --
+        # dt_proj and the kernel's delta stream then keep their 16-byte accesses.
+        vec = 16 // proj.element_size()
+        unit = vec // math.gcd(L, vec)
+        Bp = (B + unit - 1) // unit * unit
+        x_dbl = proj.new_empty((K, C, B, L)) if Bp == B else proj.new_zeros((K, C, Bp, L))
+        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl[:, :, :B].permute(2, 0, 1, 3))
+        dts = x_dbl[:, :R].reshape(K, R, Bp * L)
         if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
-            delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, B, L)
+            delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
         else:
-            delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, B, L)
-        return ss2d_core_hip(x, delta, x_dbl[:, R], x_dbl[:, R + 1], consts["As"].view(-1), consts["Ds"],
+            delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
+        return ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, R, :B], x_dbl[:, R + 1, :B], consts["As"].view(-1), consts["Ds"],
                              consts["dt_bias"], True)
 
     def _fused_core_applies(self, x):
