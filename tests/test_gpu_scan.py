@@ -305,7 +305,7 @@ def test_full_size_properties(cfg):
                            stage4=(128, 768, 49, 1), n16=(64, 192, 3136, 16), hires=(4, 96, 65536, 1),
                            # many long rows that do not start on 16-byte boundaries (the reference's 57 x 58 check size,
                            # an odd map): walked eight rows to a wavefront as one aligned stream
-                           rows57x58=(48, 96, 3306, 1), rows75x75=(24, 192, 5625, 1))[cfg]
+                           rows57x58=(48, 96, 3306, 1), rows75x75=(8, 192, 5625, 1))[cfg]
     K = 4
     g = torch.Generator(device=DEV).manual_seed(28)
     rn = lambda *s: torch.randn(*s, generator=g, device=DEV)

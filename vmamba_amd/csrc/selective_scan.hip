@@ -447,9 +447,9 @@ static bool span_fits_u32(const ScanArgs &a, int64_t elem_bytes) {
 static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
     const int64_t L = a.L, KD = a.dim;
     // rows of four passes and more only where the row kernel would fall back to element-wise accesses (the caller
-    // checks that) and there are rows enough to fill the chip eight to a wavefront (measured: 27 264 unaligned rows of
-    // 5625 positions 515 us against 1112; 512 such rows 585 against 76)
-    const bool length_ok = L < 4 * kPass || (L <= (1 << 24) && a.N == 1 && a.rows >= 16384);
+    // checks that) and there are rows enough to fill the chip eight to a wavefront (measured, unaligned bf16 rows of
+    // 5625 positions: 27 264 rows 515 us against 1112, 6144 rows 191 against 241, 3072 rows 153 against 114)
+    const bool length_ok = L < 4 * kPass || (L <= (1 << 24) && a.N == 1 && a.rows >= 6144);
     return a.x == nullptr && L >= kItems && length_ok && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
            a.u_ds == L && a.dl_ds == L && a.o_ds == L && a.u_bs == KD * L && a.dl_bs == KD * L && a.o_bs == KD * L &&
            aligned16(q->u) && aligned16(q->delta) && aligned16(q->out) &&
