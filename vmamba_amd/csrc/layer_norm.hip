@@ -821,7 +821,8 @@ static bool ln_image_plan(int B, int C, int L, size_t out_size, bool out_channel
     for (int T = 1; T <= t_max; ++T) {
         const int Qn = (Q + T - 1) / T;
         if ((Qn - 1) * T >= Q) continue;                       // an empty last share: the split of a smaller T
-        if (found && (Qn < 12 || (Qn < 24 && (int64_t)B * p.T >= 256))) break;
+        // (a tile beyond half a CU's LDS keeps the CU to one workgroup: split on until two fit)
+        if (found && p.smem <= 76 * 1024 && (Qn < 12 || (Qn < 24 && (int64_t)B * p.T >= 256))) break;
         const int positions = p.kch == 1 ? 4 * Qn : L;
         if (positions > kLnImgStat) continue;
         const size_t smem = (size_t)4 * kLnImgBlock * 4 + 2 * kLnImgStat * 4 + (size_t)2 * C * 4 +
