@@ -818,20 +818,25 @@ static bool ln_image_plan(int B, int C, int L, size_t out_size, bool out_channel
     // 192 bytes while there are fewer workgroups than CUs.
     const int t_max = p.kch == 1 ? Q : 1;
     bool found = false;
+    size_t tile_cl = 0;                                        // LDS of the plan found so far if it wrote channel-last
     for (int T = 1; T <= t_max; ++T) {
         const int Qn = (Q + T - 1) / T;
         if ((Qn - 1) * T >= Q) continue;                       // an empty last share: the split of a smaller T
-        // (a tile beyond half a CU's LDS keeps the CU to one workgroup: split on until two fit)
-        if (found && p.smem <= 76 * 1024 && (Qn < 12 || (Qn < 24 && (int64_t)B * p.T >= 256))) break;
+        // (a channel-last tile beyond half a CU's LDS keeps the CU to one workgroup, which is fine while the chip holds
+        // every workgroup at once; with more workgroups than CUs split on until two fit.  The channel-first output
+        // takes the same split, so that both layouts hold the same values bit for bit)
+        const bool one_round = tile_cl <= 76 * 1024 || (int64_t)B * p.T <= 256;
+        if (found && one_round && (Qn < 12 || (Qn < 24 && (int64_t)B * p.T >= 256))) break;
         const int positions = p.kch == 1 ? 4 * Qn : L;
         if (positions > kLnImgStat) continue;
-        const size_t smem = (size_t)4 * kLnImgBlock * 4 + 2 * kLnImgStat * 4 + (size_t)2 * C * 4 +
-                            (out_channel_last ? (size_t)positions * p.pitch_dw * 4 : 0);
+        const size_t smem_cl = (size_t)4 * kLnImgBlock * 4 + 2 * kLnImgStat * 4 + (size_t)2 * C * 4 + (size_t)positions * p.pitch_dw * 4;
+        const size_t smem = out_channel_last ? smem_cl : smem_cl - (size_t)positions * p.pitch_dw * 4;
         if (smem > 100 * 1024) continue;
         for (int ku : {8, 10}) {
             const int G = (n_units + ku - 1) / ku;
             if ((int64_t)G * Qn > kLnImgBlock) continue;
             p.ku = ku; p.T = T; p.Qn = Qn; p.G = G; p.threads = ((G * Qn + kWave - 1) / kWave) * kWave; p.smem = smem;
+            tile_cl = smem_cl;
             found = true;
             break;
         }
