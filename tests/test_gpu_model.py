@@ -180,6 +180,20 @@ def test_other_model_widths_match_reference_core(dims, ratio, d_state, size):
     assert (got - want).abs().max().item() <= 2e-2 * scale
 
 
+def test_with_layout_twin_gives_the_same_logits():
+    """A model built channel-first (what the reference's "ln2d" configurations do) and its channel-last twin: same
+    logits to the bf16 bound."""
+    print("CASE vssm-with-layout", flush=True)
+    torch.manual_seed(31)
+    cf = vmamba_tiny_s1l8(channel_first=True).eval().bfloat16().to(DEV)
+    cl = cf.with_layout(False)
+    assert next(cl.parameters()).device.type == "cuda" and next(cl.parameters()).dtype == torch.bfloat16
+    x = torch.randn(3, 3, 224, 224, device=DEV).bfloat16()
+    with torch.no_grad():
+        a, b = cf(x).float(), cl(x).float()
+    assert (a - b).abs().max().item() <= 2e-2 * a.abs().max().item()
+
+
 def test_small_vssm_trains_on_the_gpu():
     """One training step: gradients of a small model on the GPU (HIP scan / cross-scan / cross-merge backward, torch
     autograd for the rest) against the all-torch CPU model with the same weights."""

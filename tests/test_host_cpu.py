@@ -130,3 +130,20 @@ def test_inference_constants_are_kept_per_batch_size_and_follow_the_parameters()
         assert fresh is not c2 and torch.equal(fresh["As"], -m.A_logs.float().exp())
         assert all(k[0] == 2 for k in m._const_cache)
     assert m._inference_constants(2) is not m._inference_constants(2)      # under autograd nothing is kept
+
+
+def test_with_layout_keeps_keys_values_and_mode():
+    """VSSM.with_layout: the channel-last twin of a channel-first model holds the same state_dict (names, shapes, values)
+    -- a Linear2d weight (out, in, 1, 1) and the nn.Linear weight (out, in) are one tensor viewed two ways
+    (vmamba.py:47-49) -- and converts back."""
+    from vmamba_amd.vssm import VSSM
+    torch.manual_seed(3)
+    m = VSSM(depths=(1, 1, 1, 1), dims=(16, 32, 64, 128), d_state=2, ssm_ratio=2.0, num_classes=10, channel_first=True).eval()
+    twin = m.with_layout(False)
+    assert not twin.training and twin.layers[0].blocks[0].op.channel_first is False
+    sd, sd2 = m.state_dict(), twin.state_dict()
+    assert list(sd) == list(sd2)
+    for k in sd:
+        assert sd[k].numel() == sd2[k].numel() and torch.equal(sd[k].reshape(-1), sd2[k].reshape(-1)), k
+    back = twin.with_layout(True).state_dict()
+    assert all(back[k].shape == sd[k].shape and torch.equal(back[k], sd[k]) for k in sd)

@@ -170,6 +170,8 @@ class VSSM(nn.Module):
     def __init__(self, in_chans=3, num_classes=1000, depths=(2, 2, 8, 2), dims=(96, 192, 384, 768), d_state=1,
                  ssm_ratio=1.0, mlp_ratio=4.0, ss2d_cls=SS2D, channel_first=True, layers=HipLayers, **ss2d_kwargs):
         super().__init__()
+        self._build_args = dict(in_chans=in_chans, num_classes=num_classes, depths=tuple(depths), dims=tuple(dims), d_state=d_state,
+                                ssm_ratio=ssm_ratio, mlp_ratio=mlp_ratio, ss2d_cls=ss2d_cls, layers=layers, **ss2d_kwargs)
         cf = channel_first
         Norm = layers.LayerNorm2d if cf else layers.LayerNorm
         d0 = dims[0]
@@ -223,6 +225,17 @@ class VSSM(nn.Module):
         for layer in self.layers:
             x = layer(x)
         return self.classifier(x)
+
+    def with_layout(self, channel_first):
+        """The same model (a copy of the weights, same device, dtype and mode) with its blocks in the other activation
+        layout.  The reference's "ln2d" configurations build channel-first blocks (vmamba.py:1281); the two layouts
+        compute the same function and share one state_dict (a Linear2d weight is a view of the nn.Linear one, vmamba.py:
+        47-49), and the channel-last build is the one whose projections, MLPs and LayerNorms run on this package's fused
+        kernels."""
+        twin = VSSM(channel_first=channel_first, **self._build_args)
+        twin.load_state_dict(self.state_dict())
+        p = next(self.parameters())
+        return twin.to(device=p.device, dtype=p.dtype).train(self.training)
 
 
 def vmamba_tiny_s1l8(channel_first=True, **kwargs):
