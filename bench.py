@@ -602,8 +602,19 @@ def main():
                 model(x4)
                 tune(model, x4)
                 t4 = time_steps(lambda: model(x4), 5, 10) / 10
-                extra["config4"] = dict(workload="VMamba-T forward, 4 x 1024^2, bf16, eager launches (stage maps 256/128/64/32)",
+                extra["config4"] = dict(workload="VMamba-T forward, 4 x 1024^2, bf16 (stage maps 256/128/64/32); ms_per_forward = eager "
+                                                 "launches (four images leave them bound by the host's launch rate), "
+                                                 "ms_per_forward_one_graph = the forward replayed as one captured HIP graph",
                                         ms_per_forward=t4 * 1e3, img_per_s=4 / t4)
+                if not args.eager:
+                    try:
+                        captured4 = capture_forward(model, x4)
+                        if captured4 is not None:
+                            t4g = time_steps(captured4[0].replay, 5, 10) / 10
+                            extra["config4"].update(ms_per_forward_one_graph=t4g * 1e3, img_per_s_one_graph=4 / t4g)
+                        captured4 = None
+                    except Exception as e:
+                        log(f"config-4 graph capture failed ({type(e).__name__}: {e})")
                 log("config 4:", extra["config4"])
                 del x4
             except Exception as e:
