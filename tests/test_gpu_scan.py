@@ -296,6 +296,21 @@ def test_scan_errors_from_host_api():
     assert torch.equal(leaf.grad, torch.zeros_like(leaf))
 
 
+@pytest.mark.parametrize("batch,dim,G,L,dtype", [(16, 384, 4, 2051, torch.bfloat16), (24, 256, 4, 2307, torch.float32),
+                                                 (13, 512, 2, 2049, torch.float16)])
+def test_many_long_rows_off_the_vector_grid(batch, dim, G, L, dtype):
+    """6144 rows and more of odd length (no row but the first starts on a 16-byte boundary): the library walks them eight
+    to a wavefront as one aligned stream.  Every row against the oracle; with chunk states requested the row kernel
+    runs instead and must agree too."""
+    _announce("scan-long-unaligned", batch, dim, G, L, dtype)
+    args = make_inputs(batch * 1000 + L, batch, dim, G, 1, L, dtype, ss2d_like=True)
+    want = orc.selective_scan(*args, True, out_float=True)
+    for want_x in (False, True):
+        got, _ = run_gpu(*args, True, True, want_x=want_x)
+        bound = 2e-4 + 1e-3 * want.abs() + 5e-5 * want.abs().amax(dim=-1, keepdim=True)
+        assert bool(((got - want).abs() <= bound).all()), (want_x, (got - want).abs().max().item())
+
+
 @pytest.mark.parametrize("cfg", ["stage1", "stage2", "stage3", "stage4", "n16", "hires", "rows57x58", "rows75x75"])
 def test_full_size_properties(cfg):
     """the benchmark configurations at full size: exact scaling linearity in u, exact skip path with B=0, and a
