@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
     }
 }
 
-// Image variant for fp32 channel-first input of SHORT images (7 x 7 ... 28 x 28 maps): the tile kernels above cut an
+// Image variant for channel-first input (fp32, or 16-bit with 8-byte vectors) of SHORT images (7 x 7 ... 28 x 28 maps): the tile kernels above cut an
 // image into pieces of 16 or 32 positions, i.e. 64- or 128-byte runs per channel row, and on short rows that is what
 // they are bound by.  Here a workgroup of up to 1024 threads takes a whole image, or a 1/T share of its positions, and
 // reads it as 16-byte vectors of ONE flat stream:
@@ -516,8 +516,8 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
 constexpr int kLnImgBlock = 1024;
 constexpr int kLnImgStat = 256;                      // positions per workgroup at most
 
-template <typename w_t, typename out_t, bool kOutChannelLast, int kCh, int kU>
-__global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const float *__restrict__ x, const w_t *__restrict__ weight,
+template <typename in_t, typename w_t, typename out_t, bool kOutChannelLast, int kCh, int kU>
+__global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const in_t *__restrict__ x, const w_t *__restrict__ weight,
                                                                           const w_t *__restrict__ bias, out_t *__restrict__ y, int C,
                                                                           int L, int T, int Qn, int G, int pitch_dw, float eps) {
     static_assert(kCh == 1 || kCh == 4, "a unit is one channel row or four");
@@ -548,8 +548,8 @@ __global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const 
         }
     }
     const int n_valid = lane_on ? min(max(n_units - g * kU, 0), kU) : 0;       // units this lane really holds
-    const float *xb = x + (size_t)b * C * L;
-    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(xb), 0, C * L * 4, 0x00020000);
+    const in_t *xb = x + (size_t)b * C * L;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<in_t *>(xb), 0, C * L * (int)sizeof(in_t), 0x00020000);
 
     float v[kU][4];
     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -557,10 +557,19 @@ __global__ __launch_bounds__(kLnImgBlock) void layer_norm_cf_image_kernel(const 
     for (int n = 0; n < kU; ++n) {
         const int unit = g * kU + n;
         // idle lanes and units past the last point past the end of the buffer, where the hardware returns 0
-        const uint32_t off = n < n_valid ? (uint32_t)(unit * Q + q0 + q) * 16u : 0x7ffffff0u;
-        const auto r = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+        // (a vector is four positions: 16 bytes of fp32 input, 8 bytes of 16-bit input)
+        const uint32_t off = n < n_valid ? (uint32_t)(unit * Q + q0 + q) * (4u * (uint32_t)sizeof(in_t)) : 0x7ffffff0u;
+        if constexpr (sizeof(in_t) == 4) {
+            const auto r = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { v[n][j] = bits_to_f32(r[j]); s[j] += v[n][j]; }
+            for (int j = 0; j < 4; ++j) v[n][j] = bits_to_f32(r[j]);
+        } else {
+            const auto r = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, (int)off, 0, 0);
+            v[n][0] = unpack_lo<in_t>(r[0]); v[n][1] = unpack_hi<in_t>(r[0]);
+            v[n][2] = unpack_lo<in_t>(r[1]); v[n][3] = unpack_hi<in_t>(r[1]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[j] += v[n][j];
     }
     // weight and bias wait in LDS (read after the barriers of the two reductions)
     for (int c = t; c < C; c += (int)blockDim.x) {
@@ -844,18 +853,18 @@ static bool ln_image_plan(int B, int C, int L, size_t out_size, bool out_channel
     return found;
 }
 
-template <typename w_t, typename out_t>
+template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_cf_image(const LnImagePlan &p, const void *x, const void *w, const void *b, void *y, int B, int C, int L,
                               float eps, int out_channel_last, hipStream_t stream) {
     const int64_t n_wg = (int64_t)B * p.T;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
 #define SS2D_LN_IMAGE(CL, KCH, KU)                                                                                              \
     {                                                                                                                            \
-        auto kern = layer_norm_cf_image_kernel<w_t, out_t, CL, KCH, KU>;                                                         \
+        auto kern = layer_norm_cf_image_kernel<in_t, w_t, out_t, CL, KCH, KU>;                                                   \
         if (p.smem > 64 * 1024 &&                                                                                                \
             hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)p.smem) != hipSuccess) \
             return SS2D_ELAUNCH;                                                                                                 \
-        hipLaunchKernelGGL(kern, dim3((uint32_t)n_wg), dim3(p.threads), p.smem, stream, (const float *)x, (const w_t *)w,        \
+        hipLaunchKernelGGL(kern, dim3((uint32_t)n_wg), dim3(p.threads), p.smem, stream, (const in_t *)x, (const w_t *)w,         \
                            (const w_t *)b, (out_t *)y, C, L, p.T, p.Qn, p.G, p.pitch_dw, eps);                                   \
     }
     if (out_channel_last) {
@@ -872,11 +881,13 @@ static int launch_ln_cf_image(const LnImagePlan &p, const void *x, const void *w
 template <typename in_t, typename w_t, typename out_t>
 static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
                         int out_channel_last, hipStream_t stream) {
-    if constexpr (sizeof(in_t) == 4) {
+    {
         // short images: a whole image, or an even share of one, per workgroup
         LnImagePlan plan;
         if (L <= 1024 && ln_aligned16(x) && ln_aligned16(y) && ln_image_plan(B, C, L, sizeof(out_t), out_channel_last != 0, plan))
-            return launch_ln_cf_image<w_t, out_t>(plan, x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            return launch_ln_cf_image<in_t, w_t, out_t>(plan, x, w, b, y, B, C, L, eps, out_channel_last, stream);
+    }
+    if constexpr (sizeof(in_t) == 4) {
         // fp32 input, quads of positions: 16-byte loads (and 16-byte channel-last stores)
         const bool quad_ok = L % 4 == 0 && ln_aligned16(x) && (int64_t)C * L * 4 < 0x7ffffff0ll && (int64_t)B * ((L + 15) / 16) <= 0x7fffffff &&
                              (out_channel_last ? (C % (16 / (int)sizeof(out_t)) == 0 && ln_aligned16(y)) : ln_aligned16(y));
