@@ -342,7 +342,8 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
                                                                   const T *__restrict__ bias, T *__restrict__ y, int D, int H,
                                                                   int W, int TH, int row_tiles, int ch_tiles, int col_tiles,
                                                                   int TW, int pitch, int plane_dw, int nseg, int n_it,
-                                                                  int flat_out, FastDiv divHalf, FastDiv divNseg) {
+                                                                  int flat_out, int in_channel_first, FastDiv divHalf,
+                                                                  FastDiv divNseg, FastDiv divItems) {
     constexpr int kLpc = kBlock / kCh;                           // lanes per channel in the compute phase
     constexpr int kCv = kCh / 8;                                 // 16-byte channel vectors per position
     constexpr int kPer = kBlock / kCv;                           // position pairs per staging pass
@@ -371,7 +372,36 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_planes_kernel(const T *__res
     const float bv = bias ? to_f32(bias[c]) : 0.0f;
 
     // ---- staging: rows h0-1 .. h0+rows of kCh channels into the planes, zeros outside the image
-    {
+    if (in_channel_first) {
+        // x (B, D, H, W): a plane dword is two neighbouring elements of a channel's row, starting at an odd column
+        // (padded column 0 is image column -1), so the pair is put together from two 16-bit loads; consecutive lanes
+        // take consecutive dwords of a plane.  kAhead dwords per lane are requested before the first is parked.
+        constexpr int kAhead = 4;
+        const T *xb = x + ((size_t)b * D + c_base) * H * W;
+        // (planes are indexed as for a full tile of TH rows; a short last tile leaves the lanes of its missing rows idle)
+        const int n_items = (rows + 2) * half, total = kCh * (TH + 2) * half;
+        for (int i0 = threadIdx.x; i0 < total; i0 += kAhead * kBlock) {
+            uint32_t lo[kAhead], hi[kAhead];
+            int dst[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int idx = min(i0 + u * kBlock, total - 1);
+                uint32_t pc, q, rr, pp;
+                divmod((uint32_t)idx, divItems, pc, q);
+                divmod(q, divHalf, rr, pp);
+                const int h = h0 - 1 + (int)rr, w0 = wb + 2 * (int)pp - 1, w1 = w0 + 1;
+                const bool row_ok = h >= 0 && h < H && (int)q < n_items;
+                const T *src = xb + ((size_t)pc * H + (row_ok ? h : 0)) * W;
+                const bool ok0 = row_ok && w0 >= 0 && w0 < W, ok1 = row_ok && w1 < W;
+                lo[u] = src[ok0 ? w0 : 0].bits; hi[u] = src[ok1 ? w1 : 0].bits;
+                lo[u] = ok0 ? lo[u] : 0u; hi[u] = ok1 ? hi[u] : 0u;
+                dst[u] = (int)q < n_items ? plane_at((int)pc, plane_dw) + (int)q : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u)
+                if (i0 + u * kBlock < total && dst[u] >= 0) dwp_smem[dst[u]] = lo[u] | (hi[u] << 16);
+        }
+    } else {
         const int cv = threadIdx.x % kCv;
         const int c0 = c_base + cv * 8;
         const T *xb = x + (size_t)b * H * W * D;
@@ -621,7 +651,8 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
         if (W > 120 && W % 8 == 0)
             for (int n = kBlock / (D % 64 == 0 ? 64 : 32); n >= 4 && seg_t == 0; --n)
                 if ((W / 8) % n == 0) seg_t = n;
-        if (in_channel_last && D % 32 == 0 && (W <= 120 || seg_t > 0) && al16(x) && al16(y) &&
+        // (channel-first input takes the same kernel with element-wise staging: no alignment asked of x)
+        if (D % 32 == 0 && (W <= 120 || seg_t > 0) && (al16(x) || !in_channel_last) && al16(y) &&
             (int64_t)H * W * D * 2 < 0x7ffffff0ll) {
             const int kch = D % 64 == 0 ? 64 : 32, lpc = kBlock / kch;
             const int TW = seg_t > 0 ? 8 * seg_t : W, col_tiles = seg_t > 0 ? W / TW : 1;
@@ -641,7 +672,8 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
 #define SS2D_DW_PLANES(SILU, KCH)                                                                                              \
     hipLaunchKernelGGL((dwconv3x3_planes_kernel<T, SILU, KCH>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, (const T *)x,  \
                        (const T *)w, (const T *)bias, (T *)y, D, H, W, TH, row_tiles, ch_tiles, col_tiles, TW, pitch, plane_dw,  \
-                       nseg, n_it, flat_out, make_fastdiv((uint32_t)(pitch / 2)), make_fastdiv((uint32_t)nseg))
+                       nseg, n_it, flat_out, in_channel_last ? 0 : 1, make_fastdiv((uint32_t)(pitch / 2)),                     \
+                       make_fastdiv((uint32_t)nseg), make_fastdiv((uint32_t)((TH + 2) * (pitch / 2))))
                 if (kch == 64) { if (apply_silu) SS2D_DW_PLANES(true, 64); else SS2D_DW_PLANES(false, 64); }
                 else { if (apply_silu) SS2D_DW_PLANES(true, 32); else SS2D_DW_PLANES(false, 32); }
 #undef SS2D_DW_PLANES
