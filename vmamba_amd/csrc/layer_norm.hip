@@ -376,13 +376,14 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_reg_kernel(const in_t *_
     }
 }
 
-// Quad variant of the register kernel for fp32 channel-first input (the merged scan output feeding out_norm): a lane
-// owns FOUR consecutive positions, so every load is 16 bytes (the address pipeline is priced per instruction, and the
+// Quad variant of the register kernel for channel-first input (fp32: the merged scan output feeding out_norm; 16-bit:
+// LayerNorm2d on activations): a lane owns FOUR consecutive positions, so every load is 16 bytes (8 of 16-bit input;
+// the address pipeline is priced per instruction, and the
 // 4-byte loads of the variant above leave it the bottleneck on short images).  Threads are laid out quads x groups;
 // group g holds channels g, g+kG, ... of its four positions.  Sums cross the groups of a wavefront by lane
 // exchanges and the wavefronts through a few floats of LDS.
-template <typename w_t, typename out_t, bool kOutChannelLast, int kQ, int kG, int kCPL>
-__global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float *__restrict__ x, const w_t *__restrict__ weight,
+template <typename in_t, typename w_t, typename out_t, bool kOutChannelLast, int kQ, int kG, int kCPL>
+__global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const in_t *__restrict__ x, const w_t *__restrict__ weight,
                                                                     const w_t *__restrict__ bias, out_t *__restrict__ y, int C,
                                                                     int L, int tiles_per_image, int Cp, float eps) {
     static_assert(kQ * kG == kBlock && kQ <= kWave, "one thread per (position quad, group)");
@@ -396,8 +397,8 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
     const int wave = threadIdx.x / kWave;
     const int l = l0 + 4 * q;
     const bool valid = l < L;                        // L % 4 == 0 (host-checked): a quad is inside or outside
-    const float *xb = x + (size_t)b * C * L;
-    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(xb), 0, C * L * 4, 0x00020000);
+    const in_t *xb = x + (size_t)b * C * L;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<in_t *>(xb), 0, C * L * (int)sizeof(in_t), 0x00020000);
 
     float v[kCPL][4];
     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -405,10 +406,18 @@ __global__ __launch_bounds__(kBlock) void layer_norm_cf_quad_kernel(const float 
     for (int i = 0; i < kCPL; ++i) {
         const int c = g + i * kG;
         // outside the image: pointed past the end of the buffer, where the hardware returns 0 (loads stay unconditional)
-        const uint32_t off = (valid && c < C) ? (uint32_t)(c * L + l) * 4u : 0x7ffffff0u;
-        const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
+        const uint32_t off = (valid && c < C) ? (uint32_t)(c * L + l) * (uint32_t)sizeof(in_t) : 0x7ffffff0u;
+        if constexpr (sizeof(in_t) == 4) {
+            const auto t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { v[i][j] = bits_to_f32(t[j]); s[j] += v[i][j]; }
+            for (int j = 0; j < 4; ++j) v[i][j] = bits_to_f32(t[j]);
+        } else {
+            const auto t = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, (int)off, 0, 0);
+            v[i][0] = unpack_lo<in_t>(t[0]); v[i][1] = unpack_hi<in_t>(t[0]);
+            v[i][2] = unpack_lo<in_t>(t[1]); v[i][3] = unpack_hi<in_t>(t[1]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[j] += v[i][j];
     }
     auto reduce_groups = [&](float (&acc)[4], int which) {
 #pragma unroll
@@ -792,7 +801,7 @@ static int launch_ln_cf_reg(const void *x, const void *w, const void *b, void *y
     return launch_status();
 }
 
-template <typename w_t, typename out_t, int kQ, int kG, int kCPL>
+template <typename in_t, typename w_t, typename out_t, int kQ, int kG, int kCPL>
 static int launch_ln_cf_quad(const void *x, const void *w, const void *b, void *y, int B, int C, int L, float eps,
                              int out_channel_last, hipStream_t stream) {
     constexpr int kTP = 4 * kQ;
@@ -803,11 +812,11 @@ static int launch_ln_cf_quad(const void *x, const void *w, const void *b, void *
     const int Cp = ((C + piece - 1) / piece) * piece + piece;
     if (out_channel_last) {
         const size_t smem = (size_t)kTP * Cp * sizeof(out_t);
-        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<w_t, out_t, true, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
-                           stream, (const float *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<in_t, w_t, out_t, true, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), smem,
+                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
     } else {
-        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<w_t, out_t, false, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), 0,
-                           stream, (const float *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
+        hipLaunchKernelGGL((layer_norm_cf_quad_kernel<in_t, w_t, out_t, false, kQ, kG, kCPL>), dim3((uint32_t)n_wg), dim3(kBlock), 0,
+                           stream, (const in_t *)x, (const w_t *)w, (const w_t *)b, (out_t *)y, C, L, tiles, Cp, eps);
     }
     return launch_status();
 }
@@ -887,15 +896,15 @@ static int launch_ln_cf(const void *x, const void *w, const void *b, void *y, in
         if (L <= 1024 && ln_aligned16(x) && ln_aligned16(y) && ln_image_plan(B, C, L, sizeof(out_t), out_channel_last != 0, plan))
             return launch_ln_cf_image<in_t, w_t, out_t>(plan, x, w, b, y, B, C, L, eps, out_channel_last, stream);
     }
-    if constexpr (sizeof(in_t) == 4) {
-        // fp32 input, quads of positions: 16-byte loads (and 16-byte channel-last stores)
+    {
+        // quads of positions: 16-byte loads of fp32 input, 8-byte loads of 16-bit input (and 16-byte channel-last stores)
         const bool quad_ok = L % 4 == 0 && ln_aligned16(x) && (int64_t)C * L * 4 < 0x7ffffff0ll && (int64_t)B * ((L + 15) / 16) <= 0x7fffffff &&
                              (out_channel_last ? (C % (16 / (int)sizeof(out_t)) == 0 && ln_aligned16(y)) : ln_aligned16(y));
         if (quad_ok) {
-            if (C <= 96) return launch_ln_cf_quad<w_t, out_t, 16, 16, 6>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
-            if (C <= 192) return launch_ln_cf_quad<w_t, out_t, 16, 16, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
-            if (C <= 384) return launch_ln_cf_quad<w_t, out_t, 8, 32, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
-            if (C <= 768) return launch_ln_cf_quad<w_t, out_t, 4, 64, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 96) return launch_ln_cf_quad<in_t, w_t, out_t, 16, 16, 6>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 192) return launch_ln_cf_quad<in_t, w_t, out_t, 16, 16, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 384) return launch_ln_cf_quad<in_t, w_t, out_t, 8, 32, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
+            if (C <= 768) return launch_ln_cf_quad<in_t, w_t, out_t, 4, 64, 12>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
         }
     }
     if (C <= 96) return launch_ln_cf_reg<in_t, w_t, out_t, 64, 4, 24>(x, w, b, y, B, C, L, eps, out_channel_last, stream);
