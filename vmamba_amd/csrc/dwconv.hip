@@ -606,6 +606,60 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_cl2cf_f32_kernel(const float
     }
 }
 
+// fp32, channel-first input (the reference harness's own precision and layout), W a multiple of 4, 16-byte aligned maps:
+// four consecutive outputs of a row per lane from three 16-byte row loads and the six neighbours either side -- a
+// quarter of the load instructions of the one-output-per-lane kernel below, 16-byte stores.  Same arithmetic as that
+// kernel: taps accumulated in (kh, kw) order with fused multiply-adds, bias added last, exact SiLU.
+template <bool kSilu>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_cf_f32_kernel(const float *__restrict__ x, const float *__restrict__ weight,
+                                                                  const float *__restrict__ bias, float *__restrict__ y, int D, int H,
+                                                                  int W, int64_t total_quads, FastDiv divD) {
+    const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;     // over (b, d, h, w / 4)
+    if (idx >= total_quads) return;
+    const int Wq = W / 4;
+    const int64_t rows_idx = idx / Wq;                                  // (b, d, h)
+    const int wq = (int)(idx - rows_idx * Wq);
+    const uint32_t map = (uint32_t)(rows_idx / H);
+    const int h = (int)(rows_idx - (int64_t)map * H);
+    uint32_t b, d;
+    divmod(map, divD, b, d);
+    (void)b;
+    const float *xm = x + (size_t)map * H * W;
+    float wt[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) wt[t] = weight[(size_t)d * 9 + t];
+    const int w0 = 4 * wq;
+    float in[3][6];
+    bool row_in[3];
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh) {
+        const int hh = h + kh - 1;
+        row_in[kh] = hh >= 0 && hh < H;
+        const float *row = xm + (size_t)(row_in[kh] ? hh : h) * W;
+        const float4 m = *reinterpret_cast<const float4 *>(row + w0);
+        in[kh][0] = w0 > 0 ? row[w0 - 1] : 0.0f;
+        in[kh][1] = m.x; in[kh][2] = m.y; in[kh][3] = m.z; in[kh][4] = m.w;
+        in[kh][5] = w0 + 4 < W ? row[w0 + 4] : 0.0f;
+    }
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+            if (row_in[kh]) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int ww = w0 + j + kw - 1;
+                    if (ww >= 0 && ww < W) acc[j] = fmaf(wt[kh * 3 + kw], in[kh][j + kw], acc[j]);
+                }
+            }
+    const float bv = bias ? bias[d] : 0.0f;
+    float o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { o[j] = acc[j] + bv; if (kSilu) o[j] = silu_f32(o[j]); }
+    *reinterpret_cast<float4 *>(y + (size_t)rows_idx * W + w0) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
 // Generic variant: any element type, either input layout, one output element per lane (lanes along W).
 template <typename T, bool kInChannelLast, bool kSilu>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_generic_kernel(const T *__restrict__ x, const T *__restrict__ weight,
@@ -738,6 +792,22 @@ static int launch_dwconv(const void *x, const void *w, const void *bias, void *y
                     hipLaunchKernelGGL((dwconv3x3_cl2cf_f32_kernel<false>), dim3((uint32_t)n_tiles), dim3(kBlock), 0, stream,
                                        (const float *)x, (const float *)w, (const float *)bias, (float *)y, D, H, W, pos_tiles,
                                        ch_tiles, make_fastdiv((uint32_t)W));
+                }
+                return launch_status();
+            }
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        if (!in_channel_last && W % 4 == 0 && al16(x) && al16(y) && (int64_t)B * D <= 0x7fffffff) {
+            const int64_t quads = (int64_t)B * D * H * (W / 4);
+            const int64_t n_q = (quads + kBlock - 1) / kBlock;
+            if (n_q <= 0x7fffffff) {
+                if (apply_silu) {
+                    hipLaunchKernelGGL((dwconv3x3_cf_f32_kernel<true>), dim3((uint32_t)n_q), dim3(kBlock), 0, stream, (const float *)x,
+                                       (const float *)w, (const float *)bias, (float *)y, D, H, W, quads, make_fastdiv((uint32_t)D));
+                } else {
+                    hipLaunchKernelGGL((dwconv3x3_cf_f32_kernel<false>), dim3((uint32_t)n_q), dim3(kBlock), 0, stream, (const float *)x,
+                                       (const float *)w, (const float *)bias, (float *)y, D, H, W, quads, make_fastdiv((uint32_t)D));
                 }
                 return launch_status();
             }
