@@ -631,6 +631,18 @@ def main():
                                               f"harness's precision, no AMP), eager launches, {gemm_mode}",
                                      ms_per_step=t32 * 1e3, img_per_s=args.batch / t32)
                 log("fp32:", extra["fp32"])
+                if args.layout != "channel_first" and hasattr(model32, "with_layout"):
+                    # the reference's own "ln2d" build of the model (channel-first blocks, Linear2d = 1x1 convolutions) in
+                    # fp32: the configuration its published throughput figures were taken in
+                    model_cf = model32.with_layout(True)
+                    model_cf(x32)
+                    tcf = time_steps(lambda: model_cf(x32), 2, 5) / 5
+                    extra["fp32_channel_first"] = dict(
+                        workload=f"VMamba-T forward, batch {args.batch} @{args.image_size}^2, fp32, channel-first blocks (the reference's "
+                                 f"ln2d configuration, vmamba.py:1281), eager launches",
+                        ms_per_step=tcf * 1e3, img_per_s=args.batch / tcf)
+                    log("fp32 channel-first:", extra["fp32_channel_first"])
+                    del model_cf
                 del x32, model32
             except Exception as e:
                 log(f"fp32 forward failed ({type(e).__name__}: {e})")
