@@ -189,9 +189,11 @@ def test_with_layout_twin_gives_the_same_logits():
     cl = cf.with_layout(False)
     assert next(cl.parameters()).device.type == "cuda" and next(cl.parameters()).dtype == torch.bfloat16
     x = torch.randn(3, 3, 224, 224, device=DEV).bfloat16()
+    shared = cf.with_layout(False, share_weights=True)
     with torch.no_grad():
-        a, b = cf(x).float(), cl(x).float()
+        a, b, c = cf(x).float(), cl(x).float(), shared(x).float()
     assert (a - b).abs().max().item() <= 2e-2 * a.abs().max().item()
+    assert torch.equal(b, c)                                       # same weights, same kernels
 
 
 def test_small_vssm_trains_on_the_gpu():

@@ -147,3 +147,12 @@ def test_with_layout_keeps_keys_values_and_mode():
         assert sd[k].numel() == sd2[k].numel() and torch.equal(sd[k].reshape(-1), sd2[k].reshape(-1)), k
     back = twin.with_layout(True).state_dict()
     assert all(back[k].shape == sd[k].shape and torch.equal(back[k], sd[k]) for k in sd)
+    # shared weights: the same Parameter objects under the same names; a change through one model is seen by the other
+    shared = m.with_layout(False, share_weights=True)
+    for (k, p), (k2, p2) in zip(m.named_parameters(), shared.named_parameters()):
+        assert k == k2 and p is p2
+    with torch.no_grad():
+        m.classifier.head.weight.mul_(2.0)
+    assert shared.classifier.head.weight is m.classifier.head.weight
+    m.double()
+    assert next(shared.parameters()).dtype == torch.float64

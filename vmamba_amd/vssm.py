@@ -226,16 +226,28 @@ class VSSM(nn.Module):
             x = layer(x)
         return self.classifier(x)
 
-    def with_layout(self, channel_first):
-        """The same model (a copy of the weights, same device, dtype and mode) with its blocks in the other activation
-        layout.  The reference's "ln2d" configurations build channel-first blocks (vmamba.py:1281); the two layouts
-        compute the same function and share one state_dict (a Linear2d weight is a view of the nn.Linear one, vmamba.py:
-        47-49), and the channel-last build is the one whose projections, MLPs and LayerNorms run on this package's fused
-        kernels."""
+    def with_layout(self, channel_first, share_weights=False):
+        """The same model (same device, dtype and mode) with its blocks in the other activation layout.  The reference's
+        "ln2d" configurations build channel-first blocks (vmamba.py:1281); the two layouts compute the same function and
+        share one state_dict (a Linear2d weight is a view of the nn.Linear one, vmamba.py:47-49), and the channel-last
+        build is the one whose projections, MLPs and LayerNorms run on this package's fused kernels.
+
+        The twin holds a copy of the weights, or -- ``share_weights=True`` -- the very same Parameter and buffer objects
+        (every parameter has the same shape in both builds), so that loading, casting, moving or training either model
+        is seen by the other."""
         twin = VSSM(channel_first=channel_first, **self._build_args)
-        twin.load_state_dict(self.state_dict())
-        p = next(self.parameters())
-        return twin.to(device=p.device, dtype=p.dtype).train(self.training)
+        if not share_weights:
+            twin.load_state_dict(self.state_dict())
+            p = next(self.parameters())
+            return twin.to(device=p.device, dtype=p.dtype).train(self.training)
+        mine = dict(self.named_modules())
+        for name, module in twin.named_modules():
+            src = mine[name]
+            for key in list(module._parameters):
+                module._parameters[key] = src._parameters[key]
+            for key in list(module._buffers):
+                module._buffers[key] = src._buffers[key]
+        return twin.train(self.training)
 
 
 def vmamba_tiny_s1l8(channel_first=True, **kwargs):
