@@ -89,7 +89,10 @@ def kernel_lines(reps):
     benchmark config 3 / config 4 operator shapes."""
     import torch
     import vmamba_amd as va
+    from vmamba_amd import oflex_ext
     from vmamba_amd.core import core_fits, dt_proj_hip, ss2d_core_hip
+    from vmamba_amd.csms6s import scan_kernel_name
+    ext = oflex_ext.load()
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(0)
     out = []
@@ -113,6 +116,10 @@ def kernel_lines(reps):
         E = B * D * L
         t_cs = time_op(lambda: va.cross_scan_fn(x), reps)
         t_sc = time_op(lambda: va.selective_scan_fn(u, delta, A, Bm, Cm, Dv, bias, True), reps)
+        # the same scan through the reference's extension interface, which always returns the chunk states too
+        # (out, x = selective_scan_cuda_oflex.fwd(...), classification/models/csms6s.py:81)
+        t_ext = time_op(lambda: ext.fwd(u, delta, A, Bm, Cm, Dv, bias, True, 1, True), reps)
+        scan_kernel = scan_kernel_name(u, delta, A, Bm, Cm, ys, torch.empty(B, K * D, (L + 2047) // 2048, 2 * N, device=dev))
         t_cm = time_op(lambda: va.cross_merge_fn(ys5), reps)
         b_cs, b_sc, b_cm = 5 * E * 2, scan_bytes(B, K * D, L, N, K, 2, 4), 5 * E * 4
         fused = {}
@@ -191,7 +198,8 @@ def kernel_lines(reps):
                 del img
         out.append(dict(shape=name, B=B, D=D, H=H, W=W, N=N,
                         cross_scan_us=t_cs * 1e6, cross_scan_GBs=b_cs / t_cs / 1e9,
-                        scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9,
+                        scan_us=t_sc * 1e6, scan_GBs=b_sc / t_sc / 1e9, scan_kernel=scan_kernel,
+                        ext_fwd_us=t_ext * 1e6, ext_fwd_GBs=b_sc / t_ext / 1e9, ext_fwd_over_fn=t_ext / t_sc,
                         cross_merge_us=t_cm * 1e6, cross_merge_GBs=b_cm / t_cm / 1e9,
                         core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
                         scan_bytes=b_sc, **fused))

@@ -120,6 +120,21 @@ typedef struct ss2d_scan_params {
 int ss2d_selective_scan_fwd(const ss2d_scan_params *params, void *stream);
 
 /*
+ * Which kernel ss2d_selective_scan_fwd would launch for `params` (the same validation, nothing is launched):
+ * one of the ids below, or a negative SS2D_E* code.  Every kernel writes `x` when it is requested, so the answer
+ * does not depend on params->x.  No counterpart in the reference (its one kernel template serves every shape,
+ * selective_scan_oflex.cpp:224-226); here so that a caller, a benchmark or a test can tell which code path a
+ * shape takes.
+ */
+#define SS2D_SCAN_KERNEL_NONE 0  /* empty problem: nothing to launch                                           */
+#define SS2D_SCAN_KERNEL_ROW 1   /* one wavefront per (batch, channel) row                                       */
+#define SS2D_SCAN_KERNEL_ROW4 2  /* few long rows: the four wavefronts of a workgroup share a row                */
+#define SS2D_SCAN_KERNEL_FLAT 3  /* short or unaligned rows walked several to a wavefront as one stream          */
+#define SS2D_SCAN_KERNEL_SMALL 4 /* rows of 49 / 196 positions, one state: a segment of a row per lane           */
+#define SS2D_SCAN_KERNEL_CHAN 5  /* several states per channel: one channel per lane, positions walked serially  */
+int ss2d_selective_scan_kernel(const ss2d_scan_params *params);
+
+/*
  * Selective-scan backward.  Replaces selective_scan_bwd + selective_scan_bwd_kernel
  * (kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:233-355,
  *  .../selective_scan_bwd_kernel_oflex.cuh); inputs as in the forward plus

@@ -90,6 +90,42 @@ def test_scan_argument_validation():
     assert L.ss2d_selective_scan_fwd(p, None) == _lib.SS2D_EINVAL           # out dtype neither f32 nor input
 
 
+def _scan_plan(batch, dim, L, N, G, in_dtype=_lib.SS2D_BF16, with_x=True, base=1 << 20):
+    """ss2d_selective_scan_kernel for dense tensors of these sizes at made-up, 256-byte aligned addresses (the query
+    reads the struct only)."""
+    p = _lib.ScanParams()
+    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups, p.delta_dim = batch, dim, L, N, G, dim
+    p.in_dtype, p.out_dtype, p.delta_softplus = in_dtype, _lib.SS2D_F32, 1
+    p.u, p.delta, p.A, p.B, p.C, p.out = (base * k for k in range(1, 7))
+    p.x = base * 7 if with_x else None
+    p.u_batch_stride, p.u_d_stride = dim * L, L
+    p.delta_batch_stride, p.delta_d_stride = dim * L, L
+    p.A_d_stride, p.A_dstate_stride = N, 1
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = G * N * L, N * L, L
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = G * N * L, N * L, L
+    p.out_batch_stride, p.out_d_stride = dim * L, L
+    return _lib.lib().ss2d_selective_scan_kernel(p)
+
+
+def test_scan_kernel_choice_does_not_depend_on_the_chunk_state_output():
+    """The reference's extension interface always asks for the chunk states `x`
+    (selective_scan_oflex.cpp:207-208): every benchmark shape must reach the same kernel with and without it."""
+    shapes = {  # batch, dim = 4 * d_inner, L, N -> kernel
+        (128, 384, 3136, 1): _lib.SCAN_KERNEL_ROW, (128, 768, 784, 1): _lib.SCAN_KERNEL_ROW,
+        (128, 1536, 196, 1): _lib.SCAN_KERNEL_SMALL, (128, 3072, 49, 1): _lib.SCAN_KERNEL_SMALL,
+        (64, 768, 3136, 16): _lib.SCAN_KERNEL_CHAN, (4, 384, 65536, 1): _lib.SCAN_KERNEL_ROW4,
+        (4, 768, 16384, 1): _lib.SCAN_KERNEL_ROW, (48, 384, 3306, 1): _lib.SCAN_KERNEL_FLAT,
+        (16, 384, 100, 1): _lib.SCAN_KERNEL_FLAT,
+    }
+    for (batch, dim, L, N), kernel in shapes.items():
+        for with_x in (False, True):
+            assert _scan_plan(batch, dim, L, N, 4, with_x=with_x) == kernel, (batch, dim, L, N, with_x)
+    assert _scan_plan(0, 384, 3136, 1, 4) == _lib.SCAN_KERNEL_NONE
+    assert _scan_plan(2, 384, 3136, 1, 5) == _lib.SS2D_EINVAL
+    assert _lib.lib().ss2d_selective_scan_kernel(None) == _lib.SS2D_EINVAL
+    assert len(_lib.SCAN_KERNEL_NAMES) == 6
+
+
 def test_host_api_rejects_cpu_tensors_and_unsupported_modes():
     import torch
     import vmamba_amd as va

@@ -55,6 +55,24 @@ def run_gpu(u, delta, A, B, C, D, bias, softplus, out_float=True, want_x=True):
     return out.cpu(), (x.cpu() if want_x else None)
 
 
+def check_states(xg, xw, tol=None):
+    """chunk-end states x[..., 2n + 1] = h_n and decay products x[..., 2n] against the oracle's."""
+    assert xg.shape == xw.shape and xg.dtype == torch.float32
+    assert torch.allclose(xg[..., 1::2], xw[..., 1::2], **(tol or TOL32)), \
+        f"chunk-end states: max abs err {(xg[..., 1::2] - xw[..., 1::2]).abs().max().item()}"
+    assert torch.allclose(xg[..., 0::2], xw[..., 0::2], rtol=1e-3, atol=1e-30), "chunk-end decay products"
+
+
+def kernel_of(u, delta, A, B, C, want_x, out_float=True):
+    """Name of the kernel the library picks for these tensors once they sit on the GPU."""
+    from vmamba_amd.csms6s import scan_kernel_name
+    dev = lambda t: t.to(DEV)
+    n_chunks = (u.shape[-1] + _lib.SCAN_CHUNK - 1) // _lib.SCAN_CHUNK
+    out = torch.empty(u.shape, device=DEV, dtype=torch.float32 if out_float else u.dtype)
+    x = torch.empty(u.shape[0], u.shape[1], n_chunks, 2 * A.shape[1], device=DEV) if want_x else None
+    return scan_kernel_name(dev(u), dev(delta), dev(A), dev(B), dev(C), out, x)
+
+
 def check(u, delta, A, B, C, D, bias, softplus, out_float=True, tol32=None):
     want, xw = orc.selective_scan(u, delta, A, B, C, D, bias, softplus, out_float=out_float, return_x=True)
     got, xg = run_gpu(u, delta, A, B, C, D, bias, softplus, out_float)
@@ -62,10 +80,8 @@ def check(u, delta, A, B, C, D, bias, softplus, out_float=True, tol32=None):
     tol = (tol32 or TOL32) if out_float or u.dtype == torch.float32 else TOL16
     err = (got.float() - want.float()).abs().max().item()
     assert torch.allclose(got.float(), want.float(), **tol), f"max abs err {err}"
-    assert torch.allclose(xg[..., 1::2], xw[..., 1::2], **TOL32), "chunk-end states"
-    assert torch.allclose(xg[..., 0::2], xw[..., 0::2], rtol=1e-3, atol=1e-30), "chunk-end decay products"
-    # without the chunk-state output the library may pick a different kernel (short rows are packed several to a
-    # wavefront): same bound
+    check_states(xg, xw, tol32)
+    # without the chunk-state output the same kernel runs as another instantiation: same bound
     got2, _ = run_gpu(u, delta, A, B, C, D, bias, softplus, out_float, want_x=False)
     err2 = (got2.float() - want.float()).abs().max().item()
     assert torch.allclose(got2.float(), want.float(), **tol), f"no-x path: max abs err {err2}"
@@ -126,22 +142,26 @@ CHAN_GRID = [
 def test_scan_channel_per_lane_kernel_matches_oracle(batch, dim, G, N, L, dtype):
     _announce("scan-chan", batch, dim, G, N, L, dtype)
     args = make_inputs(31, batch, dim, G, N, L, dtype)
-    want = orc.selective_scan(*args, True, out_float=True)
+    assert kernel_of(*args[:5], want_x=False) == kernel_of(*args[:5], want_x=True) == "chan"
+    want, xw = orc.selective_scan(*args, True, out_float=True, return_x=True)
     got, _ = run_gpu(*args, True, True, want_x=False)
     # Long rows of the reference's test distribution (A down to 1e-4: the state remembers the whole row and reaches
     # |y| ~ 200 while single outputs cancel to ~0): fp32 recurrences agree to ~1e-5 of the output scale, which the
     # absolute part of the tolerance has to carry there (the reference's own fp32 atol is 2e-3, test_selective_scan.py:401)
     tol = TOL32 if L <= 2048 else dict(rtol=1e-3, atol=max(2e-3, 2e-5 * want.abs().max().item()))
     assert torch.allclose(got, want, **tol), f"max abs err {(got - want).abs().max().item()}"
-    # the same rows with the chunk states requested go through the wavefront-scan kernel: two kernels, one answer
+    # the same kernel with the chunk states requested (what the reference's extension interface always does): the
+    # outputs are unchanged and the states after every 2048 positions and at the row's end are the oracle's
     got_x, x = run_gpu(*args, True, True, want_x=True)
-    assert torch.allclose(got_x, want, **tol)
+    assert torch.equal(got_x, got)
+    check_states(x, xw, tol)
     # SS2D-style constants (A = -(1..N), D = 1, dt bias), output in the input dtype
     args = make_inputs(32, batch, dim, G, N, L, dtype, ss2d_like=True)
-    want = orc.selective_scan(*args, True, out_float=False)
-    got, _ = run_gpu(*args, True, False, want_x=False)
+    want, xw = orc.selective_scan(*args, True, out_float=False, return_x=True)
+    got, x = run_gpu(*args, True, False, want_x=True)
     tol = TOL32 if dtype == torch.float32 else TOL16
     assert got.dtype == dtype and torch.allclose(got.float(), want.float(), **tol)
+    check_states(x, xw)
 
 
 @pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False)])
@@ -154,9 +174,10 @@ def test_scan_channel_per_lane_optional_arguments_and_delta_groups(has_D, has_bi
     assert torch.allclose(got, want, **TOL32), f"max abs err {(got - want).abs().max().item()}"
     # one delta row shared by 4 channels
     u, delta, A, B, C, D, bias = make_inputs(34, 2, 128, 2, 8, 136, torch.float32, delta_dim=32)
-    want = orc.selective_scan(u, delta, A, B, C, D, bias, True, out_float=True)
-    got, _ = run_gpu(u, delta, A, B, C, D, bias, True, True, want_x=False)
+    want, xw = orc.selective_scan(u, delta, A, B, C, D, bias, True, out_float=True, return_x=True)
+    got, x = run_gpu(u, delta, A, B, C, D, bias, True, True, want_x=True)
     assert torch.allclose(got, want, **TOL32)
+    check_states(x, xw)
 
 
 # Shapes that select scan_small_kernel (rows of 49 / 196 positions, one state, 16-bit inputs: one segment of a row per
@@ -173,17 +194,20 @@ SMALL_GRID = [
 def test_scan_short_row_kernel_matches_oracle(batch, dim, G, N, L, dtype):
     _announce("scan-small", batch, dim, G, N, L, dtype)
     args = make_inputs(41, batch, dim, G, N, L, dtype)
-    want = orc.selective_scan(*args, True, out_float=True)
+    assert kernel_of(*args[:5], want_x=False) == kernel_of(*args[:5], want_x=True) == "small"
+    want, xw = orc.selective_scan(*args, True, out_float=True, return_x=True)
     got, _ = run_gpu(*args, True, True, want_x=False)
     assert torch.allclose(got, want, **TOL32), f"max abs err {(got - want).abs().max().item()}"
-    # the same rows with the chunk states requested go through the wavefront-scan kernel: two kernels, one answer
-    got_x, _ = run_gpu(*args, True, True, want_x=True)
-    assert torch.allclose(got_x, want, **TOL32)
+    # the same kernel with the row-end states requested (what the reference's extension interface always does)
+    got_x, x = run_gpu(*args, True, True, want_x=True)
+    assert torch.equal(got_x, got)
+    check_states(x, xw)
     # SS2D-style constants (A = -1, D = 1, dt bias), output in the input dtype
     args = make_inputs(42, batch, dim, G, N, L, dtype, ss2d_like=True)
-    want = orc.selective_scan(*args, True, out_float=False)
-    got, _ = run_gpu(*args, True, False, want_x=False)
+    want, xw = orc.selective_scan(*args, True, out_float=False, return_x=True)
+    got, x = run_gpu(*args, True, False, want_x=True)
     assert got.dtype == dtype and torch.allclose(got.float(), want.float(), **TOL16)
+    check_states(x, xw)
 
 
 @pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False)])
@@ -300,15 +324,17 @@ def test_scan_errors_from_host_api():
                                                  (13, 512, 2, 2049, torch.float16)])
 def test_many_long_rows_off_the_vector_grid(batch, dim, G, L, dtype):
     """6144 rows and more of odd length (no row but the first starts on a 16-byte boundary): the library walks them eight
-    to a wavefront as one aligned stream.  Every row against the oracle; with chunk states requested the row kernel
-    runs instead and must agree too."""
+    to a wavefront as one aligned stream.  Every row against the oracle, without and with the chunk states."""
     _announce("scan-long-unaligned", batch, dim, G, L, dtype)
     args = make_inputs(batch * 1000 + L, batch, dim, G, 1, L, dtype, ss2d_like=True)
-    want = orc.selective_scan(*args, True, out_float=True)
+    assert kernel_of(*args[:5], want_x=False) == kernel_of(*args[:5], want_x=True) == "flat"
+    want, xw = orc.selective_scan(*args, True, out_float=True, return_x=True)
     for want_x in (False, True):
-        got, _ = run_gpu(*args, True, True, want_x=want_x)
+        got, x = run_gpu(*args, True, True, want_x=want_x)
         bound = 2e-4 + 1e-3 * want.abs() + 5e-5 * want.abs().amax(dim=-1, keepdim=True)
         assert bool(((got - want).abs() <= bound).all()), (want_x, (got - want).abs().max().item())
+        if want_x:      # two chunks per row: the state after 2048 positions and at the row's end
+            check_states(x, xw, dict(rtol=1e-3, atol=2e-4 + 5e-5 * want.abs().max().item()))
 
 
 @pytest.mark.parametrize("cfg", ["stage1", "stage2", "stage3", "stage4", "n16", "hires", "rows57x58", "rows75x75"])

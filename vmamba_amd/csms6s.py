@@ -21,6 +21,35 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
+def _scan_params(u, delta, A, B, C, D, delta_bias, delta_softplus, out, x):
+    """struct ss2d_scan_params for these tensors (shapes and dtypes already checked)."""
+    p = _lib.ScanParams()
+    p.batch, p.dim, p.seqlen = u.shape
+    p.dstate, p.n_groups, p.delta_dim = A.size(1), B.size(1), delta.size(1)
+    p.in_dtype, p.out_dtype = _DTYPE_CODE[u.dtype], _DTYPE_CODE[out.dtype]
+    p.delta_softplus = int(bool(delta_softplus))
+    p.u, p.delta, p.A, p.B, p.C = u.data_ptr(), delta.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
+    p.D = D.data_ptr() if D is not None else None
+    p.delta_bias = delta_bias.data_ptr() if delta_bias is not None else None
+    p.out = out.data_ptr()
+    p.x = x.data_ptr() if x is not None else None
+    p.u_batch_stride, p.u_d_stride = u.stride(0), u.stride(1)
+    p.delta_batch_stride, p.delta_d_stride = delta.stride(0), delta.stride(1)
+    p.A_d_stride, p.A_dstate_stride = A.stride(0), A.stride(1)
+    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = B.stride(0), B.stride(1), B.stride(2)
+    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = C.stride(0), C.stride(1), C.stride(2)
+    p.out_batch_stride, p.out_d_stride = out.stride(0), out.stride(1)
+    return p
+
+
+def scan_kernel_name(u, delta, A, B, C, out, x=None):
+    """Which kernel of the library serves these (already allocated) tensors: one of _lib.SCAN_KERNEL_NAMES.  Nothing
+    is launched (ss2d_selective_scan_kernel)."""
+    rc = _lib.lib().ss2d_selective_scan_kernel(_scan_params(u, delta, A, B, C, None, None, True, out, x))
+    _lib.check(min(rc, 0), "ss2d_selective_scan_kernel")
+    return _lib.SCAN_KERNEL_NAMES[rc]
+
+
 def selective_scan_fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, nrows=1, out_float=True,
                        want_x=True):
     """Python twin of ``selective_scan_cuda_oflex.fwd``: returns [out, x].
@@ -61,21 +90,7 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplu
     out = torch.empty((batch, dim, seqlen), device=u.device, dtype=torch.float32 if out_float else u.dtype)
     x = torch.empty((batch, dim, n_chunks, dstate * 2), device=u.device, dtype=torch.float32) if want_x else None
 
-    p = _lib.ScanParams()
-    p.batch, p.dim, p.seqlen, p.dstate, p.n_groups, p.delta_dim = batch, dim, seqlen, dstate, n_groups, delta_dim
-    p.in_dtype, p.out_dtype = _DTYPE_CODE[u.dtype], _DTYPE_CODE[out.dtype]
-    p.delta_softplus = int(bool(delta_softplus))
-    p.u, p.delta, p.A, p.B, p.C = u.data_ptr(), delta.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
-    p.D = D.data_ptr() if D is not None else None
-    p.delta_bias = delta_bias.data_ptr() if delta_bias is not None else None
-    p.out = out.data_ptr()
-    p.x = x.data_ptr() if x is not None else None
-    p.u_batch_stride, p.u_d_stride = u.stride(0), u.stride(1)
-    p.delta_batch_stride, p.delta_d_stride = delta.stride(0), delta.stride(1)
-    p.A_d_stride, p.A_dstate_stride = A.stride(0), A.stride(1)
-    p.B_batch_stride, p.B_group_stride, p.B_dstate_stride = B.stride(0), B.stride(1), B.stride(2)
-    p.C_batch_stride, p.C_group_stride, p.C_dstate_stride = C.stride(0), C.stride(1), C.stride(2)
-    p.out_batch_stride, p.out_d_stride = out.stride(0), out.stride(1)
+    p = _scan_params(u, delta, A, B, C, D, delta_bias, delta_softplus, out, x)
     with torch.cuda.device(u.device):
         rc = _lib.lib().ss2d_selective_scan_fwd(p, torch.cuda.current_stream(u.device).cuda_stream)
     _lib.check(rc, "ss2d_selective_scan_fwd")

@@ -126,7 +126,12 @@ struct ChanGeom {
     FastDiv div_cb, div_groups;
 };
 
-template <typename in_t, typename out_t, int kSpw, bool kSoftplus>
+// kX: the chunk-end states are written as well -- x[row][chunk][2n] = product of a_n since the row's start,
+// x[..][2n + 1] = h_n, after every 2048 positions and at the row's end.  h is what the lane holds; the product is
+// exp2(A_n log2e * sum dl), and the sum is per CHANNEL, not per state: each of the four wavefronts adds up a quarter of
+// every round's positions for its lane's channel (one LDS read, four adds per 16 positions) and the quarters meet in LDS
+// when a chunk ends.
+template <typename in_t, typename out_t, int kSpw, bool kSoftplus, bool kX>
 __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restrict__ u_all, const in_t *__restrict__ dl_all,
                                                            const in_t *__restrict__ B_all, const in_t *__restrict__ C_all,
                                                            const float *__restrict__ A_all, out_t *__restrict__ o_all,
@@ -134,6 +139,7 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
     __shared__ __align__(16) float s_dl[kChanBlock * kChanTilePitch];
     __shared__ __align__(16) float s_du[kChanBlock * kChanTilePitch];
     __shared__ __align__(16) float s_y[kWavesPerWg * kChanBlock * kChanSubPitch];
+    __shared__ float s_sum[kX ? kWavesPerWg * kChanBlock : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -173,6 +179,9 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
     const float *my_dl = s_dl + lane * kChanTilePitch, *my_du = s_du + lane * kChanTilePitch;
     float *my_y = s_y + (wave * kChanBlock + lane) * kChanSubPitch;
     const float *sum_y = s_y + r * kChanSubPitch + 4 * q;
+    float dl_sum = 0.0f;                                    // kX: this wavefront's quarter of the channel's sum of dl
+    const bool chan_ok = (int)cb * kChanBlock + lane < dpg;
+    float *x_lane = kX ? p.x + ((int64_t)b * p.dim + dc) * p.n_chunks * 2 * p.N + 2 * (wave * kSpw) : nullptr;
 
     constexpr float kFill = delta_fill<kSoftplus>();
     Raw4<in_t> ru[2], rd[2];
@@ -232,6 +241,10 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
                 }
 #pragma unroll
                 for (int i = 0; i < kChanSub; ++i) y[i] = 0.0f;
+                if constexpr (kX) {
+                    const float4 q4 = *reinterpret_cast<const float4 *>(my_dl + s * kChanSub + 4 * wave);
+                    dl_sum += (q4.x + q4.y) + (q4.z + q4.w);  // (dl is 0 past the row's end)
+                }
                 // the LDS reads above have landed before the first scalar request below is made (one wait covers both
                 // kinds of traffic, so a request issued earlier would be waited for at once)
                 asm volatile("" ::"v"(dl[0]), "v"(dl[4]), "v"(dl[8]), "v"(dl[12]), "v"(du[0]), "v"(du[4]), "v"(du[8]), "v"(du[12]));
@@ -282,13 +295,28 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
             // (after the second round the barrier at the top of the next step does this: its staging writes touch
             //  dl / du only, which every wavefront has finished reading by then)
         }
+        if constexpr (kX) {
+            const int t_end = t0 + kChanTile;
+            if (t_end % SS2D_SCAN_CHUNK == 0 || t_end >= L) {   // uniform over the workgroup; at least 64 steps apart
+                s_sum[wave * kChanBlock + lane] = dl_sum;
+                __syncthreads();
+                const float total = (s_sum[lane] + s_sum[kChanBlock + lane]) + (s_sum[2 * kChanBlock + lane] + s_sum[3 * kChanBlock + lane]);
+                if (chan_ok) {
+                    float *xo = x_lane + (int64_t)((min(t_end, L) - 1) / SS2D_SCAN_CHUNK) * 2 * p.N;
+#pragma unroll
+                    for (int j = 0; j < kSpw; ++j) {
+                        xo[2 * j] = __builtin_amdgcn_exp2f(A2[j] * total);
+                        xo[2 * j + 1] = h[j];
+                    }
+                }
+            }
+        }
     }
 }
 
 bool scan_chan_eligible(const ScanArgs &a) {
-    // N/4 states per wavefront; rows in whole 8-position vectors; at least half a wavefront of channels per group;
-    // no chunk-state output (the row kernels provide it)
-    return (a.N == 4 || a.N == 8 || a.N == 16 || a.N == 32) && a.L % 8 == 0 && a.dim_per_group >= 32 && a.x == nullptr;
+    // N/4 states per wavefront; rows in whole 8-position vectors; at least half a wavefront of channels per group
+    return (a.N == 4 || a.N == 8 || a.N == 16 || a.N == 32) && a.L % 8 == 0 && a.dim_per_group >= 32;
 }
 
 template <typename in_t, typename out_t>
@@ -300,17 +328,21 @@ static int launch_chan_typed(const ScanArgs &a, hipStream_t stream) {
     geo.div_groups = make_fastdiv((uint32_t)groups);
     const int64_t n_wg = (int64_t)a.batch * groups * geo.n_cb;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-#define SS2D_LAUNCH_CHAN(SPW, SP)                                                                                          \
-    hipLaunchKernelGGL((scan_chan_kernel<in_t, out_t, SPW, SP>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,             \
+#define SS2D_LAUNCH_CHAN(SPW, SP, X)                                                                                       \
+    hipLaunchKernelGGL((scan_chan_kernel<in_t, out_t, SPW, SP, X>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,          \
                        (const in_t *)a.u, (const in_t *)a.delta, (const in_t *)a.B, (const in_t *)a.C, a.A, (out_t *)a.out, a, geo)
-#define SS2D_LAUNCH_CHAN_N(SP)                                  \
+#define SS2D_LAUNCH_CHAN_N(SP, X)                               \
     switch (a.N) {                                              \
-        case 4: SS2D_LAUNCH_CHAN(1, SP); break;                 \
-        case 8: SS2D_LAUNCH_CHAN(2, SP); break;                 \
-        case 16: SS2D_LAUNCH_CHAN(4, SP); break;                \
-        default: SS2D_LAUNCH_CHAN(8, SP); break;                \
+        case 4: SS2D_LAUNCH_CHAN(1, SP, X); break;              \
+        case 8: SS2D_LAUNCH_CHAN(2, SP, X); break;              \
+        case 16: SS2D_LAUNCH_CHAN(4, SP, X); break;             \
+        default: SS2D_LAUNCH_CHAN(8, SP, X); break;             \
     }
-    if (a.softplus) { SS2D_LAUNCH_CHAN_N(true) } else { SS2D_LAUNCH_CHAN_N(false) }
+    if (a.x) {
+        if (a.softplus) { SS2D_LAUNCH_CHAN_N(true, true) } else { SS2D_LAUNCH_CHAN_N(false, true) }
+    } else {
+        if (a.softplus) { SS2D_LAUNCH_CHAN_N(true, false) } else { SS2D_LAUNCH_CHAN_N(false, false) }
+    }
 #undef SS2D_LAUNCH_CHAN_N
 #undef SS2D_LAUNCH_CHAN
     return launch_status();

@@ -223,6 +223,38 @@ __device__ __forceinline__ void wave_scan_pairs(float a, float h, float &a_ex, f
     h_tot = read_lane(h, kWave - 1);
 }
 
+// The same scan for two recurrences that share their multipliers: (a, h) and (a, g).  Per step one more fused
+// multiply-add; the exclusive prefixes and totals of both come back.
+__device__ __forceinline__ void wave_scan_pairs2(float a, float h, float g, float &a_ex, float &h_ex, float &g_ex, float &a_tot,
+                                                 float &h_tot, float &g_tot) {
+    float ax = 1.0f, hx = 0.0f, gx = 0.0f;
+#define SS2D_SCAN_STEP2(CTRL)                                  \
+    "v_fmac_f32_dpp %1, %1, %0 " CTRL " bank_mask:0xf\n\t" \
+    "v_fmac_f32_dpp %2, %2, %0 " CTRL " bank_mask:0xf\n\t" \
+    "v_mul_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"  \
+    "s_nop 0\n\t"
+    asm("s_nop 1\n\t"
+                 SS2D_SCAN_STEP2("row_shr:1 row_mask:0xf")
+                 SS2D_SCAN_STEP2("row_shr:2 row_mask:0xf")
+                 SS2D_SCAN_STEP2("row_shr:4 row_mask:0xf")
+                 SS2D_SCAN_STEP2("row_shr:8 row_mask:0xf")
+                 SS2D_SCAN_STEP2("row_bcast:15 row_mask:0xa")
+                 SS2D_SCAN_STEP2("row_bcast:31 row_mask:0xc")
+                 "s_nop 0\n\t"
+                 "v_mov_b32_dpp %3, %0 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "v_mov_b32_dpp %4, %1 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "v_mov_b32_dpp %5, %2 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1"
+                 : "+v"(a), "+v"(h), "+v"(g), "+v"(ax), "+v"(hx), "+v"(gx));
+#undef SS2D_SCAN_STEP2
+    a_ex = ax;
+    h_ex = hx;
+    g_ex = gx;
+    a_tot = read_lane(a, kWave - 1);
+    h_tot = read_lane(h, kWave - 1);
+    g_tot = read_lane(g, kWave - 1);
+}
+
 // One state of one pass: lane-local scan of its 8 items, wave scan of the lane totals, then
 // the state entering the lane (from `carry`, the state entering the pass) is pushed through
 // the items and C*h is accumulated into y.  Returns the pass totals.

@@ -9,9 +9,9 @@
 //     as loaded and read back as per-lane runs; the B and C rows (one pair per tile: its rows belong to one image and
 //     one group) go the same way; a wavefront walks two or four such tiles, the next one's loads in flight while one
 //     is computed, and nothing is shared between wavefronts (no workgroup barrier);
-//   * a lane scans its kNi items serially in registers, the lane totals are combined by a DPP scan over the lane group,
-//     and the state entering the lane is pushed through its items; a row's first item is forced to a = 0, which stops
-//     anything arriving from the neighbouring group;
+//   * a lane scans its kNi items serially in registers, the lane totals are combined by a DPP scan over the DPP row of
+//     16 lanes, and the state entering the lane is pushed through its items; the idle lanes behind a row's segments
+//     enter that scan as the pair (0, 0), which stops anything on its way to the next group of the same DPP row;
 //   * every index is a compile-time constant; the outputs go back through LDS (over the u / delta tiles) and leave as
 //     16-byte stores of consecutive lanes, like the loads.
 // Semantics: selective_scan_fn forward (classification/models/csms6s.py:25-68; kernel
@@ -23,7 +23,9 @@ namespace ss2d {
 // Tiles a wavefront walks, the next one's loads in flight while one is computed (more where a tile is smaller).
 template <int kNl> constexpr int small_tiles() { return kNl <= 8 ? 4 : 2; }
 
-template <typename in_t, typename out_t, int kNl, int kNi, bool kSoftplus>
+// kX: the state at the end of every row is written too (rows are shorter than a 2048-position chunk, so that is the whole
+// chunk-state output): x[row][0] = product of a over the row, x[row][1] = h at its last position.
+template <typename in_t, typename out_t, int kNl, int kNi, bool kSoftplus, bool kX>
 __global__ __launch_bounds__(kBlock) void scan_small_kernel(const ScanArgs p, int bc_vec, FastDiv div_dim, FastDiv div_dpg) {
     constexpr int kSmallTiles = small_tiles<kNl>();
     constexpr int kLanes = kNl <= 8 ? 8 : 16;                // lanes per row
@@ -149,18 +151,33 @@ __global__ __launch_bounds__(kBlock) void scan_small_kernel(const ScanArgs p, in
             float dl;
             if constexpr (kSoftplus) dl = softplus_log2(fmaf(raw.item(j), kLog2e, bias * kLog2e));
             else dl = raw.item(j) + bias;
-            float a = __builtin_amdgcn_exp2f(dl * A2);
-            if (j == 0) a = i == 0 ? 0.0f : a;              // nothing enters a row from the lanes before it
+            const float a = __builtin_amdgcn_exp2f(dl * A2);
             const float bb = Bv.item(j) * (dl * uu.item(j));
             ac[j] = j == 0 ? a : ac[j - 1] * a;
             hh[j] = j == 0 ? bb : fmaf(a, hh[j - 1], bb);
         }
-        // lanes that hold no segment pass the state through unchanged
-        const float a_tot = active ? ac[kNi - 1] : 1.0f, h_tot = active ? hh[kNi - 1] : 0.0f;
+        // lanes that hold no segment stop the state: nothing travels from one group of lanes into the next (the first
+        // lane of a DPP row has no lane below it)
+        const float a_tot = active ? ac[kNi - 1] : 0.0f, h_tot = active ? hh[kNi - 1] : 0.0f;
         const float h_in = row_scan_state_in<false>(a_tot, h_tot);
         float y[kNi];
 #pragma unroll
         for (int j = 0; j < kNi; ++j) y[j] = fmaf(Cv.item(j), fmaf(ac[j], h_in, hh[j]), Dk * uu.item(j));
+        if constexpr (kX) {
+            // the product of the row's lane products ends up in its last lane: each step multiplies in the lane 1 / 2 / 4
+            // (/ 8) below, lanes without a source and idle lanes count as 1, and with groups of 8 lanes the steps stop
+            // at 4 so that a lane reaches back 7 lanes, to its own group's idle lane at most
+            float pr = active ? ac[kNi - 1] : 1.0f;
+            pr *= dpp_move<kDppRowShr1>(1.0f, pr);
+            pr *= dpp_move<kDppRowShr2>(1.0f, pr);
+            pr *= dpp_move<kDppRowShr4>(1.0f, pr);
+            if constexpr (kLanes == 16) pr *= dpp_move<kDppRowShr8>(1.0f, pr);
+            if (active && i == kNl - 1) {
+                float *xo = p.x + (int64_t)(row0 + g) * 2;
+                xo[0] = pr;
+                xo[1] = fmaf(ac[kNi - 1], h_in, hh[kNi - 1]);
+            }
+        }
         if (nr == kRows && p.vec_out_ok) {
             // a full tile: park the outputs where u / delta sat (every lane has read its runs) and store the tile as it
             // lies in memory, 16 bytes per lane
@@ -197,7 +214,7 @@ static bool small_rows_of(int L, int &rows_per_wave) {
 bool scan_small_eligible(const ScanArgs &a, int in_dtype, const void *u, const void *delta, const void *out) {
     int rpw;
     if (in_dtype != SS2D_BF16 && in_dtype != SS2D_F16) return false;
-    if (a.N != 1 || a.x != nullptr || a.dim_per_delta != 1 || !small_rows_of(a.L, rpw)) return false;
+    if (a.N != 1 || a.dim_per_delta != 1 || !small_rows_of(a.L, rpw)) return false;
     const int64_t L = a.L, KD = a.dim;
     // rows adjacent in every stream; a wavefront's rows inside one image and one group
     if (a.u_ds != L || a.dl_ds != L || a.o_ds != L || a.u_bs != KD * L || a.dl_bs != KD * L || a.o_bs != KD * L) return false;
@@ -220,11 +237,14 @@ static int launch_small_typed(const ScanArgs &a, hipStream_t stream) {
     ScanArgs b = a;
     b.vec_out_ok = reinterpret_cast<uintptr_t>(a.out) % 16 == 0;   // a wavefront's output tile starts on a 16-byte boundary
     const int bc_vec = a.L % 4 == 0 && bases % 8 == 0 && a.B_bs % 4 == 0 && a.B_gs % 4 == 0 && a.C_bs % 4 == 0 && a.C_gs % 4 == 0;
-#define SS2D_LAUNCH_SMALL(NL, NI, SP)                                                                                       \
-    hipLaunchKernelGGL((scan_small_kernel<in_t, out_t, NL, NI, SP>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream, b, bc_vec, \
+#define SS2D_LAUNCH_SMALL(NL, NI, SP, X)                                                                                       \
+    hipLaunchKernelGGL((scan_small_kernel<in_t, out_t, NL, NI, SP, X>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream, b, bc_vec, \
                        make_fastdiv((uint32_t)a.dim), make_fastdiv((uint32_t)a.dim_per_group))
-    if (a.L == 196) { if (a.softplus) SS2D_LAUNCH_SMALL(14, 14, true); else SS2D_LAUNCH_SMALL(14, 14, false); }
-    else { if (a.softplus) SS2D_LAUNCH_SMALL(7, 7, true); else SS2D_LAUNCH_SMALL(7, 7, false); }
+#define SS2D_LAUNCH_SMALL_L(SP, X) \
+    if (a.L == 196) SS2D_LAUNCH_SMALL(14, 14, SP, X); else SS2D_LAUNCH_SMALL(7, 7, SP, X)
+    if (a.x) { if (a.softplus) { SS2D_LAUNCH_SMALL_L(true, true); } else { SS2D_LAUNCH_SMALL_L(false, true); } }
+    else { if (a.softplus) { SS2D_LAUNCH_SMALL_L(true, false); } else { SS2D_LAUNCH_SMALL_L(false, false); } }
+#undef SS2D_LAUNCH_SMALL_L
 #undef SS2D_LAUNCH_SMALL
     return launch_status();
 }

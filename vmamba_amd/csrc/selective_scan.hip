@@ -204,7 +204,13 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
 // group, not per item, and B/C are gathered kGran elements at a time through buffer
 // descriptors (their rows are shared by dim/n_groups channels and stay in L1/L2).  A lane
 // touches at most two rows (L >= 8); with kGran == 8 exactly one.
-template <typename in_t, typename out_t, int kN, bool kSoftplus, int kGran>
+//
+// kX: the chunk-end states are written too.  h at a chunk's (or row's) last position is what the scan yields there.  The
+// product of a since the row's start is a second recurrence on the SAME multipliers: with a forced to 0 at a row's
+// first position, g_t = a_t g_(t-1) + c_t with c = the true a at that first position and 0 elsewhere gives
+// g_t = a_start ... a_t, so it rides through the lane-local and the wavefront scan beside h (wave_scan_pairs2).  Chunk
+// and row ends fall on group boundaries (rows start at multiples of kGran in the stream, chunks at multiples of 8).
+template <typename in_t, typename out_t, int kN, bool kSoftplus, int kGran, bool kX>
 __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int rows_per_wave, FastDiv divL,
                                                            FastDiv divDim, FastDiv divDpg) {
     constexpr int kGroups = kItems / kGran;
@@ -223,9 +229,11 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
 
-    float h_reg[kN];
+    float h_reg[kN], g_reg[kX ? kN : 1];
 #pragma unroll
     for (int n = 0; n < kN; ++n) h_reg[n] = 0.0f;
+#pragma unroll
+    for (int n = 0; n < (kX ? kN : 1); ++n) g_reg[n] = 0.0f;
 
     const int n_pass = (n_el + kPass - 1) / kPass;
     for (int pass = 0; pass < n_pass; ++pass) {
@@ -280,11 +288,18 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
         float du[kItems], y[kItems], bias_items[kItems];
         bool in_a[kGroups], first[kGroups];
         uint32_t boff[kGroups], coff[kGroups];
+        float *x_end[kX ? kGroups : 1];       // kX: where the group's last item puts its state (null: not a chunk end)
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             in_a[gi] = kGran == kItems ? true : gi * kGran < k;
             const uint32_t li = in_a[gi] ? l0 + gi * kGran : (uint32_t)(gi * kGran - k);
             first[gi] = li == 0;
+            if constexpr (kX) {
+                const uint32_t l_end = li + kGran;
+                const bool ends = e0 + gi * kGran < n_el && (l_end == (uint32_t)L || l_end % SS2D_SCAN_CHUNK == 0);
+                const int64_t row = r0 + rl + (in_a[gi] ? 0 : 1);
+                x_end[gi] = ends ? p.x + (row * p.n_chunks + (l_end - 1) / SS2D_SCAN_CHUNK) * 2 * kN : nullptr;
+            }
             boff[gi] = (in_a[gi] ? Boff_a : Boff_b) + li;
             coff[gi] = (in_a[gi] ? Coff_a : Coff_b) + li;
 #pragma unroll
@@ -309,20 +324,41 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
 #pragma unroll
                 for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
             }
-            float ac[kItems], hh[kItems];
+            float ac[kItems], hh[kItems], gg[kX ? kItems : 1];
 #pragma unroll
             for (int i = 0; i < kItems; ++i) {
                 const int gi = i / kGran;
                 float a = __builtin_amdgcn_exp2f(dl[i] * (in_a[gi] ? A_a[n] : A_b[n]));
-                if (i % kGran == 0) a = first[gi] ? 0.0f : a;
+                float c = 0.0f;
+                if (i % kGran == 0) {
+                    if constexpr (kX) c = first[gi] ? a : 0.0f;
+                    a = first[gi] ? 0.0f : a;
+                }
                 // past the end of the run the gathered B belongs to some other row: keep it out
                 const float bb = (e0 + i < n_el) ? Bv[i] * du[i] : 0.0f;
                 ac[i] = i == 0 ? a : ac[i - 1] * a;
                 hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
+                if constexpr (kX) gg[i] = i == 0 ? c : (i % kGran == 0 ? fmaf(a, gg[i - 1], c) : a * gg[i - 1]);
             }
-            float a_ex, h_ex, a_tot, h_tot;
-            wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
-            const float s_in = fmaf(a_ex, h_reg[n], h_ex);
+            float a_ex, h_ex, a_tot, h_tot, s_in;
+            if constexpr (kX) {
+                float g_ex, g_tot;
+                wave_scan_pairs2(ac[kItems - 1], hh[kItems - 1], gg[kItems - 1], a_ex, h_ex, g_ex, a_tot, h_tot, g_tot);
+                s_in = fmaf(a_ex, h_reg[n], h_ex);
+                const float g_in = fmaf(a_ex, g_reg[n], g_ex);
+#pragma unroll
+                for (int gi = 0; gi < kGroups; ++gi) {
+                    const int ie = gi * kGran + kGran - 1;
+                    if (x_end[gi]) {
+                        x_end[gi][2 * n] = fmaf(ac[ie], g_in, gg[ie]);
+                        x_end[gi][2 * n + 1] = fmaf(ac[ie], s_in, hh[ie]);
+                    }
+                }
+                g_reg[n] = fmaf(a_tot, g_reg[n], g_tot);
+            } else {
+                wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+                s_in = fmaf(a_ex, h_reg[n], h_ex);
+            }
 #pragma unroll
             for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
             h_reg[n] = fmaf(a_tot, h_reg[n], h_tot);
@@ -443,14 +479,14 @@ static bool span_fits_u32(const ScanArgs &a, int64_t elem_bytes) {
 }
 
 // The flat kernel needs dense u / delta / out (rows adjacent in memory, base 16-byte aligned), one delta row
-// per channel, no chunk-state output, rows of at least one lane vector, and dstate 1 or 16.
+// per channel, rows of at least one lane vector, and dstate 1 or 16.
 static bool flat_eligible(const ScanArgs &a, const ss2d_scan_params *q) {
     const int64_t L = a.L, KD = a.dim;
     // rows of four passes and more only where the row kernel would fall back to element-wise accesses (the caller
     // checks that) and there are rows enough to fill the chip eight to a wavefront (measured, unaligned bf16 rows of
     // 5625 positions: 27 264 rows 515 us against 1112, 6144 rows 191 against 241, 3072 rows 153 against 114)
     const bool length_ok = L < 4 * kPass || (L <= (1 << 24) && a.N == 1 && a.rows >= 6144);
-    return a.x == nullptr && L >= kItems && length_ok && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
+    return L >= kItems && length_ok && (a.N == 1 || a.N == 16) && q->delta_dim == q->dim &&
            a.u_ds == L && a.dl_ds == L && a.o_ds == L && a.u_bs == KD * L && a.dl_bs == KD * L && a.o_bs == KD * L &&
            aligned16(q->u) && aligned16(q->delta) && aligned16(q->out) &&
            span_fits_u32(a, q->in_dtype == SS2D_F32 ? 4 : 2);
@@ -480,29 +516,30 @@ static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
     const FastDiv dL = make_fastdiv((uint32_t)a.L), dDim = make_fastdiv((uint32_t)a.dim),
                   dDpg = make_fastdiv((uint32_t)a.dim_per_group);
     const int gran = flat_granularity(a, (int64_t)sizeof(in_t));
-#define SS2D_LAUNCH_FLAT(N, SP, G) \
-    hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, N, SP, G>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL, dDim, dDpg)
-#define SS2D_LAUNCH_FLAT_G(N, SP)                                   \
+#define SS2D_LAUNCH_FLAT(N, SP, G, X) \
+    hipLaunchKernelGGL((scan_flat_kernel<in_t, out_t, N, SP, G, X>), dim3(n_wg), dim3(kBlock), 0, stream, a, rows_per_wave, dL, dDim, dDpg)
+#define SS2D_LAUNCH_FLAT_G(N, SP, X)                                \
     switch (gran) {                                                  \
-        case 8: SS2D_LAUNCH_FLAT(N, SP, 8); break;                   \
-        case 4: SS2D_LAUNCH_FLAT(N, SP, 4); break;                   \
-        case 2: SS2D_LAUNCH_FLAT(N, SP, 2); break;                   \
-        default: SS2D_LAUNCH_FLAT(N, SP, 1); break;                  \
+        case 8: SS2D_LAUNCH_FLAT(N, SP, 8, X); break;                \
+        case 4: SS2D_LAUNCH_FLAT(N, SP, 4, X); break;                \
+        case 2: SS2D_LAUNCH_FLAT(N, SP, 2, X); break;                \
+        default: SS2D_LAUNCH_FLAT(N, SP, 1, X); break;               \
     }
+#define SS2D_LAUNCH_FLAT_X(N, SP) \
+    if (a.x) { SS2D_LAUNCH_FLAT_G(N, SP, true) } else { SS2D_LAUNCH_FLAT_G(N, SP, false) }
     if (a.N == 1) {
-        if (a.softplus) { SS2D_LAUNCH_FLAT_G(1, true) } else { SS2D_LAUNCH_FLAT_G(1, false) }
+        if (a.softplus) { SS2D_LAUNCH_FLAT_X(1, true) } else { SS2D_LAUNCH_FLAT_X(1, false) }
     } else {
-        if (a.softplus) { SS2D_LAUNCH_FLAT_G(16, true) } else { SS2D_LAUNCH_FLAT_G(16, false) }
+        if (a.softplus) { SS2D_LAUNCH_FLAT_X(16, true) } else { SS2D_LAUNCH_FLAT_X(16, false) }
     }
+#undef SS2D_LAUNCH_FLAT_X
 #undef SS2D_LAUNCH_FLAT_G
 #undef SS2D_LAUNCH_FLAT
     return launch_status();
 }
 
 template <typename in_t, typename out_t, bool kVec>
-static int launch_scan(const ScanArgs &a, hipStream_t stream) {
-    // Few long rows: split every row over the 4 wavefronts of a workgroup.
-    const bool split_rows = a.L > SS2D_SCAN_CHUNK && a.rows < 2048;      // (3072 rows and more: a wavefront per row is faster)
+static int launch_scan(const ScanArgs &a, bool split_rows, hipStream_t stream) {
     if (split_rows) {
         const size_t smem = (size_t)(2 * a.N * kWavesPerWg + 2 * a.N) * sizeof(float2);
         if (a.softplus) {
@@ -537,26 +574,29 @@ static int launch_scan(const ScanArgs &a, hipStream_t stream) {
 }
 
 template <typename in_t, typename out_t>
-static int dispatch_vec(const ScanArgs &a, bool vec, bool flat, hipStream_t stream) {
-    if (flat) return launch_flat<in_t, out_t>(a, stream);
-    return vec ? launch_scan<in_t, out_t, true>(a, stream) : launch_scan<in_t, out_t, false>(a, stream);
+static int dispatch_vec(const ScanArgs &a, bool vec, int kernel, hipStream_t stream) {
+    if (kernel == SS2D_SCAN_KERNEL_FLAT) return launch_flat<in_t, out_t>(a, stream);
+    const bool split_rows = kernel == SS2D_SCAN_KERNEL_ROW4;
+    return vec ? launch_scan<in_t, out_t, true>(a, split_rows, stream) : launch_scan<in_t, out_t, false>(a, split_rows, stream);
 }
 
 }  // namespace ss2d
 
-extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) {
-    using namespace ss2d;
+namespace ss2d {
+
+// Validation and kernel choice shared by the launch and the query entry points.  Returns an SS2D_SCAN_KERNEL_* id
+// (SS2D_SCAN_KERNEL_NONE for an empty problem) or a negative status; fills `a` and `vec` for the launch.
+static int plan_scan(const ss2d_scan_params *q, ScanArgs &a, bool &vec) {
     if (!q) return SS2D_EINVAL;
     if (q->batch < 0 || q->dim < 0 || q->seqlen < 0) return SS2D_EINVAL;
     if (q->dstate <= 0 || q->dstate > 256 || q->n_groups <= 0 || q->delta_dim <= 0) return SS2D_EINVAL;
     if (q->in_dtype != SS2D_F32 && q->in_dtype != SS2D_BF16 && q->in_dtype != SS2D_F16) return SS2D_EINVAL;
     if (q->out_dtype != SS2D_F32 && q->out_dtype != q->in_dtype) return SS2D_EINVAL;
     if (q->dim % q->n_groups != 0 || q->dim % q->delta_dim != 0) return SS2D_EINVAL;
-    if (q->batch == 0 || q->dim == 0 || q->seqlen == 0) return SS2D_OK;
+    if (q->batch == 0 || q->dim == 0 || q->seqlen == 0) return SS2D_SCAN_KERNEL_NONE;
     if (!q->u || !q->delta || !q->A || !q->B || !q->C || !q->out) return SS2D_EINVAL;
     if ((int64_t)q->batch * q->dim > 0x7fffffff - kWavesPerWg) return SS2D_ENOTSUP;
 
-    ScanArgs a;
     a.u = q->u; a.delta = q->delta; a.B = q->B; a.C = q->C;
     a.A = (const float *)q->A; a.D = (const float *)q->D; a.bias = (const float *)q->delta_bias;
     a.out = q->out; a.x = (float *)q->x;
@@ -572,6 +612,7 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     a.C_bs = q->C_batch_stride; a.C_gs = q->C_group_stride; a.C_ns = q->C_dstate_stride;
     a.o_bs = q->out_batch_stride; a.o_ds = q->out_d_stride;
     a.rows = q->batch * q->dim;
+    a.vec_out_ok = 0;
     a.B_span_bytes = a.C_span_bytes = 0;
     const int64_t in_bytes = q->in_dtype == SS2D_F32 ? 4 : 2;
     const bool spans_fit = span_fits_u32(a, in_bytes);
@@ -584,26 +625,48 @@ extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) 
     const int64_t in_vec = q->in_dtype == SS2D_F32 ? 4 : 8;
     const int64_t out_vec = q->out_dtype == SS2D_F32 ? 4 : 8;
     const int64_t in_strides[] = {a.u_bs, a.u_ds, a.dl_bs, a.dl_ds, a.B_bs, a.B_gs, a.B_ns, a.C_bs, a.C_gs, a.C_ns};
-    bool vec = aligned16(q->u) && aligned16(q->delta) && aligned16(q->B) && aligned16(q->C) && aligned16(q->out);
+    vec = aligned16(q->u) && aligned16(q->delta) && aligned16(q->B) && aligned16(q->C) && aligned16(q->out);
     vec = vec && (q->seqlen % in_vec == 0) && (q->seqlen % out_vec == 0);
     for (int64_t s : in_strides) vec = vec && (s % in_vec == 0);
     vec = vec && (a.o_bs % out_vec == 0) && (a.o_ds % out_vec == 0);
 
+    // rows of 49 / 196 positions, one state, rows adjacent in memory: one segment of a row per lane
+    if (scan_small_eligible(a, q->in_dtype, q->u, q->delta, q->out)) return SS2D_SCAN_KERNEL_SMALL;
+    // several states per channel and enough channels per group to fill wavefronts: one channel per lane
+    if (vec && scan_chan_eligible(a)) return SS2D_SCAN_KERNEL_CHAN;
     // A pass of the flat kernel costs about 1.4x a pass of the row kernel (measured), so the flat kernel wins
     // when the row kernel would leave more than ~30 % of its lanes idle, or cannot use vector I/O at all.
     const int64_t row_slots = ((int64_t)q->seqlen + kPass - 1) / kPass * kPass;
-    const bool flat = flat_eligible(a, q) && (!vec || 10 * (int64_t)q->seqlen < 7 * row_slots);
+    if (flat_eligible(a, q) && (!vec || 10 * (int64_t)q->seqlen < 7 * row_slots)) return SS2D_SCAN_KERNEL_FLAT;
+    // few long rows: every row split over the four wavefronts of a workgroup (3072 rows and more: a wavefront per row is faster)
+    if (a.L > SS2D_SCAN_CHUNK && a.rows < 2048) return SS2D_SCAN_KERNEL_ROW4;
+    return SS2D_SCAN_KERNEL_ROW;
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_selective_scan_kernel(const ss2d_scan_params *q) {
+    ss2d::ScanArgs a;
+    bool vec = false;
+    return ss2d::plan_scan(q, a, vec);
+}
+
+extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) {
+    using namespace ss2d;
+    ScanArgs a;
+    bool vec = false;
+    const int kernel = plan_scan(q, a, vec);
+    if (kernel < 0) return kernel;
+    if (kernel == SS2D_SCAN_KERNEL_NONE) return SS2D_OK;
     hipStream_t s = (hipStream_t)stream;
-    // rows of 49 / 196 positions, one state, rows adjacent in memory: one segment of a row per lane
-    if (scan_small_eligible(a, q->in_dtype, q->u, q->delta, q->out)) return launch_scan_small(a, q->in_dtype, q->out_dtype, s);
-    // several states per channel and enough channels per group to fill wavefronts: one channel per lane
-    if (vec && scan_chan_eligible(a)) return launch_scan_chan(a, q->in_dtype, q->out_dtype, s);
-    if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, flat, s);
+    if (kernel == SS2D_SCAN_KERNEL_SMALL) return launch_scan_small(a, q->in_dtype, q->out_dtype, s);
+    if (kernel == SS2D_SCAN_KERNEL_CHAN) return launch_scan_chan(a, q->in_dtype, q->out_dtype, s);
+    if (q->in_dtype == SS2D_F32) return dispatch_vec<float, float>(a, vec, kernel, s);
     if (q->in_dtype == SS2D_BF16) {
-        return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, flat, s)
-                                        : dispatch_vec<bf16_t, bf16_t>(a, vec, flat, s);
+        return q->out_dtype == SS2D_F32 ? dispatch_vec<bf16_t, float>(a, vec, kernel, s)
+                                        : dispatch_vec<bf16_t, bf16_t>(a, vec, kernel, s);
     }
-    return q->out_dtype == SS2D_F32 ? dispatch_vec<f16_t, float>(a, vec, flat, s) : dispatch_vec<f16_t, f16_t>(a, vec, flat, s);
+    return q->out_dtype == SS2D_F32 ? dispatch_vec<f16_t, float>(a, vec, kernel, s) : dispatch_vec<f16_t, f16_t>(a, vec, kernel, s);
 }
 
 extern "C" int ss2d_abi_version(void) { return SS2D_ABI_VERSION; }
