@@ -96,6 +96,50 @@ def test_core_matches_oracle_composition(shape, dtype):
     assert torch.allclose(got, want, **TOL), f"max abs err {err}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("S", [7, 14, 9, 19])
+@pytest.mark.parametrize("B", [1, 3, 5, 9, 11])
+def test_core_small_maps_in_the_padded_batch_layout(B, S, dtype):
+    """The layout SS2D.forward_core_fused hands over when batch * L is not a multiple of the 16-byte vector: delta
+    (4, D, Bp, L) and the projection rows (4, R + 2, Bp, L) with room for Bp >= B images, sliced to the first B.  This is
+    how the row-per-lane kernel meets a short last tile of an ODD number of 7 x 7 maps, and the general kernel a
+    16-byte-aligned stream of odd maps (9 x 9, 19 x 19) that ends in the middle of a 16-byte vector: the last
+    elements of such a stream must arrive although the vector that holds them reaches past the stream's extent.
+    Every image against the oracle."""
+    _announce("core padded batch", B, S, dtype)
+    D, L, R = 5, S * S, 3
+    unit = 8 // __import__("math").gcd(L, 8)
+    Bp = (B + unit - 1) // unit * unit
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(100 * B + S, B, D, S, S, dtype)
+    delta_buf = torch.zeros(4, D, Bp, L, dtype=dtype)
+    x_dbl = torch.zeros(4, R + 2, Bp, L, dtype=dtype)
+    delta_buf[:, :, :B] = delta
+    x_dbl[:, R, :B], x_dbl[:, R + 1, :B] = Bs, Cs
+    want = oracle_core(x, delta, Bs, Cs, A, Dv, bias)
+    dbuf, xbuf = delta_buf.to(DEV), x_dbl.to(DEV)
+    dview, bview, cview = dbuf[:, :, :B], xbuf[:, R, :B], xbuf[:, R + 1, :B]
+    assert dview.stride() == (D * Bp * L, Bp * L, L, 1) and bview.stride() == ((R + 2) * Bp * L, L, 1)
+    got = ss2d_core_hip(x.to(DEV), dview, bview, cview, A.to(DEV), Dv.to(DEV), bias.to(DEV), True)
+    torch.cuda.synchronize()
+    err = (got.cpu() - want).abs().max().item()
+    assert torch.allclose(got.cpu(), want, **TOL), f"max abs err {err}"
+    # the last image's last positions in every direction's order are where a dropped stream element would show
+    assert torch.allclose(got.cpu()[B - 1, :, -S:], want[B - 1, :, -S:], **TOL)
+    assert torch.allclose(got.cpu()[B - 1, :, :S], want[B - 1, :, :S], **TOL)
+
+
+@pytest.mark.parametrize("B", [1, 3, 9])
+def test_core_small_maps_contiguous_streams_end_at_the_allocation(B):
+    """7 x 7 maps, contiguous (4, D, B, L) streams whose last tile is short and odd and whose last element is the last
+    element of the tensor: B / C rows of 8-element-aligned direction stride take the row-per-lane kernel only when
+    B * L is a multiple of 8, so this runs the general kernel at odd B -- same bound, same inputs."""
+    _announce("core contiguous odd batch", B)
+    args = make_core_inputs(700 + B, B, 4, 7, 7, torch.bfloat16)
+    want = oracle_core(*args)
+    got = run_core(*args)
+    assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
+
+
 @pytest.mark.parametrize("softplus", [True, False])
 def test_core_optional_arguments(softplus):
     _announce("core optional", softplus)

@@ -407,6 +407,18 @@ template <typename in_t, int kS> struct Run {
             w[kWords - 1] = r[kWords - 1] >> shift;
         }
     }
+    // Odd kS, global memory: the kS elements that follow the first `skip` (0 or 1) of the kS + 1 elements at src.
+    // src may sit on any 2-byte boundary; every element read lies in [src, src + kS + 1).
+    __device__ __forceinline__ void read_from(const uint16_t *src, int skip) {
+        static_assert(kS % 2 != 0, "even runs are read in place");
+        uint32_t r[kWords];
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) __builtin_memcpy(&r[k], src + 2 * k, 4);
+        const uint32_t shift = (uint32_t)skip * 16u;
+#pragma unroll
+        for (int k = 0; k + 1 < kWords; ++k) w[k] = __builtin_amdgcn_alignbit(r[k + 1], r[k], shift);
+        w[kWords - 1] = r[kWords - 1] >> shift;
+    }
     __device__ __forceinline__ void pack(const uint16_t (&e)[kS]) {
 #pragma unroll
         for (int k = 0; k < kS / 2; ++k) w[k] = (uint32_t)e[2 * k] | ((uint32_t)e[2 * k + 1] << 16);

@@ -614,7 +614,10 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     a.dl_ks = q->delta_dir_stride; a.dl_ds = q->delta_dim_stride; a.dl_bs = q->delta_batch_stride;
     a.B_ks = q->B_dir_stride; a.B_bs = q->B_batch_stride; a.C_ks = q->C_dir_stride; a.C_bs = q->C_batch_stride;
     const int64_t eb = q->in_dtype == SS2D_F32 ? 4 : 2;
-    const int64_t B_span = (3 * a.B_ks + (int64_t)(a.B - 1) * a.B_bs + L) * eb, C_span = (3 * a.C_ks + (int64_t)(a.B - 1) * a.C_bs + L) * eb;
+    // extents in whole 16-byte pieces: a vector load that straddles the extent loses more than the bytes behind it, and
+    // rows of odd length end in the middle of a piece (the rest of that piece lies in the same 16-byte block of memory)
+    const int64_t B_span = ((3 * a.B_ks + (int64_t)(a.B - 1) * a.B_bs + L) * eb + 15) & ~(int64_t)15;
+    const int64_t C_span = ((3 * a.C_ks + (int64_t)(a.B - 1) * a.C_bs + L) * eb + 15) & ~(int64_t)15;
     if (B_span >= 0x7fffffffll || C_span >= 0x7fffffffll) return SS2D_ENOTSUP;
     a.B_span_bytes = (uint32_t)B_span; a.C_span_bytes = (uint32_t)C_span;
     a.CB = 1; a.vec_ok = 0; a.vec_out = 0; a.stage_tiles = 0; a.tile_merge = 0;

@@ -71,7 +71,11 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
     uint4 r_dl[4][kVecsPerLane];
     {
         const in_t *dl_all = reinterpret_cast<const in_t *>(p.delta);
-        const int tile_bytes = nb * kL * 2;
+        // (the extent in whole 16-byte pieces: a piece that straddles the extent loses more than the bytes behind it --
+        //  measured: with the exact extent the last element of a short tile of odd maps came back as zero.  What the
+        //  last piece holds behind the tile is the next image's first elements or, at the tensor's end, the rest of
+        //  a 16-byte block that starts inside the tensor; no lane with a map uses it)
+        const int tile_bytes = (nb * kL * 2 + 15) & ~15;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const in_t *dl_k = dl_all + (int64_t)k * p.dl_ks + (int64_t)d * p.dl_ds + (int64_t)b0 * kL;
@@ -83,8 +87,9 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
             }
         }
     }
-    // B / C: the workgroup's threads share the 8 tiles; one descriptor over each tensor, the tile chosen per lane (what
-    // lies behind a short last tile is other images' data or, past the tensor, zeros: finite either way, never stored)
+    // B / C: the workgroup's threads share the 8 tiles; one descriptor over each tensor (its extent rounded up to whole
+    // 16-byte pieces by the host, as above), the tile chosen per lane (what lies behind a short last tile is other
+    // images' data or, past the tensor, zeros: never stored)
     uint4 r_bc[kBcPerThread];
     {
         const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bm), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
@@ -106,7 +111,15 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
     Run<in_t, kS> x_row, x_col;
     {
         const in_t *map = reinterpret_cast<const in_t *>(p.x) + ((int64_t)(b0 + gc) * p.D + d) * kL;
-        x_row.read(reinterpret_cast<const uint16_t *>(map), ic * kS);
+        if constexpr (kS % 2 == 0) {
+            x_row.read(reinterpret_cast<const uint16_t *>(map), ic * kS);
+        } else {
+            // an odd row is fetched as the kS + 1 elements that start at its first one -- for the map's last row, which
+            // ends where the map ends, as those that start one element earlier, shifted into place: nothing outside
+            // the map is touched
+            const int back = ic == kS - 1 ? 1 : 0;
+            x_row.read_from(reinterpret_cast<const uint16_t *>(map) + ic * kS - back, back);
+        }
         uint16_t e[kS];
 #pragma unroll
         for (int j = 0; j < kS; ++j) e[j] = map[j * kS + ic].bits;
