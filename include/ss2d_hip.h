@@ -10,8 +10,10 @@
  *     enqueued on it and the call returns without synchronising;
  *   - nothing is allocated, freed or synchronised inside the library; outputs are
  *     caller-allocated, inputs are only read;
- *   - re-entrant: there is no global state, so concurrent calls on different
- *     streams are independent;
+ *   - re-entrant: no entry point keeps state between calls, so concurrent calls on
+ *     different streams are independent -- with ONE exception, ss2d_cross_scan_flex_static,
+ *     whose staging buffer is a device array owned by the library (one per GPU, its address
+ *     cached per device on first use): calls of it that overlap on one GPU race on that array;
  *   - the return value is SS2D_OK or a negative SS2D_E* code (errno numbering); on
  *     error nothing has been launched.  No exception crosses this boundary.
  *

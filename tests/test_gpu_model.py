@@ -13,6 +13,27 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def bf16_ulp(scale):
+    """Spacing of bf16 numbers at magnitude `scale` (8 significand bits)."""
+    import math
+    return 2.0 ** (math.floor(math.log2(scale)) - 7)
+
+
+def logit_error_report(got, want, what):
+    """Per-element error of logits against the fp32 reference: in units of the bf16 spacing at the largest |logit|, and
+    relative to each reference logit (floored at 5 % of the largest, random-init logits crossing zero).  Returns the
+    largest error in bf16 spacings and the median relative error; prints median / p99 / max of both."""
+    got, want = got.double().cpu(), want.double().cpu()
+    scale = want.abs().max().item()
+    err = (got - want).abs().flatten()
+    rel = err / want.abs().flatten().clamp_min(0.05 * scale)
+    q = lambda t, p: torch.quantile(t, p).item()
+    print(f"{what}: largest |logit| {scale:.4g} (bf16 spacing {bf16_ulp(scale):.3g}); |error| in spacings: median "
+          f"{q(err, 0.5) / bf16_ulp(scale):.3f} p99 {q(err, 0.99) / bf16_ulp(scale):.3f} max {err.max().item() / bf16_ulp(scale):.3f}; "
+          f"relative error: median {q(rel, 0.5):.3g} p99 {q(rel, 0.99):.3g} max {rel.max().item():.3g}", flush=True)
+    return err.max().item() / bf16_ulp(scale), q(rel, 0.5)
+
+
 def _pair(d_model, d_state, ssm_ratio=1.0, disable_z=True, seed=0):
     torch.manual_seed(seed)
     ref = RefSS2D(d_model=d_model, d_state=d_state, ssm_ratio=ssm_ratio, disable_z=disable_z).eval()
@@ -123,9 +144,12 @@ def test_vmamba_tiny_bf16_benchmark_layout_matches_fp32_reference():
         with torch.no_grad():
             got[channel_first] = hip(x.to(DEV)).float().cpu()
         err = (got[channel_first] - want).abs().max().item()
-        print(f"channel_first={channel_first}: max |logit error| {err:.3e} on a scale of {scale:.3e}", flush=True)
         assert got[channel_first].shape == (2, 1000)
         assert err <= 2e-2 * scale, f"channel_first={channel_first}"
+        # per element: no logit further from the fp32 model than two bf16 spacings at the logits' scale (measured: 0.6),
+        # half of them within 1 % of their value (measured: 0.5 %)
+        worst, median_rel = logit_error_report(got[channel_first], want, f"bf16 224^2 channel_first={channel_first} vs fp32 CPU model")
+        assert worst <= 2.0 and median_rel <= 1e-2, f"channel_first={channel_first}"
     assert (got[True] - got[False]).abs().max().item() <= 2e-2 * scale
 
 
@@ -151,9 +175,10 @@ def test_vmamba_tiny_bf16_1024px_batch4():
             got[channel_first] = hip(x.to(DEV)).float().cpu()
         del hip
         err = (got[channel_first][3:4] - want).abs().max().item()
-        print(f"channel_first={channel_first}: max |logit error| {err:.3e} on a scale of {scale:.3e}", flush=True)
         assert got[channel_first].shape == (4, 1000) and torch.isfinite(got[channel_first]).all()
         assert err <= 2e-2 * scale, f"channel_first={channel_first}"
+        worst, median_rel = logit_error_report(got[channel_first][3:4], want, f"bf16 1024^2 channel_first={channel_first} vs fp32 CPU model")
+        assert worst <= 2.0 and median_rel <= 1e-2, f"channel_first={channel_first}"
     assert (got[True] - got[False]).abs().max().item() <= 2e-2 * scale
 
 
@@ -194,8 +219,10 @@ def test_with_layout_twin_gives_the_same_logits():
         a, b, c = cf(x).float(), cl(x).float(), shared(x).float()
     assert (a - b).abs().max().item() <= 2e-2 * a.abs().max().item()
     # same weights through the same kernels; not asserted bit for bit, since the library may pick another convolution
-    # or GEMM solution for the second model
-    assert (b - c).abs().max().item() <= 2e-2 * a.abs().max().item()
+    # or GEMM solution for the second model, whose fp32 sums then round differently here and there: two bf16 spacings
+    # at the logits' scale bound that (measured over three seeds: 0, 0.5 and 1 spacing)
+    worst, _ = logit_error_report(c, b, "shared-weights twin vs its channel-last original")
+    assert worst <= 2.0
 
 
 def test_small_vssm_trains_on_the_gpu():

@@ -91,6 +91,18 @@ def test_graph_survives_cache_eviction_and_refuses_stale_weights():
     assert not runner.parameters_unchanged()
     with pytest.raises(RuntimeError):
         runner.replay()
+    # a re-capture after the update pins fresh constants and drops the stale ones instead of piling them up
+    runner2 = ConcurrentGraphRunner(m, x, 2)
+    pinned = block.__dict__["_pinned_consts"]
+    assert len({k[2] for k in pinned}) == 1
+    runner2.replay()
+    torch.cuda.synchronize()
+    # storage replaced without touching the version counter (what .half() / .to() / `param.data = ...` do)
+    with torch.no_grad():
+        block.Ds.data = block.Ds.data.clone()
+    assert not runner2.parameters_unchanged()
+    with pytest.raises(RuntimeError):
+        runner2.replay()
 
 
 def test_runner_rejects_uneven_sub_batches(model):

@@ -19,8 +19,10 @@ What a graph bakes in, and how the runner keeps it valid:
     eager work ever touches one.
   * per-module constants.  The SS2D blocks cache small tensors derived from their parameters; a capture pins the ones it
     reads (``SS2D._inference_constants``) so that cache eviction cannot free them under a live graph.
-  * parameter values.  Those pinned constants are copies: after an in-place parameter update a replay would mix fresh
-    weights with stale copies, so ``replay()`` checks the parameters' version counters and refuses.
+  * parameter values.  Those pinned constants are copies, and the graphs hold the addresses of the parameters' storage:
+    after an in-place update, a ``.half()`` / ``.to()`` or a ``param.data = ...`` a replay would read stale copies or
+    freed memory, so ``replay()`` compares storage address, dtype and version counter of every parameter and buffer
+    with what they were at capture time and refuses on any difference.
 """
 import time
 
@@ -57,8 +59,8 @@ class ConcurrentGraphRunner:
                 self.graphs.append(g)
                 self.outs.append(out)
         torch.cuda.synchronize(dev)
-        self._params = [p for p in model.parameters()]
-        self._versions = [p._version for p in self._params]
+        self._tensors = list(model.parameters()) + list(model.buffers())
+        self._signature = self._tensor_signature()
         self.streams = self._pick_streams(sub_batches - 1, stream_sets)
         self.step_ms = self._time_step(self.streams) if sub_batches > 1 else None
 
@@ -102,9 +104,15 @@ class ConcurrentGraphRunner:
                 best = (ms, streams)
         return best[1]
 
+    def _tensor_signature(self):
+        # storage address, dtype and version counter of every parameter and buffer: an in-place update bumps the
+        # version; model.half() / .to() / `param.data = ...` keep it but move or retype the storage
+        return [(t.data_ptr(), t.dtype, t._version) for t in self._tensors]
+
     def parameters_unchanged(self):
-        """False once any parameter of the model was updated in place after the capture."""
-        return all(p._version == v for p, v in zip(self._params, self._versions))
+        """False once any parameter or buffer of the model was updated in place, moved or retyped after the capture (the
+        graphs hold the old storage's addresses and copies derived from the old values)."""
+        return self._tensor_signature() == self._signature
 
     def replay(self):
         if not self.parameters_unchanged():

@@ -123,7 +123,8 @@ class SS2D(nn.Module):
         four batch sizes.
 
         Under a graph capture the kernels record the addresses of these tensors.  An entry the capture reads is therefore
-        moved to ``_pinned_consts``, which never evicts, so it outlives any graph that holds its address; an entry
+        moved to ``_pinned_consts``, which keeps it while the parameters stay as they are (entries for other parameter values are
+        dropped when a new one is pinned), so it outlives any graph that may still be replayed; an entry
         missing during a capture is computed inside the graph (its memory then belongs to the graph and is rewritten by
         every replay) and is not kept.  Pinned entries are copies of the parameter values at capture time: whoever
         replays the graph must not do so after an in-place parameter update (ConcurrentGraphRunner.replay checks)."""
@@ -136,6 +137,11 @@ class SS2D(nn.Module):
             return pinned[key]
         if key in cache:
             if capturing:
+                # entries pinned for other parameter values belong to graphs that must not be replayed any more
+                # (ConcurrentGraphRunner.replay refuses them): dropping them here keeps re-captures after weight
+                # updates from piling up one set of batch-replicated weights each
+                for k in [k for k in pinned if k[2] != key[2]]:
+                    del pinned[k]
                 pinned[key] = cache.pop(key)
                 return pinned[key]
             return cache[key]
