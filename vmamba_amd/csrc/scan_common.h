@@ -178,6 +178,16 @@ __device__ __forceinline__ float softplus_log2(float z) {
     return fmaf(__builtin_fmaxf(z, 0.0f), kLn2, fmaf(kLn2, __builtin_amdgcn_logf(w), c));
 }
 
+// softplus(x) / ln 2 for z = x * log2e:  max(z, 0) + log2(1 + 2^-|z|), without the compensation term of softplus_log2.
+// 1 + t is rounded to fp32, which changes the result by at most 2^-24 * log2e in absolute terms: invisible unless the
+// step itself is below ~1e-4, where 16-bit inputs have long lost it in their own rounding (a bf16 delta of -10 is known
+// to 3 %).  For kernels whose delta arrives as bf16 / fp16 and whose time is their instruction count; results stay in
+// units of ln 2 (the recurrence is linear in the step, so the factor is applied once to the output).
+__device__ __forceinline__ float softplus_over_ln2(float z) {
+    const float t = __builtin_amdgcn_exp2f(-__builtin_fabsf(z));
+    return __builtin_fmaxf(z, 0.0f) + __builtin_amdgcn_logf(1.0f + t);
+}
+
 template <bool kSoftplus>
 __device__ __forceinline__ void delta_transform(const float (&raw)[kItems], const float (&bias)[kItems],
                                                 float (&dl)[kItems]) {

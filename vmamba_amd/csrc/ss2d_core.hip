@@ -98,6 +98,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     constexpr int kBlocks = kIt / kItems;
     constexpr int kGroups = kIt / kGran;
     constexpr int kPassLen = kWave * kIt;                // positions per pass
+    // 16-bit streams with softplus: the step is kept in units of ln 2 (softplus_over_ln2), the decay is then
+    // 2^(step * A) with A as given, the planes collect y / ln 2 and the merge multiplies by ln 2 once per position
+    constexpr bool kBits = kSoftplus && sizeof(in_t) == 2;
     using Loads = CorePassLoads<in_t, kGran, kWide>;
     const int L = p.L, H = p.H;
     const int n_max = p.CB * L;
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bm), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Cm), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     const uint32_t B_soff = (uint32_t)(dir * p.B_ks + b0 * p.B_bs), C_soff = (uint32_t)(dir * p.C_ks + b0 * p.C_bs);
-    const float A_log2e = p.A[kd] * kLog2e;
+    const float A_log2e = kBits ? p.A[kd] : p.A[kd] * kLog2e;
     const float bias = p.bias ? p.bias[kd] : 0.0f;
     const bool reverse = dir >= 2;                       // uniform per wavefront
     const uint32_t u_sel = reverse ? 0x05040706u : 0x03020100u;
@@ -274,21 +277,27 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         bool valid;        // inside the stream
     };
 
-    // One pass: C * h of its items in yv (scan order) and the plane slots of its groups.  The skip term D * u is the
-    // same multiple of x[r] in all four directions and is added once, in the merge.
+    // One pass: the states h of its items in yv (scan order) and the plane slots of its groups; the plane update
+    // multiplies by C as it adds.  The skip term D * u is the same multiple of x[r] in all four directions and is added
+    // once, in the merge.
     auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kIt], GroupSlot (&slot)[kGroups]) {
         const int e0 = pass * kPassLen + lane * kIt;
         const int j0 = (int)r.j0;
         const int k = kGran == kIt ? kIt : min(kIt, L - j0);
         const int img_base = (int)r.img;
-        float dl[kIt], Bv[kIt], Cv[kIt], uv[kIt];
+        float dl[kIt], Bv[kIt], uv[kIt];
 #pragma unroll
         for (int blk = 0; blk < kBlocks; ++blk) {
             float raw8[kItems], bias8[kItems], dl8[kItems];
             unpack_raw<in_t>(r.dl[blk], raw8);
+            if constexpr (kBits) {
 #pragma unroll
-            for (int i = 0; i < kItems; ++i) bias8[i] = bias;
-            delta_transform<kSoftplus>(raw8, bias8, dl8);
+                for (int i = 0; i < kItems; ++i) dl8[i] = softplus_over_ln2(fmaf(raw8[i], kLog2e, bias * kLog2e));
+            } else {
+#pragma unroll
+                for (int i = 0; i < kItems; ++i) bias8[i] = bias;
+                delta_transform<kSoftplus>(raw8, bias8, dl8);
+            }
 #pragma unroll
             for (int i = 0; i < kItems; ++i) dl[blk * kItems + i] = dl8[i];
         }
@@ -299,11 +308,10 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
             const int jg = in_a ? j0 + gi * kGran : gi * kGran - k;          // position of the group in its image
             const int img_off = in_a ? img_base : img_base + L;              // img * L
             first[gi] = jg == 0;
-            float bg[kGran], cg[kGran];
+            float bg[kGran];
             unpack_group<in_t, kGran>(r.b[gi], bg);
-            unpack_group<in_t, kGran>(r.c[gi], cg);
 #pragma unroll
-            for (int i = 0; i < kGran; ++i) { Bv[gi * kGran + i] = bg[i]; Cv[gi * kGran + i] = cg[i]; }
+            for (int i = 0; i < kGran; ++i) Bv[gi * kGran + i] = bg[i];
             // The group's kGran logical indices in this direction's order are consecutive and kGran-aligned (L and
             // every group start are multiples of kGran): forwards they are the stream positions e0 + gi*kGran + t,
             // backwards img*L + L-1 - (jg + t), i.e. the block starting at img*L + L - jg - kGran read downwards.
@@ -349,23 +357,28 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         const float s_in = fmaf(a_ex, h_carry, h_ex);
         h_carry = fmaf(a_tot, h_carry, h_tot);
 #pragma unroll
-        for (int i = 0; i < kIt; ++i) yv[i] = Cv[i] * fmaf(ac[i], s_in, hh[i]);
+        for (int i = 0; i < kIt; ++i) yv[i] = fmaf(ac[i], s_in, hh[i]);
     };
 
     // Plane update of one pass: every entry is reached once by the forward and once by the backward direction of its
-    // plane; both add to the zero-initialised entry, so it ends as fl(y_fwd + y_bwd) whatever the order.  Only when the
-    // two meet in the same pass could the read-add-write sequences overlap: the barrier between the two halves of a
-    // pass keeps them apart.
-    auto update_plane = [&](bool reverse, const float (&yv)[kIt], const GroupSlot (&slot)[kGroups]) {
+    // plane; each adds its C * h to the zero-initialised entry with one fused multiply-add, so the entry ends as the
+    // sum of the two outputs whatever the order (the first addition, into a zero, is the rounded product itself).  Only
+    // when the two meet in the same pass could the read-add-write sequences overlap: the barrier between the two halves
+    // of a pass keeps them apart.  C is widened here, from the registers it arrived in.
+    auto update_plane = [&](bool reverse, const Loads &r, const float (&hv)[kIt], const GroupSlot (&slot)[kGroups]) {
 #pragma unroll
         for (int gi = 0; gi < kGroups; ++gi) {
             if (slot[gi].valid) {
                 float *dst = plane + slot[gi].plane_idx;
-                float old[kGran];
+                float old[kGran], cg[kGran];
 #pragma unroll
                 for (int c = 0; c < kGran; ++c) old[c] = dst[c];
+                unpack_group<in_t, kGran>(r.c[gi], cg);
 #pragma unroll
-                for (int c = 0; c < kGran; ++c) dst[c] = old[c] + (reverse ? yv[gi * kGran + kGran - 1 - c] : yv[gi * kGran + c]);
+                for (int c = 0; c < kGran; ++c) {
+                    const int it = reverse ? kGran - 1 - c : c;
+                    dst[c] = fmaf(cg[it], hv[gi * kGran + it], old[c]);
+                }
             }
         }
     };
@@ -385,7 +398,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
             Cv = gather_elem<in_t>(C_rsrc, C_soff + i * (uint32_t)p.C_bs + jj);
             u = to_f32(xs[map_index<kEs, kFlat>(base)]);
         }
-        float dl = kSoftplus ? softplus_log2(fmaf(raw, kLog2e, bias * kLog2e)) : raw + bias;
+        float dl;
+        if constexpr (kBits) dl = softplus_over_ln2(fmaf(raw, kLog2e, bias * kLog2e));
+        else dl = kSoftplus ? softplus_log2(fmaf(raw, kLog2e, bias * kLog2e)) : raw + bias;
         dl = valid ? dl : 0.0f;
         float a = __builtin_amdgcn_exp2f(dl * A_log2e);
         a = (valid && jj == 0) ? 0.0f : a;                                   // an image starts: the state restarts
@@ -393,11 +408,10 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         float a_ex, h_ex, a_tot, h_tot;
         wave_scan_pairs(a, b, a_ex, h_ex, a_tot, h_tot);
         const float h = fmaf(a, fmaf(a_ex, h_carry, h_ex), b);
-        const float y = Cv * h;
         float *dst = plane + lds_index<4>(base);
-        if (!reverse && valid) *dst += y;
+        if (!reverse && valid) *dst = fmaf(Cv, h, *dst);
         __syncthreads();
-        if (reverse && valid) *dst += y;
+        if (reverse && valid) *dst = fmaf(Cv, h, *dst);
         __syncthreads();
     };
 
@@ -411,9 +425,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
                     float yv[kIt];
                     GroupSlot slot[kGroups];
                     compute(reverse, pass, regs[q], h_carry, yv, slot);
-                    if (!reverse) update_plane(false, yv, slot);
+                    if (!reverse) update_plane(false, regs[q], yv, slot);
                     __syncthreads();
-                    if (reverse) update_plane(true, yv, slot);
+                    if (reverse) update_plane(true, regs[q], yv, slot);
                     __syncthreads();
                     if (pass + kCoreBurst < n_pass) issue(pass + kCoreBurst, regs[q]);
                 }
@@ -426,6 +440,11 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     float Dsum = 0.0f;
     if (p.Dv) Dsum = (p.Dv[d] + p.Dv[2 * p.D + (int)d]) + (p.Dv[p.D + (int)d] + p.Dv[3 * p.D + (int)d]);
     float *yo = reinterpret_cast<float *>(p.y);
+    // (sum of the two planes, x) -> output: the planes hold y / ln 2 when the step was kept in units of ln 2
+    auto finish = [&](float planes, float xv) {
+        if constexpr (kBits) return fmaf(planes, kLn2, Dsum * xv);
+        else return fmaf(Dsum, xv, planes);
+    };
     if (p.tile_merge) {
         // H and W multiples of 4, y 16-byte aligned (host-checked): one 4 x 4 tile of a map per thread.  Its rows are
         // four consecutive entries of plane A each, its columns four consecutive entries of plane B each -- the
@@ -451,8 +470,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 *reinterpret_cast<float4 *>(dst + k * p.W) =
-                    make_float4(fmaf(Dsum, x[k][0], a[k][0] + b[0][k]), fmaf(Dsum, x[k][1], a[k][1] + b[1][k]),
-                                fmaf(Dsum, x[k][2], a[k][2] + b[2][k]), fmaf(Dsum, x[k][3], a[k][3] + b[3][k]));
+                    make_float4(finish(a[k][0] + b[0][k], x[k][0]), finish(a[k][1] + b[1][k], x[k][1]),
+                                finish(a[k][2] + b[2][k], x[k][2]), finish(a[k][3] + b[3][k], x[k][3]));
         }
         return;
     }
@@ -476,7 +495,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
                 float o[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    o[c] = fmaf(Dsum, to_f32(px[c]), pa[c] + planeB[lds_index<4>((c < n_first ? t0 : t1) + c * H)]);
+                    o[c] = finish(pa[c] + planeB[lds_index<4>((c < n_first ? t0 : t1) + c * H)], to_f32(px[c]));
                 v[u] = make_float4(o[0], o[1], o[2], o[3]);
                 off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
             }
@@ -495,8 +514,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
             uint32_t i, r, h, w;
             divmod((uint32_t)idx, divL, i, r);
             divmod(r, divW, h, w);
-            v[u] = fmaf(Dsum, to_f32(xR[map_index<kEs, kFlat>(idx)]),
-                        planeA[lds_index<4>(idx)] + planeB[lds_index<4>((int)(i * L + w * H + h))]);
+            v[u] = finish(planeA[lds_index<4>(idx)] + planeB[lds_index<4>((int)(i * L + w * H + h))],
+                          to_f32(xR[map_index<kEs, kFlat>(idx)]));
             off[u] = ((size_t)(b0 + i) * p.D + d) * L + r;
         }
 #pragma unroll

@@ -157,7 +157,9 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
         Cv.read(s_bc + (2 * kDir + 1) * kTileElems, run);
 
         const int kd = kDir * p.D + d;
-        const float A2 = p.A[kd] * kLog2e;
+        // with softplus the step is kept in units of ln 2 (softplus_over_ln2): the decay is 2^(step * A) with A as given,
+        // the sums collect y / ln 2 and the merge multiplies by ln 2 once per position
+        const float A2 = kSoftplus ? p.A[kd] : p.A[kd] * kLog2e;
         const float bias = p.bias ? p.bias[kd] : 0.0f;
         const bool first = kRev ? i == kS - 1 : i == 0;      // the lane that starts the map in this direction's order
         float ac[kS], hh[kS];
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
             const int m = kRev ? kS - 1 - j : j;             // column (directions 0 / 2) or row (1 / 3) of item j
             const float u = kCol ? x_col.item(m) : x_row.item(m);
             float dl;
-            if constexpr (kSoftplus) dl = softplus_log2(fmaf(raw.item(j), kLog2e, bias * kLog2e));
+            if constexpr (kSoftplus) dl = softplus_over_ln2(fmaf(raw.item(j), kLog2e, bias * kLog2e));
             else dl = raw.item(j) + bias;
             float a = __builtin_amdgcn_exp2f(dl * A2);
             if (j == 0) a = first ? 0.0f : a;                // nothing enters a map from the lanes before it
@@ -201,7 +203,10 @@ __global__ __launch_bounds__(kBlock, kS <= 8 ? 5 : 4) void ss2d_core_small_kerne
     wave_lds_sync();
     float out[kS];
 #pragma unroll
-    for (int j = 0; j < kS; ++j) out[j] = fmaf(Dsum, x_row.item(j), acc[j] + tile_tr[gc * kL + ic * kS + j]);
+    for (int j = 0; j < kS; ++j) {
+        const float sums = acc[j] + tile_tr[gc * kL + ic * kS + j];
+        out[j] = kSoftplus ? fmaf(sums, kLn2, Dsum * x_row.item(j)) : fmaf(Dsum, x_row.item(j), sums);
+    }
     if (active) {
         float *yo = reinterpret_cast<float *>(p.y) + ((int64_t)(b0 + g) * p.D + d) * kL + i * kS;
         if constexpr (kS % 2 == 0) {
