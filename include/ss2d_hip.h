@@ -256,6 +256,20 @@ typedef struct ss2d_core_params {
 int ss2d_core_fwd(const ss2d_core_params *params, void *stream);
 
 /*
+ * The same operator for maps of any size.  Maps that do not fit the single kernel's LDS arrays (e.g. the 256 x 256 and
+ * 128 x 128 maps of a 1024 x 1024 image) are cut into 64 x 64 tiles and walked twice -- per-run aggregates, a carry scan
+ * over them, then the outputs -- which needs scratch memory: ss2d_core_workspace_bytes returns how much (0 when the
+ * single kernel serves the problem and no workspace is needed, SS2D_ENOTSUP when neither path does: the tiled one takes
+ * 16-bit inputs, height and width multiples of 8, every stride a multiple of 8 elements and 16-byte aligned
+ * pointers), and ss2d_core_fwd_ws takes that workspace (16-byte aligned device memory; SS2D_ENOMEM when it is too
+ * small; contents need no initialisation and mean nothing afterwards).  The reference reaches every length with one
+ * kernel by looping over 2048-position chunks (selective_scan_fwd_kernel_oflex.cuh:110-111, 156-167;
+ * selective_scan_oflex.cpp:206); results as ss2d_core_fwd.
+ */
+int64_t ss2d_core_workspace_bytes(const ss2d_core_params *params);
+int ss2d_core_fwd_ws(const ss2d_core_params *params, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * CrossScan / CrossMerge for every layout and mode of the reference operators (cross_scan_fn / cross_merge_fn,
  * classification/models/csm_triton.py:501-517; semantics of the flex kernel :278-400 and of the torch functions
  * :22-179).  Flags are named from the scan's side, as in the reference, for both operations:

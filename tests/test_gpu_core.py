@@ -140,6 +140,95 @@ def test_core_small_maps_contiguous_streams_end_at_the_allocation(B):
     assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
 
 
+# Maps that do not fit the single kernel's LDS arrays: 64 x 64 tiles, walked twice with a carry scan in between
+# (16-bit inputs, sides multiples of 8).  Whole tiles; edge tiles narrower / shorter than 64; a single row or column of
+# tiles; maps with fewer than 64 rows; several images and channels.
+TILED_SHAPES = [
+    (1, 2, 128, 128), (2, 3, 80, 72), (1, 1, 64, 200), (1, 2, 256, 256), (2, 2, 8, 1024), (1, 2, 136, 64), (3, 1, 96, 104),
+    (1, 1, 1000, 8),
+]
+
+
+def core_workspace_bytes(B, D, H, W, dtype=torch.bfloat16):
+    """ss2d_core_workspace_bytes for dense, aligned tensors of these sizes (the query reads the struct only)."""
+    p = _lib.CoreParams()
+    p.batch, p.dim, p.height, p.width = B, D, H, W
+    p.in_dtype = {torch.float32: _lib.SS2D_F32, torch.bfloat16: _lib.SS2D_BF16, torch.float16: _lib.SS2D_F16}[dtype]
+    p.delta_softplus = 1
+    p.x, p.delta, p.A, p.B, p.C, p.y = (4096 * k for k in range(1, 7))
+    L = H * W
+    p.delta_dir_stride, p.delta_dim_stride, p.delta_batch_stride = D * B * L, B * L, L
+    p.B_dir_stride, p.B_batch_stride, p.C_dir_stride, p.C_batch_stride = B * L, L, B * L, L
+    return _lib.lib().ss2d_core_workspace_bytes(p)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("shape", TILED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_core_large_maps_in_tiles_match_oracle_composition(shape, dtype):
+    _announce("core tiled", shape, dtype)
+    assert core_workspace_bytes(*shape, dtype) > 0            # the two-pass path, not the single kernel
+    args = make_core_inputs(sum(shape), *shape, dtype)
+    want = oracle_core(*args)
+    got = run_core(*args)
+    assert got.dtype == torch.float32 and got.shape == want.shape
+    # rows of up to 65536 positions: the absolute part scales with the output (the state remembers ~1 / (dt |A|) steps)
+    tol = dict(rtol=1e-3, atol=max(4e-4, 2e-5 * want.abs().max().item()))
+    err = (got - want).abs().max().item()
+    assert torch.allclose(got, want, **tol), f"max abs err {err}"
+
+
+def test_core_tiled_optional_arguments_and_workspace_contract():
+    _announce("core tiled optional")
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(77, 2, 2, 80, 88, torch.bfloat16)
+    g = torch.Generator().manual_seed(3)
+    delta_pos = (0.5 * torch.rand(delta.shape, generator=g)).to(delta.dtype)
+    bias_pos = 0.5 * torch.rand(bias.shape, generator=g)
+    for dl, dv, bi, sp in ((delta, None, bias, True), (delta, Dv, None, True), (delta_pos, Dv, bias_pos, False), (delta_pos, None, None, False)):
+        want = oracle_core(x, dl, Bs, Cs, A, dv, bi, sp)
+        got = run_core(x, dl, Bs, Cs, A, dv, bi, sp)
+        assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
+    # the workspace contract of the C ABI: 0 for maps the single kernel takes, a refusal where neither path applies,
+    # SS2D_ENOMEM for a workspace that is too small, and the plain entry point still refuses large maps
+    assert core_workspace_bytes(4, 8, 56, 56) == 0
+    assert core_workspace_bytes(1, 1, 97, 97) == _lib.SS2D_ENOTSUP            # sides not multiples of 8
+    assert core_workspace_bytes(1, 1, 96, 96, torch.float32) == _lib.SS2D_ENOTSUP
+    need = core_workspace_bytes(2, 2, 80, 88)
+    assert need == 4 * 2 * 2 * max(80 * 2, 88 * 2) * 12
+    dev = [t.to(DEV) for t in (x, delta, Bs, Cs, A, Dv, bias)]
+    y = torch.empty(2, 2, 80 * 88, device=DEV)
+    p = _lib.CoreParams()
+    p.batch, p.dim, p.height, p.width, p.in_dtype, p.delta_softplus = 2, 2, 80, 88, _lib.SS2D_BF16, 1
+    p.x, p.delta, p.B, p.C, p.A, p.D, p.delta_bias, p.y = (t.data_ptr() for t in dev + [y])
+    p.delta_dir_stride, p.delta_dim_stride, p.delta_batch_stride = dev[1].stride(0), dev[1].stride(1), dev[1].stride(2)
+    p.B_dir_stride, p.B_batch_stride, p.C_dir_stride, p.C_batch_stride = dev[2].stride(0), dev[2].stride(1), dev[3].stride(0), dev[3].stride(1)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert _lib.lib().ss2d_core_fwd(p, stream) == _lib.SS2D_ENOTSUP
+    assert _lib.lib().ss2d_core_fwd_ws(p, ws.data_ptr(), need - 1, stream) == _lib.SS2D_ENOMEM
+    assert _lib.lib().ss2d_core_fwd_ws(p, None, need, stream) == _lib.SS2D_EINVAL
+    assert _lib.lib().ss2d_core_fwd_ws(p, ws.data_ptr(), need, stream) == _lib.SS2D_OK
+    torch.cuda.synchronize()
+    assert torch.allclose(y.cpu(), oracle_core(x, delta, Bs, Cs, A, Dv, bias), **TOL)
+
+
+def test_core_tiled_equals_three_kernels_at_config4_shapes():
+    """The stage-1 and stage-2 maps of four 1024 x 1024 images (256 x 256 and 128 x 128), full size: the tiled kernels
+    against this package's own cross_scan / scan / merge kernels, which the oracle pins at smaller sizes."""
+    for (B, D, H, W) in ((4, 96, 256, 256), (4, 192, 128, 128)):
+        _announce("core tiled vs kernels", B, D, H, W)
+        x, delta, Bs, Cs, A, Dv, bias = [t.to(DEV) for t in make_core_inputs(B + D, B, D, H, W, torch.bfloat16)]
+        L = H * W
+        xs = va.cross_scan_fn(x)
+        ys = va.selective_scan_fn(xs.view(B, 4 * D, L), delta.permute(2, 0, 1, 3).reshape(B, 4 * D, L), A.view(4 * D, 1),
+                                  Bs.permute(1, 0, 2).unsqueeze(2), Cs.permute(1, 0, 2).unsqueeze(2), Dv, bias, True, True)
+        want = va.cross_merge_fn(ys.view(B, 4, D, H, W))
+        got = ss2d_core_hip(x, delta, Bs, Cs, A, Dv, bias, True)
+        torch.cuda.synchronize()
+        tol = dict(rtol=1e-3, atol=max(4e-4, 2e-5 * want.abs().max().item()))
+        err = (got - want).abs().max().item()
+        assert torch.allclose(got, want, **tol), f"max abs err {err}"
+
+
 @pytest.mark.parametrize("softplus", [True, False])
 def test_core_optional_arguments(softplus):
     _announce("core optional", softplus)
@@ -289,8 +378,8 @@ def test_core_rejections():
         ss2d_core_hip(x, delta.float(), Bs, Cs, A, Dv, bias)
     with pytest.raises(RuntimeError):
         ss2d_core_hip(x.cpu(), delta, Bs, Cs, A, Dv, bias)
-    # image too large for the LDS planes: a clean "not supported", never a launch
-    big = [t.to(DEV) for t in make_core_inputs(1, 1, 1, 96, 96, torch.bfloat16)]
+    # image too large for the LDS planes with sides the tiled kernels do not take: a clean "not supported", never a launch
+    big = [t.to(DEV) for t in make_core_inputs(1, 1, 1, 97, 97, torch.bfloat16)]
     with pytest.raises(_lib.Ss2dError) as e:
         ss2d_core_hip(*big)
     assert e.value.code == _lib.SS2D_ENOTSUP

@@ -22,14 +22,17 @@ def _lds_extent(n, es):
 
 
 def core_fits(H, W, dtype):
-    """True when ss2d_core_fwd takes an H x W image of this dtype: at least 8 positions, and the LDS arrays of one
-    image (two fp32 merge planes, two copies of the x map plus a block of 8 zeros each) within 64 KiB."""
+    """True when the fused core takes an H x W image of this dtype: at least 8 positions, and either the LDS arrays
+    of one image (two fp32 merge planes, two copies of the x map plus a block of 8 zeros each) within 64 KiB -- the single
+    kernel -- or 16-bit maps whose sides are multiples of 8, which the tiled two-pass kernels take at any size."""
     if dtype not in _DTYPE_CODE:
         return False
     L = H * W
     es = 4 if dtype == torch.float32 else 2
     maps = _lds_extent(((L + 7) & ~7) + 8, es)
-    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024
+    if L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024:
+        return True
+    return es == 2 and H % 8 == 0 and W % 8 == 0
 
 
 def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True, out=None):
@@ -37,8 +40,9 @@ def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus
     scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32 (written into
     ``out`` when given: a contiguous fp32 tensor of that shape).
 
-    Raises Ss2dError with status SS2D_ENOTSUP when the shape has no fused kernel (image too large for the LDS
-    planes, unaligned delta rows): callers fall back to the three separate operators.
+    Raises Ss2dError with status SS2D_ENOTSUP when the shape has no fused kernel (an image too large for the LDS
+    planes that the tiled kernels do not take either: fp32, sides not multiples of 8, unaligned rows): callers fall
+    back to the three separate operators.
     """
     _check(x.is_cuda, "ss2d_core: vmamba_amd runs on the GPU only")
     _check(x.dim() == 4, "x must be (B, D, H, W)")
@@ -78,7 +82,15 @@ def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus
     p.B_dir_stride, p.B_batch_stride = Bs.stride(0), Bs.stride(1)
     p.C_dir_stride, p.C_batch_stride = Cs.stride(0), Cs.stride(1)
     with torch.cuda.device(x.device):
-        rc = _lib.lib().ss2d_core_fwd(p, torch.cuda.current_stream(x.device).cuda_stream)
+        # maps too large for the single kernel are walked in tiles, twice, through scratch memory of the size the library asks for
+        need = _lib.lib().ss2d_core_workspace_bytes(p)
+        _lib.check(min(need, 0), "ss2d_core_workspace_bytes")
+        stream = torch.cuda.current_stream(x.device).cuda_stream
+        if need > 0:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+            rc = _lib.lib().ss2d_core_fwd_ws(p, workspace.data_ptr(), need, stream)
+        else:
+            rc = _lib.lib().ss2d_core_fwd(p, stream)
     _lib.check(rc, "ss2d_core_fwd")
     return y
 

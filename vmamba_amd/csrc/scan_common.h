@@ -52,6 +52,12 @@ int launch_scan_small(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_
 bool core_small_eligible(const CoreArgs &a, int in_dtype);
 int launch_core_small(const CoreArgs &a, int in_dtype, hipStream_t stream);
 
+// ss2d_core_tiled.hip: the fused core for maps of any size (64 x 64 tiles, two passes and a carry scan; 16-bit inputs,
+// map sides multiples of 8).  The workspace holds the runs' aggregates and carries.
+bool core_tiled_eligible(const CoreArgs &a, int in_dtype);
+int64_t core_tiled_workspace_bytes(const CoreArgs &a);
+int launch_core_tiled(const CoreArgs &a, int in_dtype, void *workspace, hipStream_t stream);
+
 // ---- 8-wide loads / stores ------------------------------------------------------------
 // Eight consecutive elements of a row as they sit in registers before widening: 4 dwords for 16-bit
 // types, 8 for fp32.  Keeping loads in this form lets a pass issue the NEXT pass's loads before it

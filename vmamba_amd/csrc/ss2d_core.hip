@@ -536,17 +536,29 @@ template <typename in_t> static size_t lds_bytes_of(int64_t n64, bool flat) {
     return 2 * (size_t)lds_extent<4>(n) * sizeof(float) + 2 * (size_t)map_ext * sizeof(in_t);
 }
 
+// Granularity of the B / C gathers and of the walk: the largest of 8, 4, 1 positions that divides L and every B / C
+// stride and for which the B / C bases are aligned.
 template <typename in_t>
-static int launch_core(CoreArgs a, hipStream_t stream) {
-    const int64_t L = a.L;
-    // Granularity of the B / C gathers and of the walk: the largest of 8, 4, 1 positions that divides L and every B / C
-    // stride and for which the B / C bases are aligned.
-    int64_t g = core_gcd(L, kItems);
+static int64_t core_granularity(const CoreArgs &a) {
+    int64_t g = core_gcd(a.L, kItems);
     const int64_t strides[] = {a.B_ks, a.B_bs, a.C_ks, a.C_bs};
     for (int64_t s : strides) g = core_gcd(g, s == 0 ? g : s);
     const uintptr_t bases = reinterpret_cast<uintptr_t>(a.Bm) | reinterpret_cast<uintptr_t>(a.Cm);
     while (g > 1 && (bases % (uintptr_t)(g * sizeof(in_t))) != 0) g /= 2;
-    if (g == 2) g = 1;
+    return g == 2 ? 1 : g;
+}
+
+// True when one image of this problem fits the LDS arrays of ss2d_core_kernel.
+template <typename in_t>
+static bool core_fits_lds(const CoreArgs &a) {
+    const bool flat = sizeof(in_t) == 2 && core_granularity<in_t>(a) == kItems;
+    return lds_bytes_of<in_t>(a.L, flat) <= kCoreMaxLds;
+}
+
+template <typename in_t>
+static int launch_core(CoreArgs a, hipStream_t stream) {
+    const int64_t L = a.L;
+    const int64_t g = core_granularity<in_t>(a);
     const bool flat = sizeof(in_t) == 2 && g == kItems;       // core_flat_maps
     // 16 positions per lane and pass where one image alone takes more LDS than a sixth of a CU (the tile cannot be
     // shortened, six workgroups per CU are out of reach anyway); else 8, with tiles that let six workgroups share a CU
@@ -612,19 +624,19 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
 
 }  // namespace ss2d
 
-extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
-    using namespace ss2d;
+namespace ss2d {
+
+// Validation shared by the core's entry points.  Returns SS2D_OK with `a` filled, 1 for an empty problem, or a negative status.
+static int core_args(const ss2d_core_params *q, CoreArgs &a) {
     if (!q) return SS2D_EINVAL;
     if (q->batch < 0 || q->dim < 0 || q->height < 0 || q->width < 0) return SS2D_EINVAL;
     if (q->in_dtype != SS2D_F32 && q->in_dtype != SS2D_BF16 && q->in_dtype != SS2D_F16) return SS2D_EINVAL;
-    if (q->batch == 0 || q->dim == 0 || q->height == 0 || q->width == 0) return SS2D_OK;
+    if (q->batch == 0 || q->dim == 0 || q->height == 0 || q->width == 0) return 1;
     if (!q->x || !q->delta || !q->A || !q->B || !q->C || !q->y) return SS2D_EINVAL;
     const int64_t L = (int64_t)q->height * q->width;
     if (L < kItems || L > 0x0fffffff) return SS2D_ENOTSUP;
     if (q->delta_batch_stride < 0 || q->delta_dir_stride < 0 || q->delta_dim_stride < 0 || q->B_dir_stride < 0 ||
         q->B_batch_stride < 0 || q->C_dir_stride < 0 || q->C_batch_stride < 0) return SS2D_EINVAL;
-
-    CoreArgs a;
     a.x = q->x; a.delta = q->delta; a.Bm = q->B; a.Cm = q->C;
     a.A = (const float *)q->A; a.Dv = (const float *)q->D; a.bias = (const float *)q->delta_bias;
     a.y = q->y;
@@ -640,13 +652,54 @@ extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
     if (B_span >= 0x7fffffffll || C_span >= 0x7fffffffll) return SS2D_ENOTSUP;
     a.B_span_bytes = (uint32_t)B_span; a.C_span_bytes = (uint32_t)C_span;
     a.CB = 1; a.vec_ok = 0; a.vec_out = 0; a.stage_tiles = 0; a.tile_merge = 0;
+    return SS2D_OK;
+}
 
-    hipStream_t s = (hipStream_t)stream;
+// True when the single-kernel core (whole maps in LDS) takes this problem.
+static bool core_single_kernel(const CoreArgs &a, int in_dtype) {
+    if (core_small_eligible(a, in_dtype)) return true;
+    return in_dtype == SS2D_F32 ? core_fits_lds<float>(a) : core_fits_lds<bf16_t>(a);
+}
+
+static int core_launch_single(const CoreArgs &a, int in_dtype, hipStream_t s) {
     // 7 x 7 and 14 x 14 maps in the batch-innermost layout: one map row per lane, everything in registers
-    if (core_small_eligible(a, q->in_dtype)) return launch_core_small(a, q->in_dtype, s);
-    if (q->in_dtype == SS2D_F32) return launch_core<float>(a, s);
-    if (q->in_dtype == SS2D_BF16) return launch_core<bf16_t>(a, s);
+    if (core_small_eligible(a, in_dtype)) return launch_core_small(a, in_dtype, s);
+    if (in_dtype == SS2D_F32) return launch_core<float>(a, s);
+    if (in_dtype == SS2D_BF16) return launch_core<bf16_t>(a, s);
     return launch_core<f16_t>(a, s);
+}
+
+}  // namespace ss2d
+
+extern "C" int ss2d_core_fwd(const ss2d_core_params *q, void *stream) {
+    using namespace ss2d;
+    CoreArgs a;
+    const int rc = core_args(q, a);
+    if (rc != SS2D_OK) return rc > 0 ? SS2D_OK : rc;
+    return core_launch_single(a, q->in_dtype, (hipStream_t)stream);
+}
+
+extern "C" int64_t ss2d_core_workspace_bytes(const ss2d_core_params *q) {
+    using namespace ss2d;
+    CoreArgs a;
+    const int rc = core_args(q, a);
+    if (rc != SS2D_OK) return rc > 0 ? 0 : rc;
+    if (core_single_kernel(a, q->in_dtype)) return 0;
+    if (!core_tiled_eligible(a, q->in_dtype)) return SS2D_ENOTSUP;
+    return core_tiled_workspace_bytes(a);
+}
+
+extern "C" int ss2d_core_fwd_ws(const ss2d_core_params *q, void *workspace, int64_t workspace_bytes, void *stream) {
+    using namespace ss2d;
+    CoreArgs a;
+    const int rc = core_args(q, a);
+    if (rc != SS2D_OK) return rc > 0 ? SS2D_OK : rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (core_single_kernel(a, q->in_dtype)) return core_launch_single(a, q->in_dtype, s);
+    if (!core_tiled_eligible(a, q->in_dtype)) return SS2D_ENOTSUP;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) % 16) != 0) return SS2D_EINVAL;
+    if (workspace_bytes < core_tiled_workspace_bytes(a)) return SS2D_ENOMEM;
+    return launch_core_tiled(a, q->in_dtype, workspace, s);
 }
 
 // ---- CrossScan, one-by-one --------------------------------------------------------------
