@@ -270,6 +270,19 @@ int64_t ss2d_core_workspace_bytes(const ss2d_core_params *params);
 int ss2d_core_fwd_ws(const ss2d_core_params *params, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Maps whose sides do not suit the core's vector paths (57 x 58 -- the reference's own check size,
+ * classification/models/csm_triton.py:524, 670 -- 75 x 75, 19 x 19 ...) can be embedded by the caller in a map of
+ * padded_height x padded_width >= height x width: x = 0 on the added rows / columns, the projections computed on the
+ * padded map, and the step made 0 on the added positions, which makes them neutral elements of the scan (decay 1,
+ * drive 0): the outputs at the original positions are those of the original map.  This call writes delta = -infinity
+ * (softplus(-inf + bias) = 0) at the added positions of each direction's scan order; delta as in ss2d_core_params,
+ * over the padded map; delta_softplus must be on.  No counterpart in the reference, whose kernels take any length
+ * element by element.
+ */
+int ss2d_core_mask_pads(void *delta, int batch, int dim, int height, int width, int padded_height, int padded_width,
+                        int64_t delta_dir_stride, int64_t delta_dim_stride, int64_t delta_batch_stride, int dtype, void *stream);
+
+/*
  * CrossScan / CrossMerge for every layout and mode of the reference operators (cross_scan_fn / cross_merge_fn,
  * classification/models/csm_triton.py:501-517; semantics of the flex kernel :278-400 and of the torch functions
  * :22-179).  Flags are named from the scan's side, as in the reference, for both operations:

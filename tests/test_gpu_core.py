@@ -211,6 +211,68 @@ def test_core_tiled_optional_arguments_and_workspace_contract():
     assert torch.allclose(y.cpu(), oracle_core(x, delta, Bs, Cs, A, Dv, bias), **TOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
+@pytest.mark.parametrize("sizes", [(57, 58, 60, 60), (19, 19, 20, 20), (9, 13, 16, 16), (75, 75, 80, 80), (8, 8, 8, 16), (5, 3, 8, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_core_mask_pads_marks_exactly_the_added_positions(sizes, dtype):
+    """ss2d_core_mask_pads: -inf at the scan positions of every direction that fall on added rows / columns, nothing else
+    touched.  The expected positions come from the oracle's CrossScan applied to a 0 / 1 picture of the padded map."""
+    from vmamba_amd.core import core_mask_pads_hip
+    H, W, Hp, Wp = sizes
+    _announce("mask pads", sizes, dtype)
+    D, B = 3, 2
+    g = torch.Generator().manual_seed(H * W)
+    delta = torch.randn(4, D, B + 1, Hp * Wp, generator=g).to(dtype)          # a batch-padded buffer, sliced
+    picture = torch.ones(1, 1, Hp, Wp)
+    picture[:, :, :H, :W] = 0
+    marks = orc.cross_scan(picture).view(4, Hp * Wp).bool()                   # (direction, scan position): added or not
+    dev = delta.to(DEV)
+    core_mask_pads_hip(dev[:, :, :B], H, W, Hp, Wp)
+    torch.cuda.synchronize()
+    got = dev.cpu()
+    want = delta.clone()
+    want[:, :, :B] = torch.where(marks[:, None, None, :], torch.tensor(float("-inf")).to(dtype), delta[:, :, :B])
+    assert torch.equal(got.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       want.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("shape,padded", [((3, 2, 57, 58), (60, 60)), ((5, 3, 19, 19), (20, 20)), ((2, 2, 75, 75), (80, 80)),
+                                          ((2, 1, 25, 42), (28, 44)), ((1, 2, 100, 167), (104, 168))],
+                         ids=lambda v: "x".join(map(str, v)))
+def test_core_on_a_padded_map_equals_the_oracle_on_the_map_itself(shape, padded, dtype):
+    """The embedding SS2D.forward_core_fused uses for maps with awkward sides: x zero-padded, the streams given on the
+    padded map (B, C arbitrary on the added positions, delta -inf there through ss2d_core_mask_pads), the result cropped
+    -- against the oracle's composition on the ORIGINAL map with the original streams."""
+    from vmamba_amd.core import core_mask_pads_hip, padded_map_size
+    B, D, H, W = shape
+    Hp, Wp = padded
+    assert padded_map_size(H, W, dtype) == padded
+    _announce("core padded map", shape, padded, dtype)
+    g = torch.Generator().manual_seed(sum(shape))
+    # streams on the padded map, in natural (h, w) order first: (4, rows, B, Hp, Wp); the original map's streams are the crops
+    nat = lambda rows: torch.randn(4, rows, B, Hp, Wp, generator=g).to(dtype)
+    delta_nat, B_nat, C_nat = nat(D), nat(1), nat(1)
+    x, _, _, _, A, Dv, bias = make_core_inputs(sum(shape), B, D, H, W, dtype)
+
+    def in_scan_order(t, h, w):          # (4, rows, B, h, w) natural -> each direction slice in its own order: (4, rows, B, h*w)
+        rows = t.shape[1]
+        return torch_ref.cross_scan_1b1(t.permute(2, 0, 1, 3, 4).contiguous()).permute(1, 2, 0, 3).reshape(4, rows, B, h * w).contiguous()
+
+    crop = lambda t: t[..., :H, :W].contiguous()
+    want = oracle_core(x, in_scan_order(crop(delta_nat), H, W), in_scan_order(crop(B_nat), H, W)[:, 0],
+                       in_scan_order(crop(C_nat), H, W)[:, 0], A, Dv, bias)
+    x_pad = torch.nn.functional.pad(x, (0, Wp - W, 0, Hp - H))
+    delta_p = in_scan_order(delta_nat, Hp, Wp).to(DEV)
+    core_mask_pads_hip(delta_p, H, W, Hp, Wp)
+    got = ss2d_core_hip(x_pad.to(DEV), delta_p, in_scan_order(B_nat, Hp, Wp)[:, 0].to(DEV), in_scan_order(C_nat, Hp, Wp)[:, 0].to(DEV),
+                        A.to(DEV), Dv.to(DEV), bias.to(DEV), True)
+    torch.cuda.synchronize()
+    got = got.view(B, D, Hp, Wp)[:, :, :H, :W].reshape(B, D, H * W).cpu()
+    tol = dict(rtol=1e-3, atol=max(4e-4, 2e-5 * want.abs().max().item()))
+    assert torch.allclose(got, want, **tol), f"max abs err {(got - want).abs().max().item()}"
+
+
 def test_core_tiled_equals_three_kernels_at_config4_shapes():
     """The stage-1 and stage-2 maps of four 1024 x 1024 images (256 x 256 and 128 x 128), full size: the tiled kernels
     against this package's own cross_scan / scan / merge kernels, which the oracle pins at smaller sizes."""

@@ -15,7 +15,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libss2d_hip.so")
 HIP_SOURCES = ["cross_scan.hip", "cross_merge.hip", "selective_scan.hip", "scan_chan.hip", "scan_small.hip", "layer_norm.hip", "dwconv.hip",
-               "ss2d_core.hip", "ss2d_core_small.hip", "ss2d_core_tiled.hip", "dt_proj.hip", "cross_flex.hip",
+               "ss2d_core.hip", "ss2d_core_small.hip", "ss2d_core_tiled.hip", "core_pads.hip", "dt_proj.hip", "cross_flex.hip",
                "selective_scan_bwd.hip", "mlp_fused.hip", "linear_cl.hip", "stem_conv.hip", "mean_pool.hip"]
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 

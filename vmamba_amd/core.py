@@ -3,6 +3,8 @@
 Stands in for the three operator calls of SS2Dv2.forward_corev2 (classification/models/vmamba.py:604,
 625-633, 638) when the model has one state per channel; the projections between them remain the caller's.
 """
+import math
+
 import torch
 
 from . import _lib
@@ -29,10 +31,51 @@ def core_fits(H, W, dtype):
         return False
     L = H * W
     es = 4 if dtype == torch.float32 else 2
-    maps = _lds_extent(((L + 7) & ~7) + 8, es)
-    if L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024:
+    if _fits_single_kernel(L, es):
         return True
-    return es == 2 and H % 8 == 0 and W % 8 == 0
+    return es == 2 and ((H % 8 == 0 and W % 8 == 0) or padded_map_size(H, W, dtype) is not None)
+
+
+def _fits_single_kernel(L, es):
+    maps = _lds_extent(((L + 7) & ~7) + 8, es)
+    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024
+
+
+def padded_map_size(H, W, dtype):
+    """(H', W') >= (H, W) in which a caller should embed an H x W map for the fused core, or None when the map is fine
+    as it is (or padding would not pay).  16-bit maps only.  The core's vector paths want a number of positions that is
+    a multiple of 8 and, for the 4 x 4 tiles of its staging and merge, sides that are multiples of 4 (so: multiples of
+    4, whose product is a multiple of 16); maps beyond the single kernel's LDS arrays go to the tiled kernels, which want
+    multiples of 8.  Without them the core walks the map element by element at a third to a quarter of the rate, which a
+    padded area of up to 1.5 times the map's beats."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return None
+    L = H * W
+    if H == W == 7:                      # has a kernel of its own (one map row per lane)
+        return None
+    if _fits_single_kernel(L, 2):
+        if math.gcd(L, 8) >= 4:
+            return None
+        H4, W4 = (H + 3) & ~3, (W + 3) & ~3
+        if _fits_single_kernel(H4 * W4, 2):
+            return (H4, W4) if H4 * W4 <= 1.5 * L else None
+    if H % 8 == 0 and W % 8 == 0:
+        return None
+    H8, W8 = (H + 7) & ~7, (W + 7) & ~7
+    return (H8, W8) if H8 * W8 <= 1.5 * L else None
+
+
+def core_mask_pads_hip(delta, H, W, Hp, Wp):
+    """delta (4, D, B, Hp*Wp) view of the padded map's steps: -inf at the scan positions that fall on the rows >= H and the
+    columns >= W, in every direction's order (ss2d_core_mask_pads).  In place."""
+    _check(delta.is_cuda and delta.dim() == 4 and delta.shape[0] == 4 and delta.shape[3] == Hp * Wp, "delta must be (4, D, B, Hp*Wp) on the GPU")
+    _check(delta.dtype in _DTYPE_CODE and (delta.stride(3) == 1 or delta.shape[3] == 1), "delta must be contiguous along the map")
+    with torch.cuda.device(delta.device):
+        rc = _lib.lib().ss2d_core_mask_pads(delta.data_ptr(), delta.shape[2], delta.shape[1], H, W, Hp, Wp, delta.stride(0),
+                                            delta.stride(1), delta.stride(2), _DTYPE_CODE[delta.dtype],
+                                            torch.cuda.current_stream(delta.device).cuda_stream)
+    _lib.check(rc, "ss2d_core_mask_pads")
+    return delta
 
 
 def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True, out=None):

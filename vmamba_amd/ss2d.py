@@ -21,7 +21,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ._lib import SS2D_ENOTSUP, Ss2dError
-from .core import DT_PROJ_MAX_RANK, core_fits, dt_proj_hip, ss2d_core_hip
+from .core import DT_PROJ_MAX_RANK, core_fits, core_mask_pads_hip, dt_proj_hip, padded_map_size, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn
 from .conv import dwconv3x3_silu_hip
@@ -192,17 +192,27 @@ class SS2D(nn.Module):
             dts = torch.bmm(consts["Wdt"], dts)
         return dts.view(B, K * D, L), Bs, Cs
 
-    def forward_core_fused(self, x, consts):
-        """One state per channel: the three operators as ONE kernel (ss2d_core_fwd).
+    def forward_core_fused(self, x, consts, crop=True):
+        """One state per channel: the three operators as ONE kernel (ss2d_core_fwd).  Returns y (B, D, L) fp32; with
+        ``crop=False`` the pair (y on the map the kernel ran on -- possibly a padded one --, that map's (H, W)).
 
         A projection is a per-position contraction, so x_proj is applied to x in its natural order for all four
         directions at once, and only its small output (R + 2 rows per direction instead of D) is put into scan
         order -- direction-major and batch-innermost, which makes dt_proj ONE GEMM per direction over all B*L
         positions and hands the kernel delta rows of consecutive images side by side.
         """
-        B, D, H, W = x.shape
-        K, L, R = self.k_group, H * W, self.dt_rank
+        B, D, H0, W0 = x.shape
+        K, R = self.k_group, self.dt_rank
         C = R + 2
+        # Maps the kernel would walk element by element (sides like 57 x 58, 75, 19: a number of positions that is not a
+        # multiple of 4) are embedded in a slightly larger map: zeros on the added rows / columns, the projections
+        # computed on the padded map, and the step of the added positions set to 0 (delta = -inf), which makes them
+        # neutral elements of the scan; the result is cropped.
+        padded = padded_map_size(H0, W0, x.dtype)
+        if padded is not None:
+            x = F.pad(x, (0, padded[1] - W0, 0, padded[0] - H0))
+        H, W = x.shape[2], x.shape[3]
+        L = H * W
         proj = torch.bmm(consts["Wx_all"], x.view(B, D, L))                                   # (B, K*C, L)
         # Rows of B*L positions start on 16-byte boundaries only if B*L is a multiple of the 16-byte vector: maps with
         # an odd (or 2, 4 mod 8) number of positions get room for a few images more, which nothing reads back --
@@ -217,8 +227,15 @@ class SS2D(nn.Module):
             delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
         else:
             delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
-        return ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, R, :B], x_dbl[:, R + 1, :B], consts["As"].view(-1), consts["Ds"],
-                             consts["dt_bias"], True)
+        if padded is not None:
+            core_mask_pads_hip(delta[:, :, :B], H0, W0, H, W)
+        y = ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, R, :B], x_dbl[:, R + 1, :B], consts["As"].view(-1), consts["Ds"],
+                          consts["dt_bias"], True)
+        if not crop:
+            return y, (H, W)
+        if padded is not None:
+            y = y.view(B, D, H, W)[:, :, :H0, :W0].reshape(B, D, H0 * W0)
+        return y
 
     def _fused_core_applies(self, x):
         """The fused kernel is an inference kernel for one-state models whose map fits its LDS planes; under autograd
@@ -232,7 +249,13 @@ class SS2D(nn.Module):
         consts = self._inference_constants(B)
         if self._fused_core_applies(x):
             try:
-                return self.finish_core(self.forward_core_fused(x, consts), B, D, H, W, x.dtype)
+                # out_norm runs on the map the kernel ran on (a padded map has rows the norm's vector paths like as
+                # well) and the added rows / columns are cut off its 16-bit result, half the bytes of the fp32 map
+                y, (Hp, Wp) = self.forward_core_fused(x, consts, crop=False)
+                out = self.finish_core(y, B, D, Hp, Wp, x.dtype)
+                if (Hp, Wp) != (H, W):
+                    out = (out[:, :, :H, :W] if self.channel_first else out[:, :H, :W]).contiguous()
+                return out
             except Ss2dError as e:          # a shape the fused kernel has no variant for: the three operators take it
                 if e.code != SS2D_ENOTSUP:
                     raise
