@@ -137,6 +137,17 @@ int ss2d_selective_scan_fwd(const ss2d_scan_params *params, void *stream);
 int ss2d_selective_scan_kernel(const ss2d_scan_params *params);
 
 /*
+ * The same forward with CrossScan folded in, for several states per channel: params->u is not the (batch, dim, seqlen)
+ * tensor of the four scan-ordered copies (cross_scan_fn's output, classification/models/vmamba.py:604, 625) but the map
+ * itself, x (batch, dim / 4, seqlen) with u_batch_stride / u_d_stride its strides, and x_t (same strides) holds every
+ * height x width map transposed (width x height).  n_groups must be 4 and group k is scan direction k: its channels
+ * read x (k = 0, 2) or x_t (k = 1, 3), forwards (k < 2) or backwards (cross_scan_fwd, csm_triton.py:22-29).  Everything
+ * else as ss2d_selective_scan_fwd.  Served by the channel-per-lane kernel only (dstate 4 / 8 / 16 / 32, seqlen a multiple
+ * of 8, dim / 4 >= 32, 16-byte aligned rows): SS2D_ENOTSUP otherwise.
+ */
+int ss2d_selective_scan_fwd_maps(const ss2d_scan_params *params, const void *x_t, void *stream);
+
+/*
  * Selective-scan backward.  Replaces selective_scan_bwd + selective_scan_bwd_kernel
  * (kernels/selective_scan/csrc/selective_scan/cusoflex/selective_scan_oflex.cpp:233-355,
  *  .../selective_scan_bwd_kernel_oflex.cuh); inputs as in the forward plus

@@ -164,6 +164,33 @@ def test_scan_channel_per_lane_kernel_matches_oracle(batch, dim, G, N, L, dtype)
     check_states(x, xw)
 
 
+@pytest.mark.parametrize("batch,Dm,H,W,N", [(2, 32, 8, 8, 16), (1, 64, 14, 12, 4), (2, 48, 7, 8, 8), (1, 96, 56, 56, 16), (3, 40, 4, 6, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_scan_reading_the_map_through_the_cross_scan_routes(batch, Dm, H, W, N, dtype):
+    """CrossScan folded into the several-state scan (ss2d_selective_scan_fwd_maps): the kernel reads x and its transpose
+    instead of the four scan-ordered copies.  Same kernel, same values of u: bit-identical to the scan of
+    cross_scan_fn(x), which in turn is checked against the oracle."""
+    from vmamba_amd.csms6s import selective_scan_from_map
+    _announce("scan-from-map", batch, Dm, H, W, N, dtype)
+    L = H * W
+    u, delta, A, B, C, D, bias = make_inputs(35, batch, 4 * Dm, 4, N, L, dtype, ss2d_like=True)
+    x = torch.randn(batch, Dm, H, W, generator=torch.Generator().manual_seed(36)).to(dtype)
+    xs = orc.cross_scan(x).view(batch, 4 * Dm, L)
+    want = orc.selective_scan(xs, delta, A, B, C, D, bias, True, out_float=True)
+    dev = lambda t: t.to(DEV)
+    got = selective_scan_from_map(dev(x), dev(delta), dev(A), dev(B), dev(C), dev(D), dev(bias), True, True)
+    two_steps, _ = va.selective_scan_fwd(va.cross_scan_fn(dev(x)).view(batch, 4 * Dm, L), dev(delta), dev(A), dev(B), dev(C), dev(D),
+                                         dev(bias), True, 1, True, want_x=False)
+    torch.cuda.synchronize()
+    assert torch.equal(got, two_steps)
+    tol = TOL32 if L <= 2048 else dict(rtol=1e-3, atol=max(2e-3, 2e-5 * want.abs().max().item()))
+    assert torch.allclose(got.cpu(), want, **tol), f"max abs err {(got.cpu() - want).abs().max().item()}"
+    # shapes the kernel does not take are refused, not approximated
+    with pytest.raises(_lib.Ss2dError) as e:
+        selective_scan_from_map(dev(x)[:, :8], dev(delta)[:, :32].contiguous(), dev(A)[:32].contiguous(), dev(B), dev(C), None, None, True, True)
+    assert e.value.code == _lib.SS2D_ENOTSUP
+
+
 @pytest.mark.parametrize("has_D,has_bias,softplus", [(False, False, False), (True, False, True), (False, True, False)])
 def test_scan_channel_per_lane_optional_arguments_and_delta_groups(has_D, has_bias, softplus):
     _announce("scan-chan-opt", has_D, has_bias, softplus)

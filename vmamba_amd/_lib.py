@@ -19,7 +19,7 @@ SCAN_KERNEL_NONE, SCAN_KERNEL_ROW, SCAN_KERNEL_ROW4, SCAN_KERNEL_FLAT, SCAN_KERN
 SCAN_KERNEL_NAMES = ("none", "row", "row4", "flat", "small", "chan")
 
 EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_merge", "ss2d_selective_scan_fwd",
-           "ss2d_selective_scan_kernel",
+           "ss2d_selective_scan_kernel", "ss2d_selective_scan_fwd_maps",
            "ss2d_layer_norm", "ss2d_add_layer_norm", "ss2d_bias_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
            "ss2d_core_workspace_bytes", "ss2d_core_fwd_ws", "ss2d_core_mask_pads",
            "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_scan_flex_ws", "ss2d_cross_scan_flex_static", "ss2d_cross_merge_flex",
@@ -91,6 +91,8 @@ def lib():
         L.ss2d_cross_merge.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 6 + [ctypes.c_void_p]
         L.ss2d_selective_scan_fwd.restype = ctypes.c_int
         L.ss2d_selective_scan_fwd.argtypes = [ctypes.POINTER(ScanParams), ctypes.c_void_p]
+        L.ss2d_selective_scan_fwd_maps.restype = ctypes.c_int
+        L.ss2d_selective_scan_fwd_maps.argtypes = [ctypes.POINTER(ScanParams), ctypes.c_void_p, ctypes.c_void_p]
         L.ss2d_selective_scan_kernel.restype = ctypes.c_int
         L.ss2d_selective_scan_kernel.argtypes = [ctypes.POINTER(ScanParams)]
         L.ss2d_layer_norm.restype = ctypes.c_int

@@ -97,6 +97,42 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplu
     return [out, x]
 
 
+def selective_scan_from_map(x, delta, A, B, C, D=None, delta_bias=None, delta_softplus=True, out_float=True):
+    """``selective_scan_fwd(cross_scan_fn(x).view(batch, 4 * D, L), delta, ...)[0]`` without the four scan-ordered copies:
+    x (batch, D, H, W) is read through CrossScan's routes inside the scan kernel (its transpose is made here, one small
+    pass).  Inference only; several states per channel (ss2d_selective_scan_fwd_maps).  Raises Ss2dError with status
+    SS2D_ENOTSUP for shapes that kernel does not take: the caller then runs cross_scan_fn and selective_scan_fn."""
+    from .csm import transpose_bcl_hip
+    _check(x.is_cuda and x.dim() == 4 and x.dtype in _DTYPE_CODE, "x must be a (batch, D, H, W) GPU tensor of a supported dtype")
+    _check(A.dtype == torch.float32, "A must be float32")
+    _check(delta.dtype == x.dtype and B.dtype == x.dtype and C.dtype == x.dtype, "delta, B, C must have x's dtype")
+    batch, Dm, H, W = x.shape
+    L, dim = H * W, 4 * Dm
+    dstate = A.size(1)
+    _check(tuple(delta.shape) == (batch, dim, L) and tuple(A.shape) == (dim, dstate), "delta must be (batch, 4 D, L) and A (4 D, dstate)")
+    _check(tuple(B.shape) == (batch, 4, dstate, L) and tuple(C.shape) == (batch, 4, dstate, L), "B and C must be (batch, 4, dstate, L)")
+    for name, t in (("delta", delta), ("B", B), ("C", C)):
+        _check(t.is_cuda and (t.stride(-1) == 1 or t.size(-1) == 1), f"{name} must be a GPU tensor contiguous in its last dimension")
+    if D is not None:
+        _check(D.dtype == torch.float32 and D.is_cuda and tuple(D.shape) == (dim,), "D must be a float32 GPU tensor of shape (4 D)")
+        D = D.contiguous()
+    if delta_bias is not None:
+        _check(delta_bias.dtype == torch.float32 and delta_bias.is_cuda and tuple(delta_bias.shape) == (dim,),
+               "delta_bias must be a float32 GPU tensor of shape (4 D)")
+        delta_bias = delta_bias.contiguous()
+    x = x.contiguous()
+    x_t = transpose_bcl_hip(x.view(batch * Dm, H, W))                       # every map as W x H
+    out = torch.empty((batch, dim, L), device=x.device, dtype=torch.float32 if out_float else x.dtype)
+    p = _scan_params(out, delta, A, B, C, D, delta_bias, delta_softplus, out, None)     # shapes of the scan; u set below
+    p.in_dtype = _DTYPE_CODE[x.dtype]
+    p.u = x.data_ptr()
+    p.u_batch_stride, p.u_d_stride = Dm * L, L
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ss2d_selective_scan_fwd_maps(p, x_t.data_ptr(), torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "ss2d_selective_scan_fwd_maps")
+    return out
+
+
 def selective_scan_bwd(u, delta, A, B, C, D, delta_bias, dout, x=None, delta_softplus=False, nrows=1):
     """Python twin of ``selective_scan_cuda_oflex.bwd``: returns [du, ddelta, dA, dB, dC, dD, ddelta_bias]
     (selective_scan_oflex.cpp:233-355).  ``x`` (the forward's chunk states) and ``nrows`` are accepted and unused:

@@ -131,11 +131,30 @@ struct ChanGeom {
 // exp2(A_n log2e * sum dl), and the sum is per CHANNEL, not per state: each of the four wavefronts adds up a quarter of
 // every round's positions for its lane's channel (one LDS read, four adds per 16 positions) and the quarters meet in LDS
 // when a chunk ends.
-template <typename in_t, typename out_t, int kSpw, bool kSoftplus, bool kX>
+//
+// kMaps: CrossScan folded in.  u is not the (batch, 4 D, L) tensor of the four scan-ordered copies but the map itself,
+// x (batch, D, L), plus its transpose xt (batch, D, L: every H x W map stored as W x H): direction k = the channel's
+// group reads x (k = 0, 2) or xt (k = 1, 3), forwards (k < 2) or backwards -- position t of the scan is element t or
+// L - 1 - t of that row (cross_scan_fwd, classification/models/csm_triton.py:22-29).  A thread's four positions are then
+// the four elements that END at L - 1 - t, taken in reverse.
+template <typename in_t>
+__device__ __forceinline__ Raw4<in_t> reverse4(const Raw4<in_t> &r) {
+    Raw4<in_t> o;
+    if constexpr (sizeof(in_t) == 2) {
+        o.w[0] = __builtin_amdgcn_alignbit(r.w[1], r.w[1], 16);      // halves of a dword exchanged
+        o.w[1] = __builtin_amdgcn_alignbit(r.w[0], r.w[0], 16);
+    } else {
+        o.w[0] = r.w[3]; o.w[1] = r.w[2]; o.w[2] = r.w[1]; o.w[3] = r.w[0];
+    }
+    return o;
+}
+
+template <typename in_t, typename out_t, int kSpw, bool kSoftplus, bool kX, bool kMaps = false>
 __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restrict__ u_all, const in_t *__restrict__ dl_all,
                                                            const in_t *__restrict__ B_all, const in_t *__restrict__ C_all,
                                                            const float *__restrict__ A_all, out_t *__restrict__ o_all,
-                                                           const ScanArgs p, const ChanGeom geo) {
+                                                           const ScanArgs p, const ChanGeom geo,
+                                                           const in_t *__restrict__ ut_all = nullptr) {
     __shared__ __align__(16) float s_dl[kChanBlock * kChanTilePitch];
     __shared__ __align__(16) float s_du[kChanBlock * kChanTilePitch];
     __shared__ __align__(16) float s_y[kWavesPerWg * kChanBlock * kChanSubPitch];
@@ -159,6 +178,19 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
     const int ds = (int)grp * dpg + min(cs, dpg - 1);
     const int dgs = ds / p.dim_per_delta;
     const in_t *u_row = u_all + (int64_t)b * p.u_bs + (int64_t)ds * p.u_ds;
+    bool u_rev = false;                                     // kMaps: uniform over the workgroup (one group = one direction)
+    if constexpr (kMaps) {
+        const int Dm = p.dim >> 2, k = ds / Dm;
+        u_row = ((k & 1) ? ut_all : u_all) + (int64_t)b * p.u_bs + (int64_t)(ds - k * Dm) * p.u_ds;
+        u_rev = k >= 2;
+    }
+    // four positions of u from position pos of the scan on
+    auto load_u = [&](int pos) {
+        if constexpr (kMaps) {
+            if (u_rev) return reverse4<in_t>(load_raw4<in_t>(u_row, pos < L ? L - 4 - pos : L, L, 0.0f));
+        }
+        return load_raw4<in_t>(u_row, pos, L, 0.0f);
+    };
     const in_t *dl_row = dl_all + (int64_t)b * p.dl_bs + (int64_t)dgs * p.dl_ds;
     out_t *o_row = o_all + (int64_t)b * p.o_bs + (int64_t)ds * p.o_ds;
     const float bias_s = p.bias ? p.bias[dgs] : 0.0f;
@@ -187,7 +219,7 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
     Raw4<in_t> ru[2], rd[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-        ru[s] = load_raw4<in_t>(u_row, s * kChanSub + 4 * q, L, 0.0f);
+        ru[s] = load_u(s * kChanSub + 4 * q);
         rd[s] = load_raw4<in_t>(dl_row, s * kChanSub + 4 * q, L, kFill);
     }
     // B / C of the (round, state) processed next are always one step ahead in scalar registers: requested before the
@@ -220,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
         if (t0 + kChanTile < L) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                ru[s] = load_raw4<in_t>(u_row, t0 + kChanTile + s * kChanSub + 4 * q, L, 0.0f);
+                ru[s] = load_u(t0 + kChanTile + s * kChanSub + 4 * q);
                 rd[s] = load_raw4<in_t>(dl_row, t0 + kChanTile + s * kChanSub + 4 * q, L, kFill);
             }
         }
@@ -320,7 +352,7 @@ bool scan_chan_eligible(const ScanArgs &a) {
 }
 
 template <typename in_t, typename out_t>
-static int launch_chan_typed(const ScanArgs &a, hipStream_t stream) {
+static int launch_chan_typed(const ScanArgs &a, const void *xt, hipStream_t stream) {
     ChanGeom geo;
     geo.n_cb = (a.dim_per_group + kChanBlock - 1) / kChanBlock;
     const int groups = a.dim / a.dim_per_group;
@@ -328,32 +360,36 @@ static int launch_chan_typed(const ScanArgs &a, hipStream_t stream) {
     geo.div_groups = make_fastdiv((uint32_t)groups);
     const int64_t n_wg = (int64_t)a.batch * groups * geo.n_cb;
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-#define SS2D_LAUNCH_CHAN(SPW, SP, X)                                                                                       \
-    hipLaunchKernelGGL((scan_chan_kernel<in_t, out_t, SPW, SP, X>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,          \
-                       (const in_t *)a.u, (const in_t *)a.delta, (const in_t *)a.B, (const in_t *)a.C, a.A, (out_t *)a.out, a, geo)
-#define SS2D_LAUNCH_CHAN_N(SP, X)                               \
+#define SS2D_LAUNCH_CHAN(SPW, SP, X, M)                                                                                    \
+    hipLaunchKernelGGL((scan_chan_kernel<in_t, out_t, SPW, SP, X, M>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,       \
+                       (const in_t *)a.u, (const in_t *)a.delta, (const in_t *)a.B, (const in_t *)a.C, a.A, (out_t *)a.out, a, geo, \
+                       (const in_t *)xt)
+#define SS2D_LAUNCH_CHAN_N(SP, X, M)                            \
     switch (a.N) {                                              \
-        case 4: SS2D_LAUNCH_CHAN(1, SP, X); break;              \
-        case 8: SS2D_LAUNCH_CHAN(2, SP, X); break;              \
-        case 16: SS2D_LAUNCH_CHAN(4, SP, X); break;             \
-        default: SS2D_LAUNCH_CHAN(8, SP, X); break;             \
+        case 4: SS2D_LAUNCH_CHAN(1, SP, X, M); break;           \
+        case 8: SS2D_LAUNCH_CHAN(2, SP, X, M); break;           \
+        case 16: SS2D_LAUNCH_CHAN(4, SP, X, M); break;          \
+        default: SS2D_LAUNCH_CHAN(8, SP, X, M); break;          \
     }
-    if (a.x) {
-        if (a.softplus) { SS2D_LAUNCH_CHAN_N(true, true) } else { SS2D_LAUNCH_CHAN_N(false, true) }
+#define SS2D_LAUNCH_CHAN_X(SP, M) \
+    if (a.x) { SS2D_LAUNCH_CHAN_N(SP, true, M) } else { SS2D_LAUNCH_CHAN_N(SP, false, M) }
+    if (xt) {
+        if (a.softplus) { SS2D_LAUNCH_CHAN_X(true, true) } else { SS2D_LAUNCH_CHAN_X(false, true) }
     } else {
-        if (a.softplus) { SS2D_LAUNCH_CHAN_N(true, false) } else { SS2D_LAUNCH_CHAN_N(false, false) }
+        if (a.softplus) { SS2D_LAUNCH_CHAN_X(true, false) } else { SS2D_LAUNCH_CHAN_X(false, false) }
     }
+#undef SS2D_LAUNCH_CHAN_X
 #undef SS2D_LAUNCH_CHAN_N
 #undef SS2D_LAUNCH_CHAN
     return launch_status();
 }
 
-int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream) {
-    if (in_dtype == SS2D_F32) return launch_chan_typed<float, float>(a, stream);
+int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream, const void *xt) {
+    if (in_dtype == SS2D_F32) return launch_chan_typed<float, float>(a, xt, stream);
     if (in_dtype == SS2D_BF16) {
-        return out_dtype == SS2D_F32 ? launch_chan_typed<bf16_t, float>(a, stream) : launch_chan_typed<bf16_t, bf16_t>(a, stream);
+        return out_dtype == SS2D_F32 ? launch_chan_typed<bf16_t, float>(a, xt, stream) : launch_chan_typed<bf16_t, bf16_t>(a, xt, stream);
     }
-    return out_dtype == SS2D_F32 ? launch_chan_typed<f16_t, float>(a, stream) : launch_chan_typed<f16_t, f16_t>(a, stream);
+    return out_dtype == SS2D_F32 ? launch_chan_typed<f16_t, float>(a, xt, stream) : launch_chan_typed<f16_t, f16_t>(a, xt, stream);
 }
 
 }  // namespace ss2d

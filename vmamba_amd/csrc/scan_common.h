@@ -30,7 +30,8 @@ struct ScanArgs {
 // scan_chan.hip: the channel-per-lane kernel for several states per channel.  True when it takes this problem
 // (the caller has already established 16-byte vector I/O); launch returns an SS2D status.
 bool scan_chan_eligible(const ScanArgs &a);
-int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream);
+// xt != nullptr: a.u is the map x (batch, dim / 4, L) and xt its transpose, read through CrossScan's routes (group = direction)
+int launch_scan_chan(const ScanArgs &a, int in_dtype, int out_dtype, hipStream_t stream, const void *xt = nullptr);
 
 // Arguments of the fused core kernels (ss2d_core.hip, ss2d_core_small.hip): the C ABI's ss2d_core_params with derived
 // fields.  Strides in elements.

@@ -651,6 +651,20 @@ extern "C" int ss2d_selective_scan_kernel(const ss2d_scan_params *q) {
     return ss2d::plan_scan(q, a, vec);
 }
 
+extern "C" int ss2d_selective_scan_fwd_maps(const ss2d_scan_params *q, const void *x_t, void *stream) {
+    using namespace ss2d;
+    if (!q || !x_t) return SS2D_EINVAL;
+    if (q->n_groups != 4 || q->dim % 4 != 0) return SS2D_EINVAL;
+    ScanArgs a;
+    bool vec = false;
+    const int kernel = plan_scan(q, a, vec);
+    if (kernel < 0) return kernel;
+    if (kernel == SS2D_SCAN_KERNEL_NONE) return SS2D_OK;
+    // only the channel-per-lane kernel reads u through the routes
+    if (kernel != SS2D_SCAN_KERNEL_CHAN || !aligned16(x_t)) return SS2D_ENOTSUP;
+    return launch_scan_chan(a, q->in_dtype, q->out_dtype, (hipStream_t)stream, x_t);
+}
+
 extern "C" int ss2d_selective_scan_fwd(const ss2d_scan_params *q, void *stream) {
     using namespace ss2d;
     ScanArgs a;

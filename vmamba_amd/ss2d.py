@@ -23,7 +23,7 @@ import torch.nn.functional as F
 from ._lib import SS2D_ENOTSUP, Ss2dError
 from .core import DT_PROJ_MAX_RANK, core_fits, core_mask_pads_hip, dt_proj_hip, padded_map_size, ss2d_core_hip
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
-from .csms6s import selective_scan_fn
+from .csms6s import selective_scan_fn, selective_scan_from_map
 from .conv import dwconv3x3_silu_hip
 from .linear import linear_cf_ln_fusable, linear_cf_ln_hip, linear_cl_hip, linear_fusable
 from .norm import (LayerNorm, LayerNorm2d, add_layer_norm_fusable, add_layer_norm_hip, layer_norm_cf_hip,
@@ -259,10 +259,19 @@ class SS2D(nn.Module):
             except Ss2dError as e:          # a shape the fused kernel has no variant for: the three operators take it
                 if e.code != SS2D_ENOTSUP:
                     raise
-        xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)          # (B, 4, D, L)
         dts, Bs, Cs = self.project_from_map(x, consts)
-        ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
-                               True, True)                                                     # fp32 (oflex)
+        ys = None
+        if self.d_state > 1 and x.is_cuda and not needs_grad(x, dts, Bs, self.A_logs, self.Ds, self.dt_projs_bias):
+            # several states per channel: the scan kernel reads x through CrossScan's routes, xs is never written
+            try:
+                ys = selective_scan_from_map(x, dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"], True, True)
+            except Ss2dError as e:
+                if e.code != SS2D_ENOTSUP:
+                    raise
+        if ys is None:
+            xs = cross_scan_fn(x, in_channel_first=True, out_channel_first=True, scans=0)      # (B, 4, D, L)
+            ys = selective_scan_fn(xs.view(B, K * D, L), dts, consts["As"], Bs, Cs, consts["Ds"], consts["dt_bias"],
+                                   True, True)                                                 # fp32 (oflex)
         y = cross_merge_fn(ys.view(B, K, D, H, W), in_channel_first=True, out_channel_first=True, scans=0)
         return self.finish_core(y, B, D, H, W, x.dtype)
 
