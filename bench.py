@@ -33,6 +33,22 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 FP32_VECTOR_PEAK_TFLOPS = 157.3
 PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "ss2d_core_kernels_vmamba_t_bs128.txt")
+COUNTER_SUMMARY = os.path.join(ROOT, "profiles", "ss2d_core_sq_counters_vmamba_t_bs128.txt")
+
+
+def measured_issue(kernel_tag):
+    """Vector-ALU occupancy of a kernel from the committed rocprofv3 SQ-counter summary: the line
+        ISSUE <tag> valu_busy=<4 * SQ_ACTIVE_INST_VALU / (SIMDs * duration in cycles)> valu_per_unit=<SQ_INSTS_VALU * 64 / units>
+    Returns (dict, "file: line") or (None, reason)."""
+    try:
+        with open(COUNTER_SUMMARY) as f:
+            for n, line in enumerate(f, 1):
+                parts = line.split()
+                if len(parts) >= 3 and parts[0] == "ISSUE" and parts[1] == kernel_tag:
+                    return {k: float(v) for k, v in (p.split("=", 1) for p in parts[2:])}, f"{os.path.relpath(COUNTER_SUMMARY, ROOT)}:{n}"
+    except (OSError, ValueError) as e:
+        return None, f"{type(e).__name__}: {e}"
+    return None, f"no ISSUE line for {kernel_tag} in {os.path.relpath(COUNTER_SUMMARY, ROOT)}"
 
 
 def measured_traffic(kernel_tag):
@@ -155,10 +171,21 @@ def kernel_lines(reps):
                          layer_norm_cf_GBs=E * 6 / t_ln / 1e9)
             del x_cl, ycf, wconv
         if N > 1:
-            # several states per channel: the fp32 work by the reference's own count (csms6s.py:139-160) against the
-            # fp32 vector peak, beside the HBM figure
-            flops = 9.0 * B * K * D * L * N + B * K * D * L
-            fused.update(scan_TFLOPs=flops / t_sc / 1e12, valu_frac=flops / t_sc / 1e12 / FP32_VECTOR_PEAK_TFLOPS)
+            # several states per channel: the scan is bound by vector-ALU issue, not by HBM -- its VALU occupancy and
+            # instruction count per (position, state) come from the committed SQ-counter summary -- and CrossScan is
+            # folded into it (the kernel reads x and its transpose through the routes): core_n = that scan + CrossMerge
+            from vmamba_amd.csms6s import selective_scan_from_map
+            issue, issue_src = measured_issue("scan_chan_kernel@config3")
+            t_n = time_op(lambda: va.cross_merge_fn(selective_scan_from_map(x, delta, A, Bm, Cm, Dv, bias, True, True).view(B, K, D, H, W)), reps)
+            # the same three steps as separate operators, also timed as one chain (a kernel that follows another kind of
+            # kernel starts on a cold cache, which the per-kernel lines above do not see)
+            t_3 = time_op(lambda: va.cross_merge_fn(va.selective_scan_fn(va.cross_scan_fn(x).view(B, K * D, L), delta, A, Bm, Cm, Dv, bias,
+                                                                         True).view(B, K, D, H, W)), reps)
+            flops = 9.0 * B * K * D * L * N + B * K * D * L          # the reference's own count, csms6s.py:139-160
+            fused.update(scan_TFLOPs=flops / t_sc / 1e12, issue_frac=(issue or {}).get("valu_busy"),
+                         valu_per_position_state=(issue or {}).get("valu_per_unit"), issue_source=issue_src,
+                         core_n_us=t_n * 1e6, core_n_GBs=(b_cs + b_sc + b_cm) / t_n / 1e9,
+                         three_operators_us=t_3 * 1e6)
         if name in ("stage1", "stage2"):
             # block-level kernels of the narrow stages (harness side): fused LayerNorm + MLP + residual, and at width 96
             # the two projections with their LayerNorm / residual.  Bytes: activations in and out once (+ residual).
@@ -694,8 +721,9 @@ def main():
         """One kernel line without the harness-side entries, numbers rounded: the full lines go to stderr."""
         keep = ("shape", "B", "D", "H", "W", "N", "scan_kernel", "cross_scan_us", "cross_scan_GBs", "scan_us", "scan_GBs", "ext_fwd_us",
                 "cross_merge_us", "cross_merge_GBs", "core_GBs", "core_fused_us", "core_fused_GBs", "dt_proj_us", "dt_proj_GBs",
-                "dwconv_us", "layer_norm_cf_us", "scan_bwd_us", "issue_frac", "core_n_us", "core_n_GBs")
-        return {key: (round(v, 1) if isinstance(v, float) else v) for key, v in k.items() if key in keep}
+                "dwconv_us", "layer_norm_cf_us", "scan_bwd_us", "issue_frac", "valu_per_position_state", "core_n_us", "core_n_GBs",
+                "three_operators_us")
+        return {key: (round(v, 1 if key.endswith(("_us", "_GBs")) else 3) if isinstance(v, float) else v) for key, v in k.items() if key in keep}
 
     fp32 = extra.get("fp32") or {}
     fp32_cf = extra.get("fp32_channel_first") or {}
