@@ -230,6 +230,17 @@ def kernel_lines(reps):
                         cross_merge_us=t_cm * 1e6, cross_merge_GBs=b_cm / t_cm / 1e9,
                         core_GBs=(b_cs + b_sc + b_cm) / (t_cs + t_sc + t_cm) / 1e9,
                         scan_bytes=b_sc, **fused))
+        if name in ("stage4", "hires"):
+            # yardstick for the two kernels furthest below 0.6 of the HBM peak among the three operators: a plain device copy
+            # that moves the same number of bytes (half read, half written) -- transfers of this size do not reach the
+            # rate of the 1 GiB calibration copy either
+            b_y = b_cs if name == "stage4" else b_sc
+            src_y = torch.empty(b_y // 2, dtype=torch.uint8, device=dev)
+            dst_y = torch.empty_like(src_y)
+            t_y = time_op(lambda: dst_y.copy_(src_y), reps)
+            key = "cross_scan" if name == "stage4" else "scan"
+            out[-1].update({key + "_copy_us": t_y * 1e6, key + "_over_copy": (t_cs if name == "stage4" else t_sc) / t_y})
+            del src_y, dst_y
         if name == "stage1":
             # the scan's backward at the same shape (fp32 dout, as the oflex forward hands back): algorithmic bytes =
             # u, delta, dout in; du, ddelta out; B, C in and fp32 dB, dC out once per (batch, direction)
@@ -722,7 +733,7 @@ def main():
         keep = ("shape", "B", "D", "H", "W", "N", "scan_kernel", "cross_scan_us", "cross_scan_GBs", "scan_us", "scan_GBs", "ext_fwd_us",
                 "cross_merge_us", "cross_merge_GBs", "core_GBs", "core_fused_us", "core_fused_GBs", "dt_proj_us", "dt_proj_GBs",
                 "dwconv_us", "layer_norm_cf_us", "scan_bwd_us", "issue_frac", "valu_per_position_state", "core_n_us", "core_n_GBs",
-                "three_operators_us")
+                "three_operators_us", "cross_scan_copy_us", "cross_scan_over_copy", "scan_copy_us", "scan_over_copy")
         return {key: (round(v, 1 if key.endswith(("_us", "_GBs")) else 3) if isinstance(v, float) else v) for key, v in k.items() if key in keep}
 
     fp32 = extra.get("fp32") or {}

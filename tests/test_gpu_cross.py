@@ -24,6 +24,9 @@ SHAPES = [
     # odd maps with an even channel count (16-bit elements then travel as pairs across map boundaries): one group, several
     # groups with a short last one, single positions
     (2, 6, 7, 7), (3, 10, 5, 9), (1, 2, 1, 1), (2, 4, 3, 3), (2, 170, 7, 7), (1, 86, 7, 7), (2, 768, 7, 7),
+    # ... and with a multiple of 8 channels (16-byte vectors across map boundaries): one group, a short last group, maps of
+    # more than 256 positions, several groups of 8
+    (2, 8, 7, 7), (1, 96, 7, 7), (3, 16, 5, 9), (2, 8, 3, 3), (1, 8, 17, 17), (1, 24, 17, 17), (2, 104, 7, 7),
 ]
 
 
