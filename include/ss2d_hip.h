@@ -294,6 +294,16 @@ int ss2d_core_mask_pads(void *delta, int batch, int dim, int height, int width, 
                         int64_t delta_dir_stride, int64_t delta_dim_stride, int64_t delta_batch_stride, int dtype, void *stream);
 
 /*
+ * The copies around such an embedding, each as one pass: dst[m][r][c] = src[m][r][c] where the source map has that row
+ * and column, 0 elsewhere, for n_maps dense maps of src_rows x src_cols resp. dst_rows x dst_cols elements of 2 or 4
+ * bytes.  A larger destination is the zero-padded map (what F.pad would make of x for vmamba.py:604), a smaller one the
+ * crop of a result; a channel-last activation (B, H, W, D) is B maps of H rows of W * D elements.  Fewer than 2^32
+ * elements on either side.  No counterpart in the reference.
+ */
+int ss2d_core_embed_maps(const void *src, void *dst, int64_t n_maps, int src_rows, int64_t src_cols, int dst_rows,
+                         int64_t dst_cols, int elem_bytes, void *stream);
+
+/*
  * CrossScan / CrossMerge for every layout and mode of the reference operators (cross_scan_fn / cross_merge_fn,
  * classification/models/csm_triton.py:501-517; semantics of the flex kernel :278-400 and of the torch functions
  * :22-179).  Flags are named from the scan's side, as in the reference, for both operations:

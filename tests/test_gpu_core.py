@@ -211,6 +211,46 @@ def test_core_tiled_optional_arguments_and_workspace_contract():
     assert torch.allclose(y.cpu(), oracle_core(x, delta, Bs, Cs, A, Dv, bias), **TOL)
 
 
+# (n_maps, source rows, cols, destination rows, cols): embeddings and crops through every copy variant -- rows of whole
+# 16-byte vectors on both sides (channel-last crops), a destination of whole vectors with ragged rows (75 -> 80, 19 -> 20,
+# crops whose total size is a multiple of the vector), 4-byte pairs (57 x 58 -> 60 x 60 with an odd number of maps), single
+# elements, growth in one direction only, rows and columns at once
+EMBED_CASES = [(6, 57, 58, 60, 60), (3, 57, 58, 60, 60), (8, 75, 75, 80, 80), (5, 19, 19, 20, 20), (1, 20, 20, 19, 19),
+               (4, 60, 60 * 96, 57, 58 * 96), (8, 60, 60, 57, 58), (3, 60, 60, 57, 58), (1, 3, 3, 5, 5), (7, 9, 13, 12, 16),
+               (2, 8, 8, 8, 16), (2, 8, 16, 16, 16), (3, 5, 8, 8, 4), (2, 1, 1, 1, 1), (1, 200, 334, 200, 336)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("case", EMBED_CASES, ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("offset", [0, 1], ids=["aligned", "shifted"])
+def test_embed_maps_pads_with_zeros_and_crops(case, dtype, offset):
+    """ss2d_core_embed_maps against slicing and zero-filling in torch, bit for bit; with a source that starts one element
+    into its allocation as well (no 16-byte alignment)."""
+    from vmamba_amd.core import embed_maps_hip
+    n, sr, sc, dr, dc = case
+    print("CASE embed", case, dtype, offset, flush=True)
+    g = torch.Generator().manual_seed(sum(case))
+    src = torch.randn((n, sr, sc), generator=g).to(dtype)
+    want = torch.zeros((n, dr, dc), dtype=dtype)
+    want[:, :min(sr, dr), :min(sc, dc)] = src[:, :min(sr, dr), :min(sc, dc)]
+    buf = torch.empty(src.numel() + offset, dtype=dtype, device=DEV)
+    dev_src = buf[offset:].view(n, sr, sc)
+    dev_src.copy_(src)
+    got = embed_maps_hip(dev_src, dr, dc)
+    torch.cuda.synchronize()
+    assert got.shape == want.shape and torch.equal(got.cpu().view(torch.uint8), want.view(torch.uint8))
+
+
+def test_embed_maps_rejects_what_it_cannot_address():
+    L = _lib.lib()
+    x = torch.zeros(64, dtype=torch.int16, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.ss2d_core_embed_maps(x.data_ptr(), x.data_ptr(), 1, 2, 2, 2, 2, 1, stream) == _lib.SS2D_EINVAL      # 1-byte elements
+    assert L.ss2d_core_embed_maps(None, x.data_ptr(), 1, 2, 2, 2, 2, 2, stream) == _lib.SS2D_EINVAL
+    assert L.ss2d_core_embed_maps(x.data_ptr(), x.data_ptr(), 1 << 20, 1 << 10, 1 << 10, 1 << 10, 1 << 10, 2, stream) == _lib.SS2D_ENOTSUP
+    assert L.ss2d_core_embed_maps(x.data_ptr(), x.data_ptr(), 0, 2, 2, 2, 2, 2, stream) == _lib.SS2D_OK          # nothing to do
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
 @pytest.mark.parametrize("sizes", [(57, 58, 60, 60), (19, 19, 20, 20), (9, 13, 16, 16), (75, 75, 80, 80), (8, 8, 8, 16), (5, 3, 8, 8)],
                          ids=lambda s: "x".join(map(str, s)))

@@ -97,6 +97,35 @@ def test_forward_core_bf16_activations():
         assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), f"fused={fused}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("channel_first", [True, False], ids=["cf", "cl"])
+@pytest.mark.parametrize("d_model,B,H,W", [(96, 3, 57, 58), (32, 5, 19, 19), (192, 2, 75, 75), (128, 2, 19, 19), (48, 2, 37, 41), (768, 1, 19, 19)])
+def test_forward_core_on_maps_embedded_in_padded_ones(d_model, B, H, W, channel_first, dtype):
+    """16-bit maps whose sides the vector paths do not like run the fused core on a zero-padded map (the added positions made
+    neutral through one more dt_proj rank, or ss2d_core_mask_pads where the rank does not fit) and are cut out of its
+    result: against the fp32 CPU model at the 16-bit bound, and against the three-operator path of the same module, which
+    pads nothing, at a few roundings of the 16-bit output."""
+    from vmamba_amd.core import padded_map_size
+    print("CASE core-padded", d_model, B, H, W, channel_first, dtype, flush=True)
+    torch.manual_seed(3)
+    ref = RefSS2D(d_model=d_model, d_state=1, ssm_ratio=1.0, channel_first=channel_first).eval()
+    hip = SS2D(d_model=d_model, d_state=1, ssm_ratio=1.0, channel_first=channel_first).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip = hip.to(dtype).to(DEV)
+    assert padded_map_size(H, W, dtype) is not None
+    x = torch.randn(B, d_model, H, W, generator=torch.Generator().manual_seed(4)).to(dtype)
+    with torch.no_grad():
+        want = ref.forward_core(x.float())
+        hip.fused_core = True
+        got = hip.forward_core(x.to(DEV))
+        hip.fused_core = False
+        ops = hip.forward_core(x.to(DEV))
+    assert got.shape == want.shape and got.dtype == dtype
+    tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
+    assert torch.allclose(got.float().cpu(), want, rtol=tol, atol=tol)
+    assert torch.allclose(got.float(), ops.float(), rtol=tol / 2, atol=tol / 2)
+
+
 def test_block_with_gate_matches():
     print("CASE block-z", flush=True)
     ref, hip = _pair(24, 16, 2.0, disable_z=False)

@@ -78,6 +78,24 @@ def core_mask_pads_hip(delta, H, W, Hp, Wp):
     return delta
 
 
+def embed_maps_hip(src, dst_rows, dst_cols):
+    """src (n_maps, rows, cols), contiguous, 2- or 4-byte elements -> (n_maps, dst_rows, dst_cols): the maps zero-padded at
+    the bottom / right or cropped there, in one pass (ss2d_core_embed_maps)."""
+    _check(src.is_cuda and src.dim() == 3 and src.is_contiguous(), "embed_maps: a contiguous (n_maps, rows, cols) GPU tensor")
+    _check(src.element_size() in (2, 4), "embed_maps: 2- or 4-byte elements")
+    n, rows, cols = src.shape
+    dst = src.new_empty((n, dst_rows, dst_cols))
+    if dst.numel() == 0:
+        return dst
+    if src.numel() == 0:
+        return dst.zero_()
+    with torch.cuda.device(src.device):
+        rc = _lib.lib().ss2d_core_embed_maps(src.data_ptr(), dst.data_ptr(), n, rows, cols, dst_rows, dst_cols, src.element_size(),
+                                             torch.cuda.current_stream(src.device).cuda_stream)
+    _lib.check(rc, "ss2d_core_embed_maps")
+    return dst
+
+
 def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus=True, out=None):
     """x (B,D,H,W); delta (4,D,B,L) view; Bs, Cs (4,B,L) views (last stride 1), all of x.dtype and already in the
     scan order of their direction; As, Ds, delta_bias (4*D) fp32.  Returns the merged y (B,D,L) fp32 (written into

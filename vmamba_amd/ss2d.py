@@ -21,7 +21,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ._lib import SS2D_ENOTSUP, Ss2dError
-from .core import DT_PROJ_MAX_RANK, core_fits, core_mask_pads_hip, dt_proj_hip, padded_map_size, ss2d_core_hip
+from .core import (DT_PROJ_MAX_RANK, core_fits, core_mask_pads_hip, dt_proj_hip, embed_maps_hip, padded_map_size,
+                   ss2d_core_hip)
 from .csm import cross_merge_fn, cross_scan_1b1_hip, cross_scan_fn
 from .csms6s import selective_scan_fn, selective_scan_from_map
 from .conv import dwconv3x3_silu_hip
@@ -79,6 +80,24 @@ def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.
     A_logs = torch.log(torch.arange(1, d_state + 1, dtype=torch.float32)).repeat(k_group * d_inner, 1)
     Ds = torch.ones(k_group * d_inner)
     return nn.Parameter(A_logs), nn.Parameter(Ds), nn.Parameter(dt_w), nn.Parameter(dt_b)
+
+
+_PAD_FLAGS = {}
+
+
+def _pad_flags(H0, W0, H, W, dtype, device):
+    """(4, 1, H*W) tensor: 1 at the scan positions of each direction (cross_scan_fwd's orders,
+    classification/models/csm_triton.py:22-29, on the H x W map) that lie outside its top-left H0 x W0 part, 0 elsewhere."""
+    key = (H0, W0, H, W, dtype, str(device))
+    flags = _PAD_FLAGS.get(key)
+    if flags is None:
+        m = torch.zeros((H, W), dtype=torch.bool)
+        m[H0:, :] = True
+        m[:, W0:] = True
+        rows, cols = m.flatten(), m.t().flatten()
+        flags = torch.stack([rows, cols, rows.flip(0), cols.flip(0)]).to(dtype).view(4, 1, H * W).to(device)
+        _PAD_FLAGS[key] = flags          # never evicted: a captured graph may hold its address (a few KB per map size)
+    return flags
 
 
 class SS2D(nn.Module):
@@ -210,7 +229,7 @@ class SS2D(nn.Module):
         # neutral elements of the scan; the result is cropped.
         padded = padded_map_size(H0, W0, x.dtype)
         if padded is not None:
-            x = F.pad(x, (0, padded[1] - W0, 0, padded[0] - H0))
+            x = embed_maps_hip(x.contiguous().view(B * D, H0, W0), padded[0], padded[1]).view(B, D, padded[0], padded[1])
         H, W = x.shape[2], x.shape[3]
         L = H * W
         proj = torch.bmm(consts["Wx_all"], x.view(B, D, L))                                   # (B, K*C, L)
@@ -220,21 +239,36 @@ class SS2D(nn.Module):
         vec = 16 // proj.element_size()
         unit = vec // math.gcd(L, vec)
         Bp = (B + unit - 1) // unit * unit
-        x_dbl = proj.new_empty((K, C, B, L)) if Bp == B else proj.new_zeros((K, C, Bp, L))
-        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl[:, :, :B].permute(2, 0, 1, 3))
-        dts = x_dbl[:, :R].reshape(K, R, Bp * L)
-        if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
-            delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
+        # On a padded map the step of the added positions must be 0.  With a 16-bit dt_proj on the matrix cores that costs
+        # one more rank: a row that is 1 at the added positions of each direction's order and 0 elsewhere, in front of the
+        # dt rows, against a weight column of -1e30 (-65504 in fp16) -- delta there is that value exactly (x = 0 makes the
+        # other ranks' terms 0), softplus of it is 0, and elsewhere the extra term is -0.  Otherwise ss2d_core_mask_pads
+        # writes -inf into delta afterwards, a scattered pass over its rows.
+        flag_rank = padded is not None and proj.dtype != torch.float32 and R + 1 <= DT_PROJ_MAX_RANK
+        off = 1 if flag_rank else 0
+        x_dbl = proj.new_empty((K, C + off, B, L)) if Bp == B else proj.new_zeros((K, C + off, Bp, L))
+        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl[:, off:, :B].permute(2, 0, 1, 3))
+        if flag_rank:
+            x_dbl[:, 0].copy_(_pad_flags(H0, W0, H, W, proj.dtype, proj.device).expand(K, Bp, L))
+            w_dt = consts.get("Wdt_flag")
+            if w_dt is None:
+                big = -65504.0 if proj.dtype == torch.float16 else -1e30
+                w_dt = consts["Wdt_flag"] = torch.cat([self.dt_projs_weight.new_full((K, D, 1), big), self.dt_projs_weight], dim=2)
+            delta = dt_proj_hip(x_dbl[:, :R + 1].reshape(K, R + 1, Bp * L), w_dt).view(K, D, Bp, L)
         else:
-            delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
-        if padded is not None:
-            core_mask_pads_hip(delta[:, :, :B], H0, W0, H, W)
-        y = ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, R, :B], x_dbl[:, R + 1, :B], consts["As"].view(-1), consts["Ds"],
+            dts = x_dbl[:, :R].reshape(K, R, Bp * L)
+            if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
+                delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
+            else:
+                delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
+            if padded is not None:
+                core_mask_pads_hip(delta[:, :, :B], H0, W0, H, W)
+        y = ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, off + R, :B], x_dbl[:, off + R + 1, :B], consts["As"].view(-1), consts["Ds"],
                           consts["dt_bias"], True)
         if not crop:
             return y, (H, W)
         if padded is not None:
-            y = y.view(B, D, H, W)[:, :, :H0, :W0].reshape(B, D, H0 * W0)
+            y = embed_maps_hip(y.view(B * D, H, W), H0, W0).view(B, D, H0 * W0)
         return y
 
     def _fused_core_applies(self, x):
@@ -254,7 +288,11 @@ class SS2D(nn.Module):
                 y, (Hp, Wp) = self.forward_core_fused(x, consts, crop=False)
                 out = self.finish_core(y, B, D, Hp, Wp, x.dtype)
                 if (Hp, Wp) != (H, W):
-                    out = (out[:, :, :H, :W] if self.channel_first else out[:, :H, :W]).contiguous()
+                    if self.channel_first:
+                        out = embed_maps_hip(out.contiguous().view(-1, Hp, Wp), H, W).view(B, -1, H, W)
+                    else:
+                        Dm = out.shape[-1]
+                        out = embed_maps_hip(out.contiguous().view(B, Hp, Wp * Dm), H, W * Dm).view(B, H, W, Dm)
                 return out
             except Ss2dError as e:          # a shape the fused kernel has no variant for: the three operators take it
                 if e.code != SS2D_ENOTSUP:
