@@ -184,12 +184,20 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
         u_row = ((k & 1) ? ut_all : u_all) + (int64_t)b * p.u_bs + (int64_t)(ds - k * Dm) * p.u_ds;
         u_rev = k >= 2;
     }
-    // four positions of u from position pos of the scan on
+    // four positions of u from position pos of the scan on, as they lie in memory: backwards these are the four elements
+    // that end at L - 1 - pos, and they are put in scan order where they are widened (in_scan_order) -- not here, which
+    // would make the wavefront wait for a load it has just issued for the NEXT step
     auto load_u = [&](int pos) {
         if constexpr (kMaps) {
-            if (u_rev) return reverse4<in_t>(load_raw4<in_t>(u_row, pos < L ? L - 4 - pos : L, L, 0.0f));
+            if (u_rev) return load_raw4<in_t>(u_row, pos < L ? L - 4 - pos : L, L, 0.0f);
         }
         return load_raw4<in_t>(u_row, pos, L, 0.0f);
+    };
+    auto in_scan_order = [&](const Raw4<in_t> &r) {
+        if constexpr (kMaps) {
+            if (u_rev) return reverse4<in_t>(r);
+        }
+        return r;
     };
     const in_t *dl_row = dl_all + (int64_t)b * p.dl_bs + (int64_t)dgs * p.dl_ds;
     out_t *o_row = o_all + (int64_t)b * p.o_bs + (int64_t)ds * p.o_ds;
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(kBlock) void scan_chan_kernel(const in_t *__restric
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             float uv[4], raw[4], dl[4], du[4];
-            unpack_raw4<in_t>(ru[s], uv);
+            unpack_raw4<in_t>(in_scan_order(ru[s]), uv);
             unpack_raw4<in_t>(rd[s], raw);
             const bool in_row = t0 + s * kChanSub + 4 * q < L;
 #pragma unroll
