@@ -43,6 +43,26 @@ def test_concurrent_replays_equal_the_eager_forwards(model, batch, size, sub_bat
         assert torch.allclose(runner.output().float(), torch.cat([model(c) for c in x.chunk(sub_batches)]).float(), rtol=0, atol=TOL)
 
 
+def test_graphs_of_padded_maps_survive_other_map_sizes(model):
+    """300 x 300 images give stage maps of 75 x 75 and 19 x 19, which run on padded maps whose added positions are marked by
+    a cached 0/1 row; a captured forward holds that row's address.  Forwards on ten other odd sizes push it out of the
+    cache of recent sizes; the replays must still reproduce the eager forwards."""
+    print("CASE runner padded maps", flush=True)
+    x = torch.randn(4, 3, 300, 300, device=DEV, generator=torch.Generator(DEV).manual_seed(300)).bfloat16()
+    runner = ConcurrentGraphRunner(model, x, 2)
+    assert runner.validate(replays=3, atol=TOL)
+    with torch.no_grad():
+        for size in (68, 76, 84, 92, 100, 108, 116, 132, 140, 148):          # stage maps 17 / 19 / 21 / 23 / 25 ... : all padded
+            model(torch.randn(1, 3, size, size, device=DEV).bfloat16())
+        garbage = [torch.full((1 << 20,), float("nan"), device=DEV) for _ in range(8)]   # reuse whatever was freed
+        eager = torch.cat([model(c) for c in x.chunk(2)])
+    for _ in range(2):
+        runner.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(runner.output().float(), eager.float(), rtol=0, atol=TOL)
+    del garbage
+
+
 @pytest.mark.parametrize("sub_batches", [2, 4])
 def test_benchmark_batch_replays_are_bit_identical(model, sub_batches):
     """The benchmark's own configuration (128 images at 224^2 as 2 or 4 sub-batch graphs side by side): every concurrent

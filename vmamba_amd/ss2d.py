@@ -82,21 +82,32 @@ def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.
     return nn.Parameter(A_logs), nn.Parameter(Ds), nn.Parameter(dt_w), nn.Parameter(dt_b)
 
 
-_PAD_FLAGS = {}
+_PAD_FLAGS = {}            # the most recent map sizes
+_PAD_FLAGS_PINNED = {}     # those a graph capture has read: never dropped, a captured copy kernel holds their address
 
 
 def _pad_flags(H0, W0, H, W, dtype, device):
     """(4, 1, H*W) tensor: 1 at the scan positions of each direction (cross_scan_fwd's orders,
     classification/models/csm_triton.py:22-29, on the H x W map) that lie outside its top-left H0 x W0 part, 0 elsewhere."""
     key = (H0, W0, H, W, dtype, str(device))
-    flags = _PAD_FLAGS.get(key)
-    if flags is None:
-        m = torch.zeros((H, W), dtype=torch.bool)
+    if key in _PAD_FLAGS_PINNED:
+        return _PAD_FLAGS_PINNED[key]
+    capturing = torch.device(device).type == "cuda" and torch.cuda.is_current_stream_capturing()
+    flags = _PAD_FLAGS.pop(key, None)
+    built = flags is None
+    if built:
+        m = torch.zeros((H, W), dtype=torch.bool, device=device)      # built on the device: no host copy inside a capture
         m[H0:, :] = True
         m[:, W0:] = True
         rows, cols = m.flatten(), m.t().flatten()
-        flags = torch.stack([rows, cols, rows.flip(0), cols.flip(0)]).to(dtype).view(4, 1, H * W).to(device)
-        _PAD_FLAGS[key] = flags          # never evicted: a captured graph may hold its address (a few KB per map size)
+        flags = torch.stack([rows, cols, rows.flip(0), cols.flip(0)]).to(dtype).view(4, 1, H * W)
+    if capturing:
+        if not built:              # (built inside the capture, its memory is the graph's own and is rewritten by every replay)
+            _PAD_FLAGS_PINNED[key] = flags
+        return flags
+    _PAD_FLAGS[key] = flags                                           # (re-)inserted as the newest
+    while len(_PAD_FLAGS) > 8:
+        _PAD_FLAGS.pop(next(iter(_PAD_FLAGS)))
     return flags
 
 
