@@ -489,6 +489,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--no-odd-maps", action="store_true", help="skip the forward_core lines on maps of odd sizes")
     ap.add_argument("--no-extra-forwards", action="store_true",
                     help="skip the config-4 (4 x 1024^2) and fp32 forwards reported as extra keys")
     ap.add_argument("--kernels-only", action="store_true",
@@ -527,7 +528,8 @@ def main():
             t = time_op(lambda: dst.copy_(src), args.kernel_reps)
             log(f"calibration copy: 1 GiB read + 1 GiB write in {t * 1e6:.1f} us = {2 * (1 << 30) / t / 1e9:.0f} GB/s")
             del src, dst
-            print(json.dumps({"kernels": kernel_lines(args.kernel_reps), "odd_maps": odd_map_lines(args.kernel_reps)}))
+            print(json.dumps({"kernels": kernel_lines(args.kernel_reps),
+                              "odd_maps": None if args.no_odd_maps else odd_map_lines(args.kernel_reps)}))
         return
     torch.backends.cudnn.benchmark = True
     torch.manual_seed(0)
@@ -728,7 +730,7 @@ def main():
     if not args.no_kernels:
         with torch.no_grad():
             kernels = kernel_lines(args.kernel_reps)
-            odd_maps = odd_map_lines(args.kernel_reps)
+            odd_maps = None if args.no_odd_maps else odd_map_lines(args.kernel_reps)
         k1 = kernels[0]
         core_traffic, core_src = measured_traffic("ss2d_core_kernel@stage1")
         scan_traffic, scan_src = measured_traffic("scan_row_kernel@stage1")
