@@ -263,24 +263,29 @@ __global__ __launch_bounds__(kBlock) void core_tiled_kernel(const CoreArgs p, co
     row_pass(1, r1);
 }
 
-// One wavefront per (direction, image, channel): the state entering every run, in the direction's order of the runs.
+// One workgroup per (direction, image, channel): the state entering every run, in the direction's order of the runs.  A
+// round covers 4 x 64 x kPer runs: wavefront w scans its quarter, the four quarters' aggregates meet in LDS, and each
+// wavefront folds the ones before it into the state its quarter starts from.
 __global__ __launch_bounds__(kBlock) void core_carry_kernel(const float2 *__restrict__ agg, float *__restrict__ carry, int rows,
                                                             int BD, int nr02, int nr13, int nr_max) {
-    constexpr int kPer = 16;                                 // runs per lane and round
+    constexpr int kPer = 4;                                  // runs per lane and round
+    constexpr int kRound = kWavesPerWg * kWave * kPer;       // runs per workgroup and round
+    __shared__ float2 s_agg[2][kWavesPerWg];                 // double-buffered by round parity: one barrier per round
     const int lane = threadIdx.x & (kWave - 1);
-    const int row = (int)blockIdx.x * kWavesPerWg + (int)(threadIdx.x / kWave);
-    if (row >= rows) return;                                 // whole wavefront; no barrier in this kernel
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int row = (int)blockIdx.x;                         // grid == rows
     const int k = row / BD;
     const int n = (k & 1) ? nr13 : nr02;
     const bool rev = k >= 2;
     const float2 *src = agg + (int64_t)row * nr_max;
     float *dst = carry + (int64_t)row * nr_max;
     float state = 0.0f;
-    for (int j0 = 0; j0 < n; j0 += kWave * kPer) {
+    int par = 0;
+    for (int j0 = 0; j0 < n; j0 += kRound, par ^= 1) {       // uniform over the workgroup: every wavefront meets the barrier
         float ac[kPer], hh[kPer];
 #pragma unroll
         for (int t = 0; t < kPer; ++t) {
-            const int j = j0 + lane * kPer + t;
+            const int j = j0 + (wave * kWave + lane) * kPer + t;
             float2 v = make_float2(1.0f, 0.0f);
             if (j < n) v = src[rev ? n - 1 - j : j];
             ac[t] = t == 0 ? v.x : ac[t - 1] * v.x;
@@ -288,14 +293,23 @@ __global__ __launch_bounds__(kBlock) void core_carry_kernel(const float2 *__rest
         }
         float a_ex, h_ex, a_tot, h_tot;
         wave_scan_pairs(ac[kPer - 1], hh[kPer - 1], a_ex, h_ex, a_tot, h_tot);
-        const float s_in = fmaf(a_ex, state, h_ex);
+        if (lane == 0) s_agg[par][wave] = make_float2(a_tot, h_tot);
+        __syncthreads();
+        float c_in = state;                                  // the state this wavefront's quarter starts from ...
+#pragma unroll
+        for (int w = 0; w < kWavesPerWg; ++w) {
+            const float2 g = s_agg[par][w];
+            if (w < wave) c_in = fmaf(g.x, c_in, g.y);
+            state = fmaf(g.x, state, g.y);                   // ... and the one the next round starts from
+        }
+        const float s_in = fmaf(a_ex, c_in, h_ex);
 #pragma unroll
         for (int t = 0; t < kPer; ++t) {
-            const int j = j0 + lane * kPer + t;
+            const int j = j0 + (wave * kWave + lane) * kPer + t;
             if (j < n) dst[rev ? n - 1 - j : j] = t == 0 ? s_in : fmaf(ac[t - 1], s_in, hh[t - 1]);
         }
-        state = fmaf(a_tot, state, h_tot);
     }
+    (void)rows;
 }
 
 static TiledGeom tiled_geometry(const CoreArgs &a) {
@@ -337,7 +351,7 @@ static int launch_core_tiled_typed(const CoreArgs &a, void *workspace, hipStream
     float2 *agg = reinterpret_cast<float2 *>(workspace);
     float *carry = reinterpret_cast<float *>(agg + rows * g.nr_max);
     const uint32_t n_wg = (uint32_t)((int64_t)a.B * a.D * g.ntr * g.ntc);
-    const uint32_t carry_wg = (uint32_t)((rows + kWavesPerWg - 1) / kWavesPerWg);
+    const uint32_t carry_wg = (uint32_t)rows;                // one workgroup per (direction, image, channel)
 #define SS2D_TILED_LAUNCH(SP)                                                                                                      \
     hipLaunchKernelGGL((core_tiled_kernel<in_t, SP, false>), dim3(n_wg), dim3(kBlock), 0, stream, a, g, agg, (const float *)carry); \
     hipLaunchKernelGGL(core_carry_kernel, dim3(carry_wg), dim3(kBlock), 0, stream, (const float2 *)agg, carry, (int)rows,           \
