@@ -275,9 +275,7 @@ def odd_map_lines(reps):
     from vmamba_amd.ss2d import SS2D
     dev = "cuda:0"
     out = []
-    # (75 x 75 = 5625 positions is beyond the single kernel's LDS arrays with or without padding, so its neighbour is 80 x 80,
-    # which the tiled kernels take as well, not 72 x 72, which still fits them)
-    for odd, aligned in (((48, 96, 57, 58), (48, 96, 56, 56)), ((8, 192, 75, 75), (8, 192, 80, 80)),
+    for odd, aligned in (((48, 96, 57, 58), (48, 96, 56, 56)), ((8, 192, 75, 75), (8, 192, 72, 72)),
                          ((64, 384, 19, 19), (64, 384, 20, 20)), ((16, 96, 200, 334), (16, 96, 200, 336))):
         line = {}
         for tag, (B, D, H, W) in (("odd", odd), ("aligned", aligned)):

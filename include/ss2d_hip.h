@@ -250,7 +250,7 @@ int ss2d_cross_scan_1b1(const void *x, void *y, int B, int C, int H, int W, int 
  *          rounded to fp32 -- cross_merge_fwd's order (csm_triton.py:56-62) on the oflex fp32 scan outputs.
  * Strides in elements.  The kernel walks several images per workgroup when delta_batch_stride == height*width
  * (batch-innermost layout) and falls back to one image per workgroup otherwise.  Returns SS2D_ENOTSUP when the
- * image does not fit the kernel's LDS arrays (height*width above ~5200 for 16-bit inputs, ~3900 for fp32) or has
+ * image does not fit the kernel's LDS arrays (height*width above ~13000 for 16-bit inputs, ~9700 for fp32) or has
  * fewer than 8 positions.
  */
 typedef struct ss2d_core_params {

@@ -81,12 +81,23 @@ CORE_SHAPES = [
     (6, 5, 14, 14),      # tiles of 4 maps, the last one half full
     (2, 1, 14, 14),      # a single, half-full tile
     (12, 4, 14, 14),
+    # maps whose LDS arrays take more than a third of a CU's 160 KB (two workgroups per CU, then one): up to ~13 000 positions
+    (1, 2, 80, 80),      # 78 KB
+    (2, 1, 76, 76),      # sides multiples of 4 only
+    (1, 2, 96, 96),      # 113 KB: one workgroup per CU
+    (1, 1, 112, 112),    # 153 KB, the largest square map with sides multiples of 8
+    (1, 2, 100, 128),    # 157 KB, H != W
+    (1, 1, 75, 75),      # element-wise walk (an odd number of positions) at 69 KB
+    (1, 1, 64, 200),     # 157 KB with fewer rows than columns
 ]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape", CORE_SHAPES, ids=lambda s: "x".join(map(str, s)))
 def test_core_matches_oracle_composition(shape, dtype):
+    from vmamba_amd.core import core_fits
+    if not core_fits(shape[2], shape[3], dtype):
+        pytest.skip("fp32 maps of this size are beyond the LDS arrays (and the tiled kernels take 16-bit inputs)")
     _announce("core", shape, dtype)
     args = make_core_inputs(sum(shape), *shape, dtype)
     want = oracle_core(*args)
@@ -140,12 +151,12 @@ def test_core_small_maps_contiguous_streams_end_at_the_allocation(B):
     assert torch.allclose(got, want, **TOL), f"max abs err {(got - want).abs().max().item()}"
 
 
-# Maps that do not fit the single kernel's LDS arrays: 64 x 64 tiles, walked twice with a carry scan in between
-# (16-bit inputs, sides multiples of 8).  Whole tiles; edge tiles narrower / shorter than 64; a single row or column of
-# tiles; maps with fewer than 64 rows; several images and channels.
+# Maps that do not fit the single kernel's LDS arrays (more than ~13 000 positions): 64 x 64 tiles, walked twice with a carry
+# scan in between (16-bit inputs, sides multiples of 8).  Whole tiles; edge tiles narrower / shorter than 64; a single row
+# or column of tiles; maps with fewer than 64 rows; several images and channels.
 TILED_SHAPES = [
-    (1, 2, 128, 128), (2, 3, 80, 72), (1, 1, 64, 200), (1, 2, 256, 256), (2, 2, 8, 1024), (1, 2, 136, 64), (3, 1, 96, 104),
-    (1, 1, 1000, 8),
+    (1, 2, 128, 128), (2, 3, 144, 120), (1, 1, 64, 264), (1, 2, 256, 256), (2, 2, 8, 2048), (1, 2, 264, 64), (3, 1, 136, 120),
+    (1, 1, 2000, 8),
 ]
 
 
@@ -179,7 +190,7 @@ def test_core_large_maps_in_tiles_match_oracle_composition(shape, dtype):
 
 def test_core_tiled_optional_arguments_and_workspace_contract():
     _announce("core tiled optional")
-    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(77, 2, 2, 80, 88, torch.bfloat16)
+    x, delta, Bs, Cs, A, Dv, bias = make_core_inputs(77, 2, 2, 136, 128, torch.bfloat16)
     g = torch.Generator().manual_seed(3)
     delta_pos = (0.5 * torch.rand(delta.shape, generator=g)).to(delta.dtype)
     bias_pos = 0.5 * torch.rand(bias.shape, generator=g)
@@ -190,14 +201,15 @@ def test_core_tiled_optional_arguments_and_workspace_contract():
     # the workspace contract of the C ABI: 0 for maps the single kernel takes, a refusal where neither path applies,
     # SS2D_ENOMEM for a workspace that is too small, and the plain entry point still refuses large maps
     assert core_workspace_bytes(4, 8, 56, 56) == 0
-    assert core_workspace_bytes(1, 1, 97, 97) == _lib.SS2D_ENOTSUP            # sides not multiples of 8
-    assert core_workspace_bytes(1, 1, 96, 96, torch.float32) == _lib.SS2D_ENOTSUP
-    need = core_workspace_bytes(2, 2, 80, 88)
-    assert need == 4 * 2 * 2 * max(80 * 2, 88 * 2) * 12
+    assert core_workspace_bytes(1, 1, 112, 112) == 0                          # 153 KB of LDS: still the single kernel
+    assert core_workspace_bytes(1, 1, 129, 129) == _lib.SS2D_ENOTSUP          # sides not multiples of 8
+    assert core_workspace_bytes(1, 1, 128, 128, torch.float32) == _lib.SS2D_ENOTSUP
+    need = core_workspace_bytes(2, 2, 136, 128)
+    assert need == 4 * 2 * 2 * max(136 * 2, 128 * 3) * 12
     dev = [t.to(DEV) for t in (x, delta, Bs, Cs, A, Dv, bias)]
-    y = torch.empty(2, 2, 80 * 88, device=DEV)
+    y = torch.empty(2, 2, 136 * 128, device=DEV)
     p = _lib.CoreParams()
-    p.batch, p.dim, p.height, p.width, p.in_dtype, p.delta_softplus = 2, 2, 80, 88, _lib.SS2D_BF16, 1
+    p.batch, p.dim, p.height, p.width, p.in_dtype, p.delta_softplus = 2, 2, 136, 128, _lib.SS2D_BF16, 1
     p.x, p.delta, p.B, p.C, p.A, p.D, p.delta_bias, p.y = (t.data_ptr() for t in dev + [y])
     p.delta_dir_stride, p.delta_dim_stride, p.delta_batch_stride = dev[1].stride(0), dev[1].stride(1), dev[1].stride(2)
     p.B_dir_stride, p.B_batch_stride, p.C_dir_stride, p.C_batch_stride = dev[2].stride(0), dev[2].stride(1), dev[3].stride(0), dev[3].stride(1)
@@ -277,8 +289,8 @@ def test_core_mask_pads_marks_exactly_the_added_positions(sizes, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("shape,padded", [((3, 2, 57, 58), (60, 60)), ((5, 3, 19, 19), (20, 20)), ((2, 2, 75, 75), (80, 80)),
-                                          ((2, 1, 25, 42), (28, 44)), ((1, 2, 100, 167), (104, 168))],
+@pytest.mark.parametrize("shape,padded", [((3, 2, 57, 58), (60, 60)), ((5, 3, 19, 19), (20, 20)), ((2, 2, 75, 75), (76, 76)),
+                                          ((2, 1, 25, 42), (28, 44)), ((1, 2, 100, 167), (104, 168)), ((1, 2, 123, 125), (128, 128))],
                          ids=lambda v: "x".join(map(str, v)))
 def test_core_on_a_padded_map_equals_the_oracle_on_the_map_itself(shape, padded, dtype):
     """The embedding SS2D.forward_core_fused uses for maps with awkward sides: x zero-padded, the streams given on the
@@ -481,7 +493,7 @@ def test_core_rejections():
     with pytest.raises(RuntimeError):
         ss2d_core_hip(x.cpu(), delta, Bs, Cs, A, Dv, bias)
     # image too large for the LDS planes with sides the tiled kernels do not take: a clean "not supported", never a launch
-    big = [t.to(DEV) for t in make_core_inputs(1, 1, 1, 97, 97, torch.bfloat16)]
+    big = [t.to(DEV) for t in make_core_inputs(1, 1, 1, 129, 129, torch.bfloat16)]
     with pytest.raises(_lib.Ss2dError) as e:
         ss2d_core_hip(*big)
     assert e.value.code == _lib.SS2D_ENOTSUP

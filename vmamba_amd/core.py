@@ -25,8 +25,8 @@ def _lds_extent(n, es):
 
 def core_fits(H, W, dtype):
     """True when the fused core takes an H x W image of this dtype: at least 8 positions, and either the LDS arrays
-    of one image (two fp32 merge planes, two copies of the x map plus a block of 8 zeros each) within 64 KiB -- the single
-    kernel -- or 16-bit maps whose sides are multiples of 8, which the tiled two-pass kernels take at any size."""
+    of one image (two fp32 merge planes, two copies of the x map plus a block of 8 zeros each) within the 160 KiB of a CU --
+    the single kernel, maps of up to ~13 000 positions -- or 16-bit maps whose sides are multiples of 8, which the tiled two-pass kernels take at any size."""
     if dtype not in _DTYPE_CODE:
         return False
     L = H * W
@@ -38,7 +38,7 @@ def core_fits(H, W, dtype):
 
 def _fits_single_kernel(L, es):
     maps = _lds_extent(((L + 7) & ~7) + 8, es)
-    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 64 * 1024
+    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 160 * 1024
 
 
 def padded_map_size(H, W, dtype):

@@ -524,7 +524,12 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     }
 }
 
-constexpr size_t kCoreMaxLds = 64 * 1024;
+// What a workgroup may have of the 160 KB of LDS of a CU: all of it.  Maps of up to ~13 000 positions then run as ONE
+// workgroup per CU (four wavefronts), which still beats walking them twice in tiles (80 x 80 x 192 channels x 8 images: 59 us
+// against 145; 112 x 112 x 96 x 64: 644 against 695).  The launch passes the size as dynamic shared memory and does NOT
+// raise hipFuncAttributeMaxDynamicSharedMemorySize first: this runtime does not need it, and with the attribute set every
+// launch of that instantiation, small maps included, ran as if it held the maximum.
+constexpr size_t kCoreMaxLds = 160 * 1024;
 constexpr size_t kCoreSixPerCu = 26 * 1024;     // a sixth of the 160 KB of LDS of a CU: the kernel's registers allow six wavefronts per SIMD
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }

@@ -1,13 +1,13 @@
 // Fused SS2D core (CrossScan -> selective scan -> CrossMerge, d_state = 1) for maps of ANY size: the map is cut into
 // 64 x 64 tiles, and the kernel runs twice over the tiles with a small carry scan in between.
 //
-// The single-kernel core (ss2d_core.hip) keeps a whole map and its two merge planes in LDS, which ends at ~5200
+// The single-kernel core (ss2d_core.hip) keeps a whole map and its two merge planes in LDS, which ends at ~13 000
 // positions.  A scan direction crosses a tile as 64 separate runs of 64 consecutive positions (row pieces for the
 // row-major directions 0 / 2, column pieces for the column-major directions 1 / 3); given the state that ENTERS a run, the
 // run is an independent piece of work.  So:
 //   pass A   every workgroup takes a tile and computes, per run and direction, the run's aggregate (product of the
 //            decays, state at its end from a zero start) -- the scan operator's summary of the run;            [agg]
-//   carries  one wavefront per (direction, image, channel) combines the aggregates in that direction's order and leaves
+//   carries  one workgroup per (direction, image, channel) combines the aggregates in that direction's order and leaves
 //            the state entering every run;                                                                     [carry]
 //   pass B   every workgroup takes its tile again, starts each run from its carry and produces the outputs.
 // Both passes read x and delta once (the B / C rows are shared by the channels of an image and come from L2): 10 and 14
