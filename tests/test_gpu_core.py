@@ -89,6 +89,10 @@ CORE_SHAPES = [
     (1, 2, 100, 128),    # 157 KB, H != W
     (1, 1, 75, 75),      # element-wise walk (an odd number of positions) at 69 KB
     (1, 1, 64, 200),     # 157 KB with fewer rows than columns
+    # (above 53 KB two wavefronts per direction take alternate passes: 80 x 80 is 7 passes, 76 x 76 6, 96 x 96 9)
+    (2, 2, 72, 72),      # 5 passes and 64 positions walked one per lane
+    (1, 1, 32, 194),     # 6 passes and 64 positions; rows that are no multiple of 4
+    (3, 1, 68, 68),      # 4 passes + a fifth of 528 positions; three images
 ]
 
 

@@ -38,7 +38,7 @@ def core_fits(H, W, dtype):
 
 def _fits_single_kernel(L, es):
     maps = _lds_extent(((L + 7) & ~7) + 8, es)
-    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 160 * 1024
+    return L >= 8 and 2 * _lds_extent(L, 4) * 4 + 2 * maps * es <= 160 * 1024 - 256
 
 
 def padded_map_size(H, W, dtype):

@@ -87,10 +87,24 @@ struct CorePassLoads {
     uint32_t img, j0;     // first element of the image (its index times L) and position in it of the lane's first item
 };
 
-template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta, bool kWide>
-__global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD, FastDiv divTiles,
+// kWpd > 1: kWpd wavefronts per direction (8 or 16 in the workgroup), for maps whose LDS arrays leave a CU one or two
+// workgroups -- four or eight wavefronts on a CU cannot hide the LDS round trips and barriers of the plane updates, which
+// come one after the other.  The wavefronts of a direction take the passes of a ROUND of kWpd passes side by side:
+// everything of a pass that does not need the incoming state -- loads, softplus, decays, the scan inside the lanes and
+// across the wavefront -- then each leaves its pass's aggregate in LDS, a barrier, each folds the aggregates of the passes
+// before its own into the state the round started from, and the plane updates of the whole round happen in the usual two
+// phases (the passes of a round cover different positions, so the forward wavefronts do not meet each other, nor the
+// backward ones).  Two barriers and two update phases per kWpd passes instead of per pass.
+template <typename in_t, bool kSoftplus, int kGran, bool kVecDelta, bool kWide, int kWpd = 1>
+__global__ __launch_bounds__(kWpd * kBlock, (kWpd > 1 ? 4 : core_min_waves<in_t, kGran, kWide>())) void ss2d_core_kernel(const CoreArgs p, FastDiv divL, FastDiv divW, FastDiv divD, FastDiv divTiles,
                                                            FastDiv divWt) {
     extern __shared__ __align__(16) float core_smem[];
+    static_assert(kWpd == 1 || kWide, "several wavefronts per direction: the 16-positions-per-lane variant only");
+    constexpr bool kPair = kWpd > 1;
+    constexpr int kThreads = kWpd * kBlock;
+    constexpr int kStride = kWpd;                        // passes from one pass of a wavefront to its next
+    __shared__ float s_carry[4];                         // kWpd > 1: the state after the latest finished round, per direction
+    __shared__ float2 s_agg[4][4];                       // ... and the aggregates of the current round's passes [direction][wavefront]
     constexpr int kEs = (int)sizeof(in_t);
     constexpr bool kFlat = core_flat_maps<in_t, kGran>();
     static_assert(!kWide || core_flat_maps<in_t, kGran>(), "16 positions per lane: 16-bit maps walked in blocks of 8 only");
@@ -118,7 +132,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
 
     // ---- this wavefront's direction ---------------------------------------------------------------------------
     const int lane = threadIdx.x & (kWave - 1);
-    const int dir = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int dir = wave_id & 3, half = wave_id >> 2;    // (half is 0 without kPair)
     const int zero_block = core_zero_block(n_max);
     const in_t *xs = (dir & 1) ? xT : xR;
     float *plane = (dir & 1) ? planeB : planeA;
@@ -143,8 +158,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     // Image and position of this lane's first item in the pass issued next: passes are issued strictly in order, so
     // the pair just advances by 512 positions each time (no division in the loop).
     uint32_t next_img, next_j, step_img, step_j;
-    divmod((uint32_t)(lane * kIt), divL, next_img, next_j);
-    divmod((uint32_t)kPassLen, divL, step_img, step_j);
+    divmod((uint32_t)(lane * kIt + half * kPassLen), divL, next_img, next_j);
+    divmod((uint32_t)(kStride * kPassLen), divL, step_img, step_j);
     next_img *= (uint32_t)L; step_img *= (uint32_t)L;
     auto issue = [&](int pass, Loads &r) {
         const int e0 = pass * kPassLen + lane * kIt;
@@ -194,24 +209,24 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     Loads regs[kCoreBurst];
 #pragma unroll
     for (int q = 0; q < kCoreBurst; ++q)
-        if (q < n_pass) issue(q, regs[q]);
+        if (kStride * q + half < n_pass) issue(kStride * q + half, regs[q]);
 
     // ---- stage: copy the maps into xR / xT ------------------------------------------------------------------------
     const in_t *xin = reinterpret_cast<const in_t *>(p.x);
     auto stage_elements = [&]() {
         constexpr int kChunk = 8;
-        for (int base = 0; base < n_el; base += kChunk * kBlock) {
+        for (int base = 0; base < n_el; base += kChunk * kThreads) {
             in_t v[kChunk];
             uint32_t ii[kChunk], rr[kChunk];
 #pragma unroll
             for (int u = 0; u < kChunk; ++u) {
-                const int idx = base + u * kBlock + (int)threadIdx.x;
+                const int idx = base + u * kThreads + (int)threadIdx.x;
                 divmod((uint32_t)min(idx, n_el - 1), divL, ii[u], rr[u]);
                 v[u] = xin[((size_t)(b0 + ii[u]) * p.D + d) * L + rr[u]];
             }
 #pragma unroll
             for (int u = 0; u < kChunk; ++u) {
-                const int idx = base + u * kBlock + (int)threadIdx.x;
+                const int idx = base + u * kThreads + (int)threadIdx.x;
                 if (idx < n_el) {
                     uint32_t h, w;
                     divmod(rr[u], divW, h, w);
@@ -226,7 +241,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     // with byte permutes and go into the column-major map, 8 bytes at a time.
     auto stage_tiles = [&]() {
         const int n_tiles = nb * (int)divTiles.d;        // tiles per image: (H / 4) * (W / 4)
-        for (int q = threadIdx.x; q < n_tiles; q += kBlock) {
+        for (int q = threadIdx.x; q < n_tiles; q += kThreads) {
             uint32_t img, rest, hb, wb;
             divmod((uint32_t)q, divTiles, img, rest);
             divmod(rest, divWt, hb, wb);
@@ -262,7 +277,10 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     // does the block behind the maps
     {
         float4 *planes4 = reinterpret_cast<float4 *>(planeA);
-        for (int i = threadIdx.x; i < 2 * plane_ext / 4; i += kBlock) planes4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int i = threadIdx.x; i < 2 * plane_ext / 4; i += kThreads) planes4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if constexpr (kPair) {
+            if (threadIdx.x < 4) s_carry[threadIdx.x] = 0.0f;
+        }
         if (threadIdx.x < 2 * kItems) {
             in_t *m = threadIdx.x < kItems ? xR : xT;
             m[map_index<kEs, kFlat>(core_zero_block(n_max) + (int)(threadIdx.x % kItems))] = in_t{};
@@ -280,7 +298,12 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
     // One pass: the states h of its items in yv (scan order) and the plane slots of its groups; the plane update
     // multiplies by C as it adds.  The skip term D * u is the same multiple of x[r] in all four directions and is added
     // once, in the merge.
-    auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kIt], GroupSlot (&slot)[kGroups]) {
+    // kDefer (kPair): stops before the incoming state is needed -- yv receives the lane's running products, hv its states
+    // from a zero start, ex the wavefront scan's (a_ex, h_ex, a_tot, h_tot) -- and apply_carry finishes the pass.
+    struct WaveScan { float a_ex, h_ex, a_tot, h_tot; };
+    auto compute = [&](bool reverse, int pass, const Loads &r, float &h_carry, float (&yv)[kIt], GroupSlot (&slot)[kGroups], auto defer_tag,
+                       float (&hv)[kIt], WaveScan &ex) {
+        constexpr bool kDefer = decltype(defer_tag)::value;
         const int e0 = pass * kPassLen + lane * kIt;
         const int j0 = (int)r.j0;
         const int k = kGran == kIt ? kIt : min(kIt, L - j0);
@@ -354,10 +377,30 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         }
         float a_ex, h_ex, a_tot, h_tot;
         wave_scan_pairs(ac[kIt - 1], hh[kIt - 1], a_ex, h_ex, a_tot, h_tot);
-        const float s_in = fmaf(a_ex, h_carry, h_ex);
-        h_carry = fmaf(a_tot, h_carry, h_tot);
+        if constexpr (kDefer) {
+            ex.a_ex = a_ex; ex.h_ex = h_ex; ex.a_tot = a_tot; ex.h_tot = h_tot;
 #pragma unroll
-        for (int i = 0; i < kIt; ++i) yv[i] = fmaf(ac[i], s_in, hh[i]);
+            for (int i = 0; i < kIt; ++i) { yv[i] = ac[i]; hv[i] = hh[i]; }
+        } else {
+            const float s_in = fmaf(a_ex, h_carry, h_ex);
+            h_carry = fmaf(a_tot, h_carry, h_tot);
+#pragma unroll
+            for (int i = 0; i < kIt; ++i) yv[i] = fmaf(ac[i], s_in, hh[i]);
+        }
+    };
+    // the rest of a deferred pass: the state that enters the round folded with the aggregates of the round's earlier passes;
+    // returns the state after this pass
+    auto apply_carry = [&](float (&yv)[kIt], const float (&hv)[kIt], const WaveScan &ex) {
+        float h_carry = s_carry[dir];
+#pragma unroll
+        for (int w = 0; w < kWpd - 1; ++w) {
+            const float2 g = s_agg[dir][w];
+            if (w < half) h_carry = fmaf(g.x, h_carry, g.y);
+        }
+        const float s_in = fmaf(ex.a_ex, h_carry, ex.h_ex);
+#pragma unroll
+        for (int i = 0; i < kIt; ++i) yv[i] = fmaf(yv[i], s_in, hv[i]);
+        return fmaf(ex.a_tot, h_carry, ex.h_tot);
     };
 
     // Plane update of one pass: every entry is reached once by the forward and once by the backward direction of its
@@ -385,9 +428,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
 
     // The short last pass: lane l holds stream position kPassLen * n_pass + l.  Same arithmetic and the same two-barrier
     // plane update as a full pass, one item per lane.
-    auto short_pass = [&](bool reverse, float h_carry) {
+    auto short_pass = [&](bool reverse, float h_carry, bool active) {
         const int e = n_pass * kPassLen + lane;
-        const bool valid = e < n_el;
+        const bool valid = active && e < n_el;
         uint32_t i, jj;
         divmod((uint32_t)min(e, n_el - 1), divL, i, jj);
         const int base = reverse ? (int)(i * L) + L - 1 - (int)jj : e;      // this direction's index of the position
@@ -415,7 +458,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         __syncthreads();
     };
 
-    {
+    if constexpr (!kPair) {
         float h_carry = 0.0f;
         for (int pass0 = 0; pass0 < n_pass; pass0 += kCoreBurst) {
 #pragma unroll
@@ -424,7 +467,8 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
                 if (pass < n_pass) {                 // uniform over the workgroup: every wavefront meets every barrier
                     float yv[kIt];
                     GroupSlot slot[kGroups];
-                    compute(reverse, pass, regs[q], h_carry, yv, slot);
+                    WaveScan unused;
+                    compute(reverse, pass, regs[q], h_carry, yv, slot, std::false_type{}, yv, unused);
                     if (!reverse) update_plane(false, regs[q], yv, slot);
                     __syncthreads();
                     if (reverse) update_plane(true, regs[q], yv, slot);
@@ -433,7 +477,39 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
                 }
             }
         }
-        if (short_tail) short_pass(reverse, h_carry);
+        if (short_tail) short_pass(reverse, h_carry, true);
+    } else {
+        // rounds of kWpd passes: pass kWpd * round + w belongs to wavefront w of each direction
+        const int n_round = (n_pass + kWpd - 1) / kWpd;
+        for (int r0 = 0; r0 < n_round; r0 += kCoreBurst) {
+#pragma unroll
+            for (int q = 0; q < kCoreBurst; ++q) {
+                const int round = r0 + q;
+                if (round < n_round) {               // uniform over the workgroup
+                    const int pass = kWpd * round + half;
+                    const bool active = pass < n_pass;                          // uniform over the wavefront
+                    const bool last = pass == min(kWpd * round + kWpd, n_pass) - 1;   // the round's last pass: its owner hands on the state
+                    float yv[kIt], hv[kIt];
+                    GroupSlot slot[kGroups];
+                    WaveScan ex;
+                    float unused = 0.0f;
+                    if (active) {
+                        compute(reverse, pass, regs[q], unused, yv, slot, std::true_type{}, hv, ex);
+                        if (lane == 0 && half < kWpd - 1) s_agg[dir][half] = make_float2(ex.a_tot, ex.h_tot);
+                    }
+                    __syncthreads();                 // aggregates of this round, state and plane updates of the round before
+                    float h_out = 0.0f;
+                    if (active) h_out = apply_carry(yv, hv, ex);
+                    if (active && !reverse) update_plane(false, regs[q], yv, slot);
+                    __syncthreads();
+                    if (active && reverse) update_plane(true, regs[q], yv, slot);
+                    if (last && lane == 0) s_carry[dir] = h_out;               // (everyone has read the old one before the barrier above)
+                    if (active && pass + kWpd * kCoreBurst < n_pass) issue(pass + kWpd * kCoreBurst, regs[q]);
+                }
+            }
+        }
+        __syncthreads();                             // the last state and the last plane updates are in place
+        if (short_tail) short_pass(reverse, s_carry[dir], half == 0);
     }
 
     // ---- merge: out[r] = (A[r] + B[t(r)]) + (D0 + D1 + D2 + D3) * x[r] ---------------------------------------------
@@ -450,7 +526,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         // four consecutive entries of plane A each, its columns four consecutive entries of plane B each -- the
         // transposition is a renaming of registers -- and every row leaves as one 16-byte store.
         const int n_tiles = nb * (int)divTiles.d;
-        for (int q = threadIdx.x; q < n_tiles; q += kBlock) {
+        for (int q = threadIdx.x; q < n_tiles; q += kThreads) {
             uint32_t img, rest, hb, wb;
             divmod((uint32_t)q, divTiles, img, rest);
             divmod(rest, divWt, hb, wb);
@@ -479,12 +555,12 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         // four consecutive positions per lane (L is a multiple of kGran, so they share an image and, with W >= 4, span
         // at most two rows): one 16-byte store
         const int n_quad = n_el / 4;
-        for (int base = 0; base < n_quad; base += 2 * kBlock) {
+        for (int base = 0; base < n_quad; base += 2 * kThreads) {
             float4 v[2];
             size_t off[2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                const int idx = 4 * min(base + u * kBlock + (int)threadIdx.x, n_quad - 1);
+                const int idx = 4 * min(base + u * kThreads + (int)threadIdx.x, n_quad - 1);
                 uint32_t i, r, h, w;
                 divmod((uint32_t)idx, divL, i, r);
                 divmod(r, divW, h, w);
@@ -501,16 +577,16 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
             }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
-                if (base + u * kBlock + (int)threadIdx.x < n_quad) *reinterpret_cast<float4 *>(yo + off[u]) = v[u];
+                if (base + u * kThreads + (int)threadIdx.x < n_quad) *reinterpret_cast<float4 *>(yo + off[u]) = v[u];
         }
         return;
     }
-    for (int base = 0; base < n_el; base += 4 * kBlock) {
+    for (int base = 0; base < n_el; base += 4 * kThreads) {
         float v[4];
         size_t off[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int idx = min(base + u * kBlock + (int)threadIdx.x, n_el - 1);
+            const int idx = min(base + u * kThreads + (int)threadIdx.x, n_el - 1);
             uint32_t i, r, h, w;
             divmod((uint32_t)idx, divL, i, r);
             divmod(r, divW, h, w);
@@ -520,7 +596,7 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-            if (base + u * kBlock + (int)threadIdx.x < n_el) yo[off[u]] = v[u];
+            if (base + u * kThreads + (int)threadIdx.x < n_el) yo[off[u]] = v[u];
     }
 }
 
@@ -529,7 +605,9 @@ __global__ __launch_bounds__(kBlock, (core_min_waves<in_t, kGran, kWide>())) voi
 // against 145; 112 x 112 x 96 x 64: 644 against 695).  The launch passes the size as dynamic shared memory and does NOT
 // raise hipFuncAttributeMaxDynamicSharedMemorySize first: this runtime does not need it, and with the attribute set every
 // launch of that instantiation, small maps included, ran as if it held the maximum.
-constexpr size_t kCoreMaxLds = 160 * 1024;
+constexpr size_t kCoreMaxLds = 160 * 1024 - 256;      // (the kernel has 144 bytes of static LDS besides the arrays)
+constexpr size_t kCorePairLds = 53 * 1024;            // above a third of a CU's LDS: at most two workgroups per CU
+constexpr size_t kCoreQuadLds = 80 * 1024;            // above half: one
 constexpr size_t kCoreSixPerCu = 26 * 1024;     // a sixth of the 160 KB of LDS of a CU: the kernel's registers allow six wavefronts per SIMD
 
 static int core_gcd(int64_t a, int64_t b) { while (b) { const int64_t t = a % b; a = b; b = t; } return (int)(a < 0 ? -a : a); }
@@ -608,11 +686,17 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
     if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
     const FastDiv dL = make_fastdiv((uint32_t)L), dW = make_fastdiv((uint32_t)a.W), dD = make_fastdiv((uint32_t)a.D);
     const FastDiv dT = make_fastdiv((uint32_t)(tiled ? (a.H / 4) * (a.W / 4) : 1)), dWt = make_fastdiv((uint32_t)(tiled ? a.W / 4 : 1));
+    // several wavefronts per direction where the arrays leave a CU two workgroups (two each) or one (four)
+    const int wpd = !(wide && smem > kCorePairLds) ? 1 : smem > kCoreQuadLds ? 4 : 2;
 #define SS2D_CORE_LAUNCH_W(SP, G, V, W16)                                                                                         \
     hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, V, W16>), dim3((uint32_t)n_wg), dim3(kBlock), smem, stream, a, dL, dW, dD, dT, dWt)
+#define SS2D_CORE_LAUNCH_P(SP, G, V, WPD)                                                                                         \
+    hipLaunchKernelGGL((ss2d_core_kernel<in_t, SP, G, V, true, WPD>), dim3((uint32_t)n_wg), dim3(WPD * kBlock), smem, stream, a, dL, dW, dD, dT, dWt)
 #define SS2D_CORE_LAUNCH(SP, G)                                                                                                     \
     do {                                                                                                                            \
         if constexpr (G == kItems && sizeof(in_t) == 2) {                                                                          \
+            if (wpd == 4) { if (a.vec_ok) SS2D_CORE_LAUNCH_P(SP, G, true, 4); else SS2D_CORE_LAUNCH_P(SP, G, false, 4); break; }  \
+            if (wpd == 2) { if (a.vec_ok) SS2D_CORE_LAUNCH_P(SP, G, true, 2); else SS2D_CORE_LAUNCH_P(SP, G, false, 2); break; }  \
             if (wide) { if (a.vec_ok) SS2D_CORE_LAUNCH_W(SP, G, true, true); else SS2D_CORE_LAUNCH_W(SP, G, false, true); break; } \
         }                                                                                                                           \
         if (a.vec_ok) SS2D_CORE_LAUNCH_W(SP, G, true, false); else SS2D_CORE_LAUNCH_W(SP, G, false, false);                         \
@@ -623,6 +707,7 @@ static int launch_core(CoreArgs a, hipStream_t stream) {
         if (g == 8) SS2D_CORE_LAUNCH(false, 8); else if (g == 4) SS2D_CORE_LAUNCH(false, 4); else SS2D_CORE_LAUNCH(false, 1);
     }
 #undef SS2D_CORE_LAUNCH_W
+#undef SS2D_CORE_LAUNCH_P
 #undef SS2D_CORE_LAUNCH
     return launch_status();
 }
