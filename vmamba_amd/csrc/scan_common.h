@@ -377,8 +377,9 @@ __device__ __forceinline__ void gather_group(__amdgpu_buffer_rsrc_t rsrc, uint32
 // ---- short rows: one segment of a row per lane (ss2d_core_small.hip, scan_small.hip) --------------------------------
 // Inclusive scan of (a, h) pairs over the 16-lane DPP row, in lane order or in reverse lane order; returns the
 // EXCLUSIVE h (the state entering this lane; 0 for the first lane of the row).  Lanes without a source keep their value.
+// a_incl (optional) receives the inclusive product of a up to this lane.
 template <bool kReverse>
-__device__ __forceinline__ float row_scan_state_in(float a, float h) {
+__device__ __forceinline__ float row_scan_state_in(float a, float h, float *a_incl = nullptr) {
     float hx = 0.0f;
 #define SS2D_ROW_STEP(CTRL)                                         \
     "v_fmac_f32_dpp %1, %1, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t" \
@@ -398,6 +399,7 @@ __device__ __forceinline__ float row_scan_state_in(float a, float h) {
             : "+v"(a), "+v"(h), "+v"(hx));
     }
 #undef SS2D_ROW_STEP
+    if (a_incl) *a_incl = a;
     return hx;
 }
 

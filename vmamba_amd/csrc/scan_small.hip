@@ -159,7 +159,8 @@ __global__ __launch_bounds__(kBlock) void scan_small_kernel(const ScanArgs p, in
         // lanes that hold no segment stop the state: nothing travels from one group of lanes into the next (the first
         // lane of a DPP row has no lane below it)
         const float a_tot = active ? ac[kNi - 1] : 0.0f, h_tot = active ? hh[kNi - 1] : 0.0f;
-        const float h_in = row_scan_state_in<false>(a_tot, h_tot);
+        float a_incl = 1.0f;
+        const float h_in = row_scan_state_in<false>(a_tot, h_tot, kX ? &a_incl : nullptr);
         float y[kNi];
 #pragma unroll
         for (int j = 0; j < kNi; ++j) y[j] = fmaf(Cv.item(j), fmaf(ac[j], h_in, hh[j]), Dk * uu.item(j));
@@ -167,11 +168,15 @@ __global__ __launch_bounds__(kBlock) void scan_small_kernel(const ScanArgs p, in
             // the product of the row's lane products ends up in its last lane: each step multiplies in the lane 1 / 2 / 4
             // (/ 8) below, lanes without a source and idle lanes count as 1, and with groups of 8 lanes the steps stop
             // at 4 so that a lane reaches back 7 lanes, to its own group's idle lane at most
-            float pr = active ? ac[kNi - 1] : 1.0f;
-            pr *= dpp_move<kDppRowShr1>(1.0f, pr);
-            pr *= dpp_move<kDppRowShr2>(1.0f, pr);
-            pr *= dpp_move<kDppRowShr4>(1.0f, pr);
-            if constexpr (kLanes == 16) pr *= dpp_move<kDppRowShr8>(1.0f, pr);
+            // (with one row per DPP row -- 16 lanes, 14 x 14 maps -- the scan above has left exactly that product in the
+            // row's last lane: no idle lane sits below it)
+            float pr = a_incl;
+            if constexpr (kLanes != 16) {
+                pr = active ? ac[kNi - 1] : 1.0f;
+                pr *= dpp_move<kDppRowShr1>(1.0f, pr);
+                pr *= dpp_move<kDppRowShr2>(1.0f, pr);
+                pr *= dpp_move<kDppRowShr4>(1.0f, pr);
+            }
             if (active && i == kNl - 1) {
                 float *xo = p.x + (int64_t)(row0 + g) * 2;
                 xo[0] = pr;
