@@ -117,6 +117,8 @@ GRID = [
     # rows that end at most 128 positions past a full 512-position pass (the one-state kernel walks those one per lane):
     # across a 2048-chunk boundary, two tail passes with the second partial, exactly two, a short one, no full pass
     (1, 8, 4, 1, 2112), (2, 8, 4, 1, 1128), (1, 8, 2, 1, 128), (2, 8, 4, 1, 520), (1, 8, 4, 1, 72),
+    # few long rows (four wavefronts per row): ending four positions into a lane's eight, into a chunk, and on a chunk
+    (1, 4, 2, 1, 2052), (2, 8, 4, 1, 6148), (1, 8, 4, 1, 4096), (1, 4, 1, 1, 10240 + 264),
 ]
 
 

@@ -158,6 +158,63 @@ __device__ __forceinline__ void store_items(T *__restrict__ row, int pos, int L,
 
 constexpr int kBufferRsrcWord3 = 0x00020000;   // raw buffer, 32-bit data format (gfx9 family)
 
+// A row of n_elems elements seen through a buffer descriptor: 32-bit byte offsets, and the hardware checks every dword
+// against the row's end -- a load past it returns 0, a store past it is dropped -- so loads and stores need no branch.
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_buffer(const T *row, int n_elems) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(row), 0, n_elems * (int)sizeof(T), kBufferRsrcWord3);
+}
+
+// Eight elements from position `pos` of such a row (16-byte aligned: the vector paths' precondition).
+template <typename T>
+__device__ __forceinline__ Raw8<T> load_raw_buffer(__amdgpu_buffer_rsrc_t rsrc, int pos) {
+    Raw8<T> r;
+    const int byte_off = pos * (int)sizeof(T);
+    const auto lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
+    r.w[0] = lo[0]; r.w[1] = lo[1]; r.w[2] = lo[2]; r.w[3] = lo[3];
+    if constexpr (sizeof(T) == 4) {
+        const auto hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, 0, 0);
+        r.w[4] = hi[0]; r.w[5] = hi[1]; r.w[6] = hi[2]; r.w[7] = hi[3];
+    }
+    return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_items_buffer(__amdgpu_buffer_rsrc_t rsrc, int pos, const float (&v)[kItems]) {
+    typedef uint32_t words4_t __attribute__((ext_vector_type(4)));
+    const int byte_off = pos * (int)sizeof(T);
+    if constexpr (sizeof(T) == 2) {
+        words4_t w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = pack2_from_f32<T>(v[2 * i], v[2 * i + 1]);
+        __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, byte_off, 0, 0);
+    } else {
+        words4_t lo, hi;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo[i] = f32_to_bits(v[i]); hi[i] = f32_to_bits(v[4 + i]); }
+        __builtin_amdgcn_raw_buffer_store_b128(lo, rsrc, byte_off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(hi, rsrc, byte_off + 16, 0, 0);
+    }
+}
+
+// A pass's outputs, 8 consecutive positions per lane, stored as fp32 so that each store instruction writes 1 KB of
+// consecutive addresses: at 32 bytes per lane an instruction would write every other 16 bytes of a 2 KB span, and
+// memory takes the half-written lines measurably worse (one-state row scan of 56 x 56 maps, batch 128: 258 -> 232 us).
+// The values go through a wavefront-private LDS tile of kPass floats (LDS serves a wavefront's accesses in order:
+// no barrier), lane l then holds positions 4l .. 4l+3 and 256+4l .. 256+4l+3 of the pass.
+__device__ __forceinline__ void store_pass_f32(float *tile, __amdgpu_buffer_rsrc_t rsrc, int pass_pos, int lane,
+                                               const float (&v)[kItems]) {
+    typedef uint32_t words4_t __attribute__((ext_vector_type(4)));
+    float4 *t4 = reinterpret_cast<float4 *>(tile);
+    t4[2 * lane] = make_float4(v[0], v[1], v[2], v[3]);
+    t4[2 * lane + 1] = make_float4(v[4], v[5], v[6], v[7]);
+    const float4 lo = t4[lane], hi = t4[kWave + lane];
+    const words4_t wl = {f32_to_bits(lo.x), f32_to_bits(lo.y), f32_to_bits(lo.z), f32_to_bits(lo.w)};
+    const words4_t wh = {f32_to_bits(hi.x), f32_to_bits(hi.y), f32_to_bits(hi.z), f32_to_bits(hi.w)};
+    __builtin_amdgcn_raw_buffer_store_b128(wl, rsrc, (pass_pos + 4 * lane) * 4, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(wh, rsrc, (pass_pos + kPass / 2 + 4 * lane) * 4, 0, 0);
+}
+
 template <typename T>
 __device__ __forceinline__ float gather_elem(__amdgpu_buffer_rsrc_t rsrc, uint32_t elem_offset) {
     if constexpr (sizeof(T) == 2) {

@@ -83,6 +83,9 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
     const bool short_tail = kShortTail;
     const int n_pass = short_tail ? L / kPass : (L + kPass - 1) / kPass;
     const int L_body = short_tail ? n_pass * kPass : L;              // what the 8-per-lane passes cover
+    constexpr bool kTiledStore = kVec && sizeof(out_t) == 4;     // fp32 out as whole 1 KB runs (store_pass_f32)
+    __shared__ __align__(16) float y_tile[kTiledStore ? kWavesPerWg : 1][kTiledStore ? kPass : 4];
+    const __amdgpu_buffer_rsrc_t o_buf = row_buffer(o_row, kTiledStore ? L_body : 0);
     for (int pass0 = 0; pass0 < n_pass; pass0 += kBurst) {
         Raw8<in_t> u_burst[kBurst], dl_burst[kBurst], B_burst[kBurst], C_burst[kBurst];
 #pragma unroll
@@ -155,7 +158,8 @@ __global__ __launch_bounds__(kBlock) void scan_row_kernel(const ScanArgs p) {
                 }
             }
         }
-        store_items<out_t, kVec>(o_row, pos, L_body, y);
+        if constexpr (kVec && sizeof(out_t) == 4) store_pass_f32(y_tile[wave], o_buf, pass * kPass, lane, y);
+        else store_items<out_t, kVec>(o_row, pos, L_body, y);
         }
     }
     if constexpr (kShortTail) {
@@ -228,6 +232,9 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
     const __amdgpu_buffer_rsrc_t B_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.B), 0, (int)p.B_span_bytes, kBufferRsrcWord3);
     const __amdgpu_buffer_rsrc_t C_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.C), 0, (int)p.C_span_bytes, kBufferRsrcWord3);
     out_t *o_base = reinterpret_cast<out_t *>(p.out) + r0 * L;
+    // fp32 out leaves as whole 1 KB runs (store_pass_f32); the descriptor drops what lies past the run's last element
+    __shared__ __align__(16) float y_tile[sizeof(out_t) == 4 ? kWavesPerWg : 1][sizeof(out_t) == 4 ? kPass : 4];
+    const __amdgpu_buffer_rsrc_t o_buf = row_buffer(o_base, sizeof(out_t) == 4 ? n_el : 0);
 
     float h_reg[kN], g_reg[kX ? kN : 1];
 #pragma unroll
@@ -363,7 +370,8 @@ __global__ __launch_bounds__(kBlock) void scan_flat_kernel(const ScanArgs p, int
             for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
             h_reg[n] = fmaf(a_tot, h_reg[n], h_tot);
         }
-        if (full) store_items<out_t, true>(o_base, e0, n_el, y);
+        if constexpr (sizeof(out_t) == 4) store_pass_f32(y_tile[wave], o_buf, pass * kPass, lane, y);
+        else if (full) store_items<out_t, true>(o_base, e0, n_el, y);
         else store_items<out_t, false>(o_base, e0, n_el, y);
     }
 }
@@ -395,6 +403,9 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
     const float bias = p.bias ? p.bias[dg] : 0.0f;
     const int L = p.L;
 
+    constexpr bool kTiledStore = kVec && sizeof(out_t) == 4;     // fp32 out as whole 1 KB runs (store_pass_f32)
+    __shared__ __align__(16) float y_tile[kTiledStore ? kWavesPerWg : 1][kTiledStore ? kPass : 4];
+    const __amdgpu_buffer_rsrc_t o_buf = row_buffer(o_row, kTiledStore ? L : 0);
     const int n_chunks = (L + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
     // the next chunk's u / delta (and B / C of the first state) are requested before this chunk's arithmetic and its
     // barriers: a wavefront always has a chunk of loads in flight (positions past the row's end come back as the fill)
@@ -458,8 +469,115 @@ __global__ __launch_bounds__(kBlock) void scan_row4_kernel(const ScanArgs p) {
                 }
             }
         }
-        store_items<out_t, kVec>(o_row, pos, L, y);
+        if constexpr (kTiledStore) store_pass_f32(y_tile[wave], o_buf, chunk * SS2D_SCAN_CHUNK + wave * kPass, lane, y);
+        else store_items<out_t, kVec>(o_row, pos, L, y);
     }
+}
+
+// ---- four wavefronts per row, one state, 16-byte vectors: the chunks' loads in a ring ----------------------------------
+// The same split of a row, with u, delta, B, C and out addressed through buffer descriptors: every load and store is
+// unconditional (the hardware drops what lies past the row's end) and every chunk is the same instruction stream, so
+// the memory counter -- loads and stores retire in issue order -- can be waited on exactly.  A chunk waits for ITS four
+// loads while those of the next kRing - 1 chunks and the stores of the last ones are in flight, and re-issues its
+// registers for the chunk kRing ahead when it is done with them.  (With loads under per-lane conditions the compiler
+// has to wait for everything outstanding, the stores of the chunk before included, ahead of each chunk.)
+template <typename in_t, typename out_t, bool kSoftplus>
+__global__ __launch_bounds__(kBlock, 6) void scan_row4_ring_kernel(const ScanArgs p) {
+    constexpr int kRing = 2;      // three chunks deep measured the same and leaves a SIMD four wavefronts instead of six
+    __shared__ float2 agg[2][kWavesPerWg];                           // pass totals, by chunk parity
+    __shared__ float2 state[2];                                      // (running a-product, h) entering a chunk
+    constexpr bool kTiledStore = sizeof(out_t) == 4;
+    __shared__ __align__(16) float y_tile[kTiledStore ? kWavesPerWg : 1][kTiledStore ? kPass : 4];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int row = (int)xcd_contiguous_id(blockIdx.x, gridDim.x);   // grid == rows exactly
+
+    const int b = row / p.dim, d = row - b * p.dim;
+    const int grp = d / p.dim_per_group, dg = d / p.dim_per_delta;
+    const int L = p.L;
+    const __amdgpu_buffer_rsrc_t u_buf = row_buffer(reinterpret_cast<const in_t *>(p.u) + b * p.u_bs + d * p.u_ds, L),
+                                 dl_buf = row_buffer(reinterpret_cast<const in_t *>(p.delta) + b * p.dl_bs + dg * p.dl_ds, L),
+                                 B_buf = row_buffer(reinterpret_cast<const in_t *>(p.B) + b * p.B_bs + grp * p.B_gs, L),
+                                 C_buf = row_buffer(reinterpret_cast<const in_t *>(p.C) + b * p.C_bs + grp * p.C_gs, L),
+                                 o_buf = row_buffer(reinterpret_cast<out_t *>(p.out) + b * p.o_bs + d * p.o_ds, L);
+    float *x_row = p.x ? p.x + (size_t)row * p.n_chunks * 2 : nullptr;
+    const float A_log2e = p.A[d * p.A_ds] * kLog2e;
+    const float Dv = p.D ? p.D[d] : 0.0f;
+    const float bias = p.bias ? p.bias[dg] : 0.0f;
+
+    const int n_chunks = (L + SS2D_SCAN_CHUNK - 1) / SS2D_SCAN_CHUNK;
+    const int pos_first = wave * kPass + lane * kItems;
+    struct ChunkLoads { Raw8<in_t> u, dl, B, C; };
+    ChunkLoads ring[kRing];
+    auto issue = [&](int chunk, ChunkLoads &r) {                     // a chunk beyond the row reads nothing
+        const int pos = chunk * SS2D_SCAN_CHUNK + pos_first;
+        r.u = load_raw_buffer<in_t>(u_buf, pos);
+        r.dl = load_raw_buffer<in_t>(dl_buf, pos);
+        r.B = load_raw_buffer<in_t>(B_buf, pos);
+        r.C = load_raw_buffer<in_t>(C_buf, pos);
+    };
+#pragma unroll
+    for (int s = 0; s < kRing; ++s) {
+        issue(s, ring[s]);
+        __builtin_amdgcn_sched_barrier(0);       // in chunk order, as the loop issues them: the waits count on it
+    }
+    auto do_chunk = [&](int chunk, const ChunkLoads &r) {
+        const int par = chunk & 1;
+        const int pos = chunk * SS2D_SCAN_CHUNK + pos_first;
+        float dl[kItems], du[kItems], y[kItems], Bv[kItems], Cv[kItems];
+        prepare_delta_u<in_t, kSoftplus>(r.u, r.dl, kItems, bias, Dv, dl, du, y);
+        unpack_raw<in_t>(r.B, Bv);
+        unpack_raw<in_t>(r.C, Cv);
+        if (chunk == n_chunks - 1) {
+            // lanes past the row's end were fed zeros: u = 0 already makes their b term 0; their step must be 0 too
+            // (a = 1), or the state the row ends with would go on decaying
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) dl[i] = pos + i < L ? dl[i] : 0.0f;   // (fp32 rows may end mid-lane)
+        }
+        float ac[kItems], hh[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const float a = __builtin_amdgcn_exp2f(dl[i] * A_log2e);
+            const float bb = Bv[i] * du[i];
+            ac[i] = i == 0 ? a : ac[i - 1] * a;
+            hh[i] = i == 0 ? bb : fmaf(a, hh[i - 1], bb);
+        }
+        float a_ex, h_ex, a_tot, h_tot;
+        wave_scan_pairs(ac[kItems - 1], hh[kItems - 1], a_ex, h_ex, a_tot, h_tot);
+        if (lane == 0) agg[par][wave] = make_float2(a_tot, h_tot);
+        __syncthreads();
+        const float2 st = chunk == 0 ? make_float2(1.0f, 0.0f) : state[par];
+        float cin = st.y, aprod = st.x;
+#pragma unroll
+        for (int j = 0; j < kWavesPerWg; ++j) {
+            const float2 g = agg[par][j];
+            if (j < wave) cin = fmaf(g.x, cin, g.y);
+            aprod *= g.x;
+        }
+        const float s_in = fmaf(a_ex, cin, h_ex);
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) y[i] = fmaf(Cv[i], fmaf(ac[i], s_in, hh[i]), y[i]);
+        if (wave == kWavesPerWg - 1 && lane == 0) {
+            const float h_end = fmaf(a_tot, cin, h_tot);
+            state[par ^ 1] = make_float2(aprod, h_end);
+            if (x_row) { x_row[(size_t)chunk * 2] = aprod; x_row[(size_t)chunk * 2 + 1] = h_end; }
+        }
+        if constexpr (kTiledStore) store_pass_f32(y_tile[wave], o_buf, chunk * SS2D_SCAN_CHUNK + wave * kPass, lane, y);
+        else store_items_buffer<out_t>(o_buf, pos, y);
+    };
+    // whole turns of the ring, then the last, partial turn as straight code (a `break` inside the turn would be one more
+    // way into the loop header, from a state with fresh loads outstanding, and the waits there would have to allow for it)
+    int c0 = 0;
+    for (; c0 + kRing <= n_chunks; c0 += kRing) {
+#pragma unroll
+        for (int s = 0; s < kRing; ++s) {
+            do_chunk(c0 + s, ring[s]);
+            issue(c0 + s + kRing, ring[s]);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < kRing - 1; ++s)
+        if (c0 + s < n_chunks) do_chunk(c0 + s, ring[s]);
 }
 
 // ---- host side -----------------------------------------------------------------------------
@@ -541,6 +659,14 @@ static int launch_flat(const ScanArgs &a_in, hipStream_t stream) {
 template <typename in_t, typename out_t, bool kVec>
 static int launch_scan(const ScanArgs &a, bool split_rows, hipStream_t stream) {
     if (split_rows) {
+        if constexpr (kVec) {
+            if (a.N == 1) {
+                // one state, vector I/O: the ring kernel (256^2 maps at batch 4: 170 -> 165 us)
+                if (a.softplus) hipLaunchKernelGGL((scan_row4_ring_kernel<in_t, out_t, true>), dim3((uint32_t)a.rows), dim3(kBlock), 0, stream, a);
+                else hipLaunchKernelGGL((scan_row4_ring_kernel<in_t, out_t, false>), dim3((uint32_t)a.rows), dim3(kBlock), 0, stream, a);
+                return launch_status();
+            }
+        }
         const size_t smem = (size_t)(2 * a.N * kWavesPerWg + 2 * a.N) * sizeof(float2);
         if (a.softplus) {
             hipLaunchKernelGGL((scan_row4_kernel<in_t, out_t, kVec, true>), dim3((uint32_t)a.rows), dim3(kBlock), smem, stream, a);
@@ -627,6 +753,7 @@ static int plan_scan(const ss2d_scan_params *q, ScanArgs &a, bool &vec) {
     const int64_t in_strides[] = {a.u_bs, a.u_ds, a.dl_bs, a.dl_ds, a.B_bs, a.B_gs, a.B_ns, a.C_bs, a.C_gs, a.C_ns};
     vec = aligned16(q->u) && aligned16(q->delta) && aligned16(q->B) && aligned16(q->C) && aligned16(q->out);
     vec = vec && (q->seqlen % in_vec == 0) && (q->seqlen % out_vec == 0);
+    vec = vec && q->seqlen < (1 << 29);               // the vector paths address a row with 32-bit byte offsets
     for (int64_t s : in_strides) vec = vec && (s % in_vec == 0);
     vec = vec && (a.o_bs % out_vec == 0) && (a.o_ds % out_vec == 0);
 
