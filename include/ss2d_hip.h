@@ -387,6 +387,16 @@ int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, i
                  int64_t x_rank_stride, int dtype, void *stream);
 
 /*
+ * The same projection with chosen positions overwritten: mask is (K, N) 16-bit words, each 0 or 0xffff, and where a word
+ * is set every channel's delta at that position becomes `fill` (rounded to dtype) instead of the projection; mask == NULL
+ * is ss2d_dt_proj.  For maps with awkward sides that run embedded in padded maps (SS2Dv2.forward_corev2 takes any H x W,
+ * classification/models/vmamba.py:603-640): a delta of -1e30 at the pad positions is a step of exactly 0 after the
+ * softplus, i.e. the identity of the recurrence, so the embedded map's states pass the pads unchanged.
+ */
+int ss2d_dt_proj_masked(const void *x, const void *weight, const void *mask, float fill, void *delta, int K, int D, int R,
+                        int64_t N, int64_t x_dir_stride, int64_t x_rank_stride, int dtype, void *stream);
+
+/*
  * Fused channel-last MLP of a VSS block: out = residual + fc2(GELU(fc1([LayerNorm](x)))) in one kernel, the hidden
  * activations never leaving the registers.  Replaces Mlp.forward (classification/models/vmamba.py:1116-1131: fc1, GELU
  * (erf form), fc2), the residual add of VSSBlock (:1229) and, when ln_weight is given, the block's second LayerNorm

@@ -570,6 +570,30 @@ def test_dt_proj_matches_fp32_matmul(K, D, R, N, dtype):
     assert bool((err2 <= eps * want2.abs() * 1.01 + 1e-6).all())
 
 
+@pytest.mark.parametrize("dtype,fill", [(torch.bfloat16, -1e30), (torch.float16, -65504.0), (torch.bfloat16, 0.25)],
+                         ids=["bf16", "f16", "bf16-small"])
+@pytest.mark.parametrize("K,D,R,N", [(4, 96, 6, 2 * 3600), (4, 384, 24, 5 * 400), (2, 40, 3, 77), (1, 100, 17, 1001), (3, 200, 8, 36)])
+def test_dt_proj_masked_positions_take_the_fill_value(K, D, R, N, dtype, fill):
+    """Marked positions hold the fill value in every channel, bit for bit; the others are the plain projection, bit for bit."""
+    from vmamba_amd.core import dt_proj_hip
+    _announce("dt_proj-masked", K, D, R, N, dtype, fill)
+    g = torch.Generator().manual_seed(K * 1000 + D + R + 1)
+    x = torch.randn(K, R, N, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(K, D, R, generator=g) * R ** -0.5).to(dtype).to(DEV)
+    marked = torch.rand(K, N, generator=g) < 0.3
+    marked[:, -1] = True                                                # the last position, in an odd-length tail too
+    mask = (-marked.to(torch.int16)).to(DEV)
+    plain = dt_proj_hip(x, w)
+    got = dt_proj_hip(x, w, mask, fill)
+    torch.cuda.synchronize()
+    want = torch.where(marked.to(DEV)[:, None, :], torch.tensor(fill, dtype=dtype, device=DEV), plain)
+    assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(RuntimeError):
+        dt_proj_hip(x, w, mask[:, :-1].contiguous(), fill)             # wrong shape
+    with pytest.raises(RuntimeError):
+        dt_proj_hip(x, w, mask.to(torch.int32), fill)                  # wrong type
+
+
 def test_dt_proj_rejections():
     from vmamba_amd.core import dt_proj_hip
     with pytest.raises(RuntimeError):

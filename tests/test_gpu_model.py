@@ -99,10 +99,10 @@ def test_forward_core_bf16_activations():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("channel_first", [True, False], ids=["cf", "cl"])
-@pytest.mark.parametrize("d_model,B,H,W", [(96, 3, 57, 58), (32, 5, 19, 19), (192, 2, 75, 75), (128, 2, 19, 19), (48, 2, 37, 41), (768, 1, 19, 19)])
+@pytest.mark.parametrize("d_model,B,H,W", [(96, 3, 57, 58), (32, 5, 19, 19), (192, 2, 75, 75), (128, 2, 19, 19), (48, 2, 37, 41), (768, 1, 19, 19), (1024, 1, 19, 19)])
 def test_forward_core_on_maps_embedded_in_padded_ones(d_model, B, H, W, channel_first, dtype):
     """16-bit maps whose sides the vector paths do not like run the fused core on a zero-padded map (the added positions made
-    neutral through one more dt_proj rank, or ss2d_core_mask_pads where the rank does not fit) and are cut out of its
+    neutral by the masked dt_proj, or by ss2d_core_mask_pads where the rank is beyond that kernel -- 64 here) and are cut out of its
     result: against the fp32 CPU model at the 16-bit bound, and against the three-operator path of the same module, which
     pads nothing, at a few roundings of the 16-bit output."""
     from vmamba_amd.core import padded_map_size

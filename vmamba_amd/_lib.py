@@ -22,7 +22,7 @@ EXPORTS = ("ss2d_abi_version", "ss2d_strerror", "ss2d_cross_scan", "ss2d_cross_m
            "ss2d_selective_scan_kernel", "ss2d_selective_scan_fwd_maps",
            "ss2d_layer_norm", "ss2d_add_layer_norm", "ss2d_bias_layer_norm", "ss2d_layer_norm_cf", "ss2d_dwconv3x3_silu", "ss2d_cross_scan_1b1", "ss2d_core_fwd",
            "ss2d_core_workspace_bytes", "ss2d_core_fwd_ws", "ss2d_core_mask_pads", "ss2d_core_embed_maps",
-           "ss2d_dt_proj", "ss2d_cross_scan_flex", "ss2d_cross_scan_flex_ws", "ss2d_cross_scan_flex_static", "ss2d_cross_merge_flex",
+           "ss2d_dt_proj", "ss2d_dt_proj_masked", "ss2d_cross_scan_flex", "ss2d_cross_scan_flex_ws", "ss2d_cross_scan_flex_static", "ss2d_cross_merge_flex",
            "ss2d_selective_scan_bwd", "ss2d_transpose_bcl", "ss2d_mlp_fused", "ss2d_linear_cl", "ss2d_linear_cf_ln", "ss2d_stem_conv_ln_gelu", "ss2d_mean_pool_cl")
 
 
@@ -129,6 +129,9 @@ def lib():
         L.ss2d_dt_proj.restype = ctypes.c_int
         L.ss2d_dt_proj.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_int64] * 3 + [ctypes.c_int]
                                    + [ctypes.c_void_p])
+        L.ss2d_dt_proj_masked.restype = ctypes.c_int
+        L.ss2d_dt_proj_masked.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_float, ctypes.c_void_p] + [ctypes.c_int] * 3
+                                          + [ctypes.c_int64] * 3 + [ctypes.c_int, ctypes.c_void_p])
         L.ss2d_cross_scan_flex.restype = ctypes.c_int
         L.ss2d_cross_scan_flex.argtypes = [ctypes.c_void_p] * 2 + [ctypes.c_int] * 9 + [ctypes.c_void_p]
         L.ss2d_cross_scan_flex_ws.restype = ctypes.c_int

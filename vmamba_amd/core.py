@@ -159,9 +159,10 @@ def ss2d_core_hip(x, delta, Bs, Cs, As, Ds=None, delta_bias=None, delta_softplus
 DT_PROJ_MAX_RANK = 48
 
 
-def dt_proj_hip(x, weight):
+def dt_proj_hip(x, weight, mask=None, fill=0.0):
     """delta[k] = weight[k] @ x[k]: x (K, R, N) with contiguous rows (any direction / rank strides), weight (K, D, R),
-    both bf16 or fp16 -> (K, D, N) of the same dtype, on the matrix cores (ss2d_dt_proj)."""
+    both bf16 or fp16 -> (K, D, N) of the same dtype, on the matrix cores (ss2d_dt_proj).  With ``mask`` -- (K, N) int16,
+    0 or -1 -- every channel's delta at the positions marked -1 is ``fill`` instead (ss2d_dt_proj_masked)."""
     _check(x.is_cuda and weight.is_cuda, "dt_proj: vmamba_amd runs on the GPU only")
     _check(x.dim() == 3 and weight.dim() == 3 and x.shape[0] == weight.shape[0] and x.shape[1] == weight.shape[2],
            "dt_proj expects x (K, R, N) and weight (K, D, R)")
@@ -169,10 +170,14 @@ def dt_proj_hip(x, weight):
     _check(x.stride(2) == 1 or x.size(2) == 1, "x must be contiguous in its last dimension")
     K, R, N = x.shape
     D = weight.shape[1]
+    if mask is not None:
+        _check(mask.is_cuda and mask.device == x.device and mask.dtype == torch.int16 and tuple(mask.shape) == (K, N)
+               and mask.is_contiguous(), "dt_proj: mask must be a contiguous (K, N) int16 tensor on x's device")
     weight = weight.contiguous()
     out = torch.empty((K, D, N), device=x.device, dtype=x.dtype)
     with torch.cuda.device(x.device):
-        rc = _lib.lib().ss2d_dt_proj(x.data_ptr(), weight.data_ptr(), out.data_ptr(), K, D, R, N, x.stride(0), x.stride(1),
-                                     _DTYPE_CODE[x.dtype], torch.cuda.current_stream(x.device).cuda_stream)
+        rc = _lib.lib().ss2d_dt_proj_masked(x.data_ptr(), weight.data_ptr(), None if mask is None else mask.data_ptr(), float(fill),
+                                            out.data_ptr(), K, D, R, N, x.stride(0), x.stride(1), _DTYPE_CODE[x.dtype],
+                                            torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "ss2d_dt_proj")
     return out

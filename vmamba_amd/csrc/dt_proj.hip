@@ -16,6 +16,8 @@
 //   * the MFMA row index is mapped to positions through a permutation chosen so that a lane's 16 accumulators are
 //     16 consecutive positions of one channel (two 16-byte LDS writes);
 //   * the W fragments of up to 96 channels stay in registers for all blocks of the wavefront.
+#include <string.h>
+
 #include "ss2d_common.h"
 
 namespace ss2d {
@@ -31,6 +33,8 @@ constexpr uint32_t kDtOutOfRange = 0x7ffffff0u;   // byte offset beyond any buff
 
 struct DtArgs {
     const void *x, *W;
+    const void *mask;                    // optional (K, N) 16-bit words, 0 or 0xffff: where set, the output element is `fill`
+    uint32_t fill2;                      // the fill value's 16 bits, twice
     void *out;
     int32_t K, D, R, d_chunks, blocks_per_wave, vec_ok, w_vec;
     int64_t N, x_ks, x_rs, n_blocks, n_pos_chunks, total_waves;
@@ -98,8 +102,22 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
 
     const int64_t block0 = pos_chunk * p.blocks_per_wave;
     const int64_t block1 = block0 + p.blocks_per_wave < p.n_blocks ? block0 + p.blocks_per_wave : p.n_blocks;
+    const uint16_t *mask = p.mask ? reinterpret_cast<const uint16_t *>(p.mask) + (int64_t)k * p.N : nullptr;
     for (int64_t blk = block0; blk < block1; ++blk) {
         const int64_t n0 = blk * kDtBlock;
+        // the mask words of this lane's 16-byte piece of the block (the same positions for every channel it stores)
+        uint32_t mk[4] = {0u, 0u, 0u, 0u};
+        if (mask) {                                                   // uniform
+            const int64_t n = n0 + 8 * (lane % kPieces);
+            if (p.vec_ok && n + 8 <= p.N) {
+                const uint4 t = *reinterpret_cast<const uint4 *>(mask + n);
+                mk[0] = t.x; mk[1] = t.y; mk[2] = t.z; mk[3] = t.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (n + e < p.N) mk[e / 2] |= (uint32_t)mask[n + e] << (16 * (e % 2));
+            }
+        }
         // ---- x rows of the block -> LDS: kPieces lanes x 16 bytes per row.  With 16-byte loads all of a lane's pieces
         // (one per 8 rows) are requested before the first is parked: one memory latency per block, not one per piece
         if (p.vec_ok) {
@@ -176,7 +194,11 @@ __global__ __launch_bounds__(kBlock) void dt_proj_kernel(const DtArgs p) {
                     const int ch = lane / kPieces + kChPerStore * it, c = lane % kPieces;
                     const int d = d_base + g * kDtTile + ch;
                     const int64_t n = n0 + 8 * c;
-                    const uint4 v = *reinterpret_cast<const uint4 *>(ob + ch * kDtPitch + 8 * c);
+                    uint4 v = *reinterpret_cast<const uint4 *>(ob + ch * kDtPitch + 8 * c);
+                    if (mask) {                                       // uniform
+                        v.x = (v.x & ~mk[0]) | (p.fill2 & mk[0]); v.y = (v.y & ~mk[1]) | (p.fill2 & mk[1]);
+                        v.z = (v.z & ~mk[2]) | (p.fill2 & mk[2]); v.w = (v.w & ~mk[3]) | (p.fill2 & mk[3]);
+                    }
                     if (d < p.D) {
                         T *o = out + (int64_t)d * p.N + n;
                         if (p.vec_ok && n + 8 <= p.N) {
@@ -214,8 +236,27 @@ static int launch_dt_proj(DtArgs a, hipStream_t stream) {
 
 }  // namespace ss2d
 
+// The fill value as the 16 bits of the output type (round to nearest even; beyond the type's range: its infinity).
+static uint32_t fill_bits16(float fill, int dtype) {
+    if (dtype == SS2D_F16) {
+        const _Float16 h = (_Float16)fill;
+        uint16_t b;
+        memcpy(&b, &h, 2);
+        return b;
+    }
+    uint32_t u;
+    memcpy(&u, &fill, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;   // NaN stays NaN
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
 extern "C" int ss2d_dt_proj(const void *x, const void *weight, void *delta, int K, int D, int R, int64_t N,
                             int64_t x_dir_stride, int64_t x_rank_stride, int dtype, void *stream) {
+    return ss2d_dt_proj_masked(x, weight, nullptr, 0.0f, delta, K, D, R, N, x_dir_stride, x_rank_stride, dtype, stream);
+}
+
+extern "C" int ss2d_dt_proj_masked(const void *x, const void *weight, const void *mask, float fill, void *delta, int K, int D,
+                                   int R, int64_t N, int64_t x_dir_stride, int64_t x_rank_stride, int dtype, void *stream) {
     using namespace ss2d;
     if (K < 0 || D < 0 || R < 0 || N < 0 || x_dir_stride < 0 || x_rank_stride < 0) return SS2D_EINVAL;
     if (dtype != SS2D_F32 && dtype != SS2D_BF16 && dtype != SS2D_F16) return SS2D_EINVAL;
@@ -224,6 +265,7 @@ extern "C" int ss2d_dt_proj(const void *x, const void *weight, void *delta, int 
     if (dtype == SS2D_F32 || R > kDtMaxRank || R == 0) return SS2D_ENOTSUP;   // fp32 and wide ranks: the library GEMM
     DtArgs a;
     a.x = x; a.W = weight; a.out = delta;
+    a.mask = mask; a.fill2 = fill_bits16(fill, dtype) * 0x10001u;
     a.K = K; a.D = D; a.R = R; a.N = N; a.x_ks = x_dir_stride; a.x_rs = x_rank_stride;
     a.d_chunks = (D + kDtGroups * kDtTile - 1) / (kDtGroups * kDtTile);
     a.n_blocks = (N + kDtBlock - 1) / kDtBlock;
@@ -239,7 +281,8 @@ extern "C" int ss2d_dt_proj(const void *x, const void *weight, void *delta, int 
     a.w_vec = (R % 4 == 0) && (reinterpret_cast<uintptr_t>(weight) % 8 == 0);
     // 16-byte loads of x and stores of delta: rows and bases on 16-byte boundaries
     a.vec_ok = (N % 8 == 0) && (x_dir_stride % 8 == 0) && (x_rank_stride % 8 == 0) &&
-               (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(delta) % 16 == 0);
+               (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(delta) % 16 == 0) &&
+               (reinterpret_cast<uintptr_t>(mask) % 16 == 0);
     hipStream_t s = (hipStream_t)stream;
     return dtype == SS2D_BF16 ? launch_dt_proj<bf16_t>(a, s) : launch_dt_proj<f16_t>(a, s);
 }

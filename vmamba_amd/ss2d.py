@@ -82,33 +82,35 @@ def init_dt_A_D(d_state, dt_rank, d_inner, dt_scale=1.0, dt_min=0.001, dt_max=0.
     return nn.Parameter(A_logs), nn.Parameter(Ds), nn.Parameter(dt_w), nn.Parameter(dt_b)
 
 
-_PAD_FLAGS = {}            # the most recent map sizes
-_PAD_FLAGS_PINNED = {}     # those a graph capture has read: never dropped, a captured copy kernel holds their address
+_PAD_MASKS = {}            # the most recent (map size, image count) pairs
+_PAD_MASKS_PINNED = {}     # those a graph capture has read: never dropped, a captured kernel holds their address
 
 
-def _pad_flags(H0, W0, H, W, dtype, device):
-    """(4, 1, H*W) tensor: 1 at the scan positions of each direction (cross_scan_fwd's orders,
-    classification/models/csm_triton.py:22-29, on the H x W map) that lie outside its top-left H0 x W0 part, 0 elsewhere."""
-    key = (H0, W0, H, W, dtype, str(device))
-    if key in _PAD_FLAGS_PINNED:
-        return _PAD_FLAGS_PINNED[key]
+def _pad_mask(H0, W0, H, W, n_images, device):
+    """(4, n_images * H*W) int16 tensor for dt_proj_hip: -1 (all bits set) at the scan positions of each direction
+    (cross_scan_fwd's orders, classification/models/csm_triton.py:22-29, on the H x W map) that lie outside the map's
+    top-left H0 x W0 part, 0 elsewhere; the same for every image."""
+    key = (H0, W0, H, W, n_images, str(device))
+    if key in _PAD_MASKS_PINNED:
+        return _PAD_MASKS_PINNED[key]
     capturing = torch.device(device).type == "cuda" and torch.cuda.is_current_stream_capturing()
-    flags = _PAD_FLAGS.pop(key, None)
-    built = flags is None
+    mask = _PAD_MASKS.pop(key, None)
+    built = mask is None
     if built:
         m = torch.zeros((H, W), dtype=torch.bool, device=device)      # built on the device: no host copy inside a capture
         m[H0:, :] = True
         m[:, W0:] = True
         rows, cols = m.flatten(), m.t().flatten()
-        flags = torch.stack([rows, cols, rows.flip(0), cols.flip(0)]).to(dtype).view(4, 1, H * W)
+        one = -torch.stack([rows, cols, rows.flip(0), cols.flip(0)]).to(torch.int16)
+        mask = one.view(4, 1, H * W).expand(4, n_images, H * W).reshape(4, n_images * H * W)
     if capturing:
         if not built:              # (built inside the capture, its memory is the graph's own and is rewritten by every replay)
-            _PAD_FLAGS_PINNED[key] = flags
-        return flags
-    _PAD_FLAGS[key] = flags                                           # (re-)inserted as the newest
-    while len(_PAD_FLAGS) > 8:
-        _PAD_FLAGS.pop(next(iter(_PAD_FLAGS)))
-    return flags
+            _PAD_MASKS_PINNED[key] = mask
+        return mask
+    _PAD_MASKS[key] = mask                                            # (re-)inserted as the newest
+    while len(_PAD_MASKS) > 8:
+        _PAD_MASKS.pop(next(iter(_PAD_MASKS)))
+    return mask
 
 
 class SS2D(nn.Module):
@@ -250,31 +252,24 @@ class SS2D(nn.Module):
         vec = 16 // proj.element_size()
         unit = vec // math.gcd(L, vec)
         Bp = (B + unit - 1) // unit * unit
-        # On a padded map the step of the added positions must be 0.  With a 16-bit dt_proj on the matrix cores that costs
-        # one more rank: a row that is 1 at the added positions of each direction's order and 0 elsewhere, in front of the
-        # dt rows, against a weight column of -1e30 (-65504 in fp16) -- delta there is that value exactly (x = 0 makes the
-        # other ranks' terms 0), softplus of it is 0, and elsewhere the extra term is -0.  Otherwise ss2d_core_mask_pads
-        # writes -inf into delta afterwards, a scattered pass over its rows.
-        flag_rank = padded is not None and proj.dtype != torch.float32 and R + 1 <= DT_PROJ_MAX_RANK
-        off = 1 if flag_rank else 0
-        x_dbl = proj.new_empty((K, C + off, B, L)) if Bp == B else proj.new_zeros((K, C + off, Bp, L))
-        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl[:, off:, :B].permute(2, 0, 1, 3))
-        if flag_rank:
-            x_dbl[:, 0].copy_(_pad_flags(H0, W0, H, W, proj.dtype, proj.device).expand(K, Bp, L))
-            w_dt = consts.get("Wdt_flag")
-            if w_dt is None:
+        # On a padded map the step of the added positions must be 0: the 16-bit dt_proj on the matrix cores writes -1e30
+        # (-65504 in fp16) there instead of the projection (a mask of those positions in each direction's order), and the
+        # softplus of that is exactly 0.  Otherwise ss2d_core_mask_pads writes -inf into delta afterwards, a scattered
+        # pass over its rows.
+        x_dbl = proj.new_empty((K, C, B, L)) if Bp == B else proj.new_zeros((K, C, Bp, L))
+        cross_scan_1b1_hip(proj.view(B, K, C, H, W), out=x_dbl[:, :, :B].permute(2, 0, 1, 3))
+        dts = x_dbl[:, :R].reshape(K, R, Bp * L)
+        if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
+            if padded is not None:
                 big = -65504.0 if proj.dtype == torch.float16 else -1e30
-                w_dt = consts["Wdt_flag"] = torch.cat([self.dt_projs_weight.new_full((K, D, 1), big), self.dt_projs_weight], dim=2)
-            delta = dt_proj_hip(x_dbl[:, :R + 1].reshape(K, R + 1, Bp * L), w_dt).view(K, D, Bp, L)
-        else:
-            dts = x_dbl[:, :R].reshape(K, R, Bp * L)
-            if dts.dtype != torch.float32 and R <= DT_PROJ_MAX_RANK:
-                delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
+                delta = dt_proj_hip(dts, self.dt_projs_weight, _pad_mask(H0, W0, H, W, Bp, proj.device), big).view(K, D, Bp, L)
             else:
-                delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
+                delta = dt_proj_hip(dts, self.dt_projs_weight).view(K, D, Bp, L)
+        else:
+            delta = torch.bmm(self.dt_projs_weight, dts).view(K, D, Bp, L)
             if padded is not None:
                 core_mask_pads_hip(delta[:, :, :B], H0, W0, H, W)
-        y = ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, off + R, :B], x_dbl[:, off + R + 1, :B], consts["As"].view(-1), consts["Ds"],
+        y = ss2d_core_hip(x, delta[:, :, :B], x_dbl[:, R, :B], x_dbl[:, R + 1, :B], consts["As"].view(-1), consts["Ds"],
                           consts["dt_bias"], True)
         if not crop:
             return y, (H, W)
