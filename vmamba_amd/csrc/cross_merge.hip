@@ -26,16 +26,19 @@ template <typename T> __device__ __forceinline__ T add_rn(T a, T b) { return fro
 template <typename T, int kVec> struct MergePack { using type = T; };
 template <> struct MergePack<bf16_t, 2> { using type = uint32_t; };
 template <> struct MergePack<f16_t, 2> { using type = uint32_t; };
+template <> struct MergePack<float, 4> { using type = float4; };     // fp32 maps of 4n positions: 16 bytes to a lane
 
 template <typename T, int kVec>
 __device__ __forceinline__ T unit_get(typename MergePack<T, kVec>::type p, int i) {
     if constexpr (kVec == 1) return p;
+    else if constexpr (kVec == 4) return i == 0 ? p.x : i == 1 ? p.y : i == 2 ? p.z : p.w;
     else return T{(uint16_t)(p >> (16 * i))};
 }
 template <typename T, int kVec>
-__device__ __forceinline__ typename MergePack<T, kVec>::type unit_make(T a, T b) {
-    if constexpr (kVec == 1) return a;
-    else return (uint32_t)a.bits | ((uint32_t)b.bits << 16);
+__device__ __forceinline__ typename MergePack<T, kVec>::type unit_make(const T (&v)[kVec]) {
+    if constexpr (kVec == 1) return v[0];
+    else if constexpr (kVec == 4) return make_float4(v[0], v[1], v[2], v[3]);
+    else return (uint32_t)v[0].bits | ((uint32_t)v[1].bits << 16);
 }
 // element i of the unit that sits REVERSED in memory
 template <typename T, int kVec>
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
                 }
                 if (++w == (uint32_t)W) { w = 0; ++h; }
             }
-            reinterpret_cast<unit_t *>(o)[q] = unit_make<T, kVec>(res[0], res[kVec - 1]);
+            reinterpret_cast<unit_t *>(o)[q] = unit_make<T, kVec>(res);
         }
     }
 }
@@ -208,7 +211,17 @@ static int launch_cross_merge(const void *ys, void *out, int B, int C, int H, in
         if constexpr (sizeof(T) == 2) {
             pairs = (L % 2 == 0) && ((reinterpret_cast<uintptr_t>(ys) | reinterpret_cast<uintptr_t>(out)) % 4 == 0);
         }
-        if (pairs) {
+        bool quads = false;
+        if constexpr (sizeof(T) == 4) {
+            quads = (L % 4 == 0) && ((reinterpret_cast<uintptr_t>(ys) | reinterpret_cast<uintptr_t>(out)) % 16 == 0);
+        }
+        if (quads) {
+            if constexpr (sizeof(T) == 4) {
+                hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 4>), dim3((uint32_t)n_wg), dim3(kBlock),
+                                   (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
+                                   make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+            }
+        } else if (pairs) {
             if constexpr (sizeof(T) == 2) {
                 hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 2>), dim3((uint32_t)n_wg), dim3(kBlock),
                                    (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
