@@ -285,6 +285,27 @@ def test_scan_delta_group_broadcast(L):
     check(*make_inputs(25, 2, 24, 2, 1, L, torch.float32, delta_dim=6), True)
 
 
+@pytest.mark.parametrize("batch,dim,L,dtype", [(3, 7, 130, torch.bfloat16), (1, 5, 57, torch.float32), (1, 3, 9, torch.float16),
+                                               (7, 3, 101, torch.bfloat16), (2, 4, 2052, torch.float32), (1, 2, 4100, torch.bfloat16)])
+def test_scan_fp32_output_ends_exactly_at_its_last_element(batch, dim, L, dtype):
+    """fp32 outputs leave as 16-byte stores behind a buffer descriptor that ends with the output: a store across that end
+    must write its elements inside and nothing beyond (runs of any length, 4n + 1 .. 4n + 3 elements included)."""
+    from vmamba_amd.csms6s import _scan_params
+    _announce("scan-out-end", batch, dim, L, dtype)
+    args = make_inputs(28, batch, dim, 1, 1, L, dtype)
+    want, _ = orc.selective_scan(*args, True, out_float=True, return_x=True)
+    u, delta, A, B, C, D, bias = [a.to(DEV) for a in args]
+    n = batch * dim * L
+    buf = torch.full((n + 256,), float("nan"), device=DEV)
+    out = buf[:n].view(batch, dim, L)
+    p = _scan_params(u, delta, A, B, C, D, bias, True, out, None)
+    _lib.check(_lib.lib().ss2d_selective_scan_fwd(p, torch.cuda.current_stream().cuda_stream), "ss2d_selective_scan_fwd")
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(out).any()), "elements of the output left unwritten"
+    assert bool(torch.isnan(buf[n:]).all()), "memory behind the output written"
+    assert torch.allclose(out.cpu(), want, **TOL32)
+
+
 def test_scan_many_rows_long_sequence_uses_one_wave_per_row():
     # >= 16384 rows with L > 2048: the unsplit kernel carries state across 2048-chunks in registers
     _announce("scan-manyrows")
