@@ -72,6 +72,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
     const T *y3 = y2 + CL;
     T *o = out + ((size_t)b * C + c0) * L;
 
+    // (the four operands are read once and the result is written once: streaming accesses.  Stage 1, fp32: 150 -> 130 us
+    // alone, scan + merge 373 -> 352)
     // column-major operands -> LDS, transposed
     for (uint32_t base = threadIdx.x; base < units; base += kBlock * kMergeUnroll) {
         unit_t a[kMergeUnroll], c[kMergeUnroll];
@@ -81,8 +83,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
             const uint32_t q = base + k * kBlock;
             if (q < units) {
                 divmod(q * kVec, divL, mm[k], tt[k]);
-                a[k] = reinterpret_cast<const unit_t *>(y1)[q];
-                c[k] = *reinterpret_cast<const unit_t *>(y3 + mm[k] * L + (L - kVec - tt[k]));
+                a[k] = load_streaming(reinterpret_cast<const unit_t *>(y1) + q);
+                c[k] = load_streaming(reinterpret_cast<const unit_t *>(y3 + mm[k] * L + (L - kVec - tt[k])));
             }
         }
 #pragma unroll
@@ -115,8 +117,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
             const uint32_t q = base + k * kBlock;
             if (q < units) {
                 divmod(q * kVec, divL, mm[k], rr[k]);
-                a[k] = reinterpret_cast<const unit_t *>(y0)[q];
-                c[k] = *reinterpret_cast<const unit_t *>(y2 + mm[k] * L + (L - kVec - rr[k]));
+                a[k] = load_streaming(reinterpret_cast<const unit_t *>(y0) + q);
+                c[k] = load_streaming(reinterpret_cast<const unit_t *>(y2 + mm[k] * L + (L - kVec - rr[k])));
             }
         }
 #pragma unroll
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
                 }
                 if (++w == (uint32_t)W) { w = 0; ++h; }
             }
-            reinterpret_cast<unit_t *>(o)[q] = unit_make<T, kVec>(res);
+            store_streaming(reinterpret_cast<unit_t *>(o) + q, unit_make<T, kVec>(res));
         }
     }
 }
@@ -165,8 +167,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__res
         const uint32_t w = w0 + cc, h = h0 + lane;
         if (h < (uint32_t)H && w < (uint32_t)W) {
             const size_t t = (size_t)w * H + h;
-            const T a = y1[t];
-            const T d = y3[L - 1 - t];
+            const T a = load_streaming(y1 + t);
+            const T d = load_streaming(y3 + (L - 1 - t));
             if (kOrder == SS2D_MERGE_PAIRWISE) {
                 lds[lane * kMTilePitch + cc] = add_rn(a, d);
             } else {
@@ -180,8 +182,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__res
         const uint32_t h = h0 + rr, w = w0 + lane;
         if (h < (uint32_t)H && w < (uint32_t)W) {
             const size_t r = (size_t)h * W + w;
-            const T a = y0[r];
-            const T d = y2[L - 1 - r];
+            const T a = load_streaming(y0 + r);
+            const T d = load_streaming(y2 + (L - 1 - r));
             const uint32_t li = rr * kMTilePitch + lane;
             if (kOrder == SS2D_MERGE_PAIRWISE) {
                 o[r] = add_rn(add_rn(a, d), lds[li]);

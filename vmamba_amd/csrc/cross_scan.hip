@@ -37,13 +37,22 @@ __device__ __forceinline__ typename PackOf<T, kVec>::type pack_reversed(typename
 
 constexpr int kUnroll = 4;
 
-template <typename T, int kVec>
+// kStream: the four outputs leave as non-temporal stores.  Chosen by the host when they are more than the last-level cache
+// holds (stage 1 of VMamba-T at batch 128, 308 MB: 81 -> 65 us); smaller outputs are better left where the next kernel
+// finds them (154 MB: 33 us with ordinary stores, 51 with streaming ones).
+constexpr int64_t kStreamOutputBytes = (int64_t)256 << 20;
+
+template <typename T, int kVec, bool kStream>
 __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__restrict__ x, T *__restrict__ y, int C,
                                                                  int H, int W, int G, int groups_per_image,
                                                                  FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
     using pack_t = typename PackOf<T, kVec>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *lds = reinterpret_cast<T *>(smem_raw);
+    auto put = [](pack_t *dst, pack_t v) {
+        if constexpr (kStream) store_streaming(dst, v);
+        else *dst = v;
+    };
 
     const uint32_t wg = blockIdx.x;
     const uint32_t b = wg / (uint32_t)groups_per_image;
@@ -77,8 +86,8 @@ __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__rest
             uint32_t m, j, h, w;
             divmod(q * kVec, divL, m, j);
             divmod(j, divW, h, w);
-            y0_p[q] = v[k];
-            *reinterpret_cast<pack_t *>(y2 + m * L + (L - kVec - j)) = pack_reversed<T, kVec>(v[k]);
+            put(&y0_p[q], v[k]);
+            put(reinterpret_cast<pack_t *>(y2 + m * L + (L - kVec - j)), pack_reversed<T, kVec>(v[k]));
 #pragma unroll
             for (int i = 0; i < kVec; ++i) {
                 lds[m * Lp + h * Wp + w] = pack_get<T, kVec>(v[k], i);
@@ -104,8 +113,8 @@ __global__ __launch_bounds__(kBlock) void cross_scan_maps_kernel(const T *__rest
                 const uint32_t hi = lds[m * Lp + h * Wp + w];
                 v = lo | (hi << 16);
             }
-            y1_p[q] = v;
-            *reinterpret_cast<pack_t *>(y3 + m * L + (L - kVec - t)) = pack_reversed<T, kVec>(v);
+            put(&y1_p[q], v);
+            put(reinterpret_cast<pack_t *>(y3 + m * L + (L - kVec - t)), pack_reversed<T, kVec>(v));
         }
     }
 }
@@ -314,17 +323,19 @@ static int launch_cross_scan(const void *x, void *y, int B, int C, int H, int W,
                 }
             }
         }
+        const bool stream_out = 4 * (int64_t)B * C * L * (int64_t)sizeof(T) > kStreamOutputBytes;
+#define SS2D_LAUNCH_MAPS(VEC, ST)                                                                                              \
+    hipLaunchKernelGGL((cross_scan_maps_kernel<T, VEC, ST>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds), stream, \
+                       (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H),          \
+                       make_fastdiv((uint32_t)W), Wp)
         if (pairs) {
             if constexpr (sizeof(T) == 2) {
-                hipLaunchKernelGGL((cross_scan_maps_kernel<T, 2>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds),
-                                   stream, (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
-                                   make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+                if (stream_out) SS2D_LAUNCH_MAPS(2, true); else SS2D_LAUNCH_MAPS(2, false);
             }
         } else {
-            hipLaunchKernelGGL((cross_scan_maps_kernel<T, 1>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds),
-                               stream, (const T *)x, (T *)y, C, H, W, G, groups, make_fastdiv((uint32_t)L),
-                               make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+            if (stream_out) SS2D_LAUNCH_MAPS(1, true); else SS2D_LAUNCH_MAPS(1, false);
         }
+#undef SS2D_LAUNCH_MAPS
     } else {
         const int tiles_h = (H + kTile - 1) / kTile, tiles_w = (W + kTile - 1) / kTile;
         const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;

@@ -66,22 +66,27 @@ int launch_core_tiled(const CoreArgs &a, int in_dtype, void *workspace, hipStrea
 template <typename T> struct Raw8 { uint32_t w[sizeof(T) * 2]; };
 
 // Items at positions >= L come back as `fill`.
-template <typename T, bool kVec>
+template <typename T, bool kVec, bool kStream = false>
 __device__ __forceinline__ Raw8<T> load_raw(const T *__restrict__ row, int pos, int L, float fill = 0.0f) {
     Raw8<T> r;
+    // kStream: data read once (u, delta of a scan) as non-temporal loads of the vector path
+    auto get = [](const T *src) {
+        if constexpr (kStream) return load_streaming(reinterpret_cast<const uint4 *>(src));
+        else return *reinterpret_cast<const uint4 *>(src);
+    };
     if constexpr (kVec) {
         // the host guarantees 16-byte alignment and L % (16/sizeof(T)) == 0, so a vector is either
         // entirely inside the row or entirely outside
         if constexpr (sizeof(T) == 2) {
             const uint32_t fill2 = (uint32_t)from_f32<T>(fill).bits * 0x10001u;
             uint4 v = make_uint4(fill2, fill2, fill2, fill2);
-            if (pos < L) v = *reinterpret_cast<const uint4 *>(row + pos);
+            if (pos < L) v = get(row + pos);
             r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z; r.w[3] = v.w;
         } else {
             const uint32_t f = f32_to_bits(fill);
             uint4 lo = make_uint4(f, f, f, f), hi = lo;
-            if (pos < L) lo = *reinterpret_cast<const uint4 *>(row + pos);
-            if (pos + 4 < L) hi = *reinterpret_cast<const uint4 *>(row + pos + 4);
+            if (pos < L) lo = get(row + pos);
+            if (pos + 4 < L) hi = get(row + pos + 4);
             r.w[0] = lo.x; r.w[1] = lo.y; r.w[2] = lo.z; r.w[3] = lo.w;
             r.w[4] = hi.x; r.w[5] = hi.y; r.w[6] = hi.z; r.w[7] = hi.w;
         }
@@ -166,14 +171,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t row_buffer(const T *row, int n
 }
 
 // Eight elements from position `pos` of such a row (16-byte aligned: the vector paths' precondition).
-template <typename T>
+template <typename T, bool kStream = false>
 __device__ __forceinline__ Raw8<T> load_raw_buffer(__amdgpu_buffer_rsrc_t rsrc, int pos) {
     Raw8<T> r;
     const int byte_off = pos * (int)sizeof(T);
-    const auto lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
+    constexpr int kAux = kStream ? 2 : 0;                        // the builtin's cache-policy operand: bit 1 = nt
+    const auto lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, kAux);
     r.w[0] = lo[0]; r.w[1] = lo[1]; r.w[2] = lo[2]; r.w[3] = lo[3];
     if constexpr (sizeof(T) == 4) {
-        const auto hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, 0, 0);
+        const auto hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off + 16, 0, kAux);
         r.w[4] = hi[0]; r.w[5] = hi[1]; r.w[6] = hi[2]; r.w[7] = hi[3];
     }
     return r;
@@ -211,8 +217,11 @@ __device__ __forceinline__ void store_pass_f32(float *tile, __amdgpu_buffer_rsrc
     const float4 lo = t4[lane], hi = t4[kWave + lane];
     const words4_t wl = {f32_to_bits(lo.x), f32_to_bits(lo.y), f32_to_bits(lo.z), f32_to_bits(lo.w)};
     const words4_t wh = {f32_to_bits(hi.x), f32_to_bits(hi.y), f32_to_bits(hi.z), f32_to_bits(hi.w)};
-    __builtin_amdgcn_raw_buffer_store_b128(wl, rsrc, (pass_pos + 4 * lane) * 4, 0, 0);
-    __builtin_amdgcn_raw_buffer_store_b128(wh, rsrc, (pass_pos + kPass / 2 + 4 * lane) * 4, 0, 0);
+    // non-temporal: the outputs are written once and read back by another kernel after hundreds of MB of other traffic
+    // (stand-alone scan -2.5 .. -8 % by shape, scan + CrossMerge chains -2 .. -8 % except +2 % on 256 x 256 maps)
+    constexpr int kNonTemporal = 2;      // the builtin's cache-policy operand: bit 1 = nt
+    __builtin_amdgcn_raw_buffer_store_b128(wl, rsrc, (pass_pos + 4 * lane) * 4, 0, kNonTemporal);
+    __builtin_amdgcn_raw_buffer_store_b128(wh, rsrc, (pass_pos + kPass / 2 + 4 * lane) * 4, 0, kNonTemporal);
 }
 
 template <typename T>

@@ -104,6 +104,24 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
     return bits_to_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_to_bits(v), lane));
 }
 
+// ---- streaming accesses ---------------------------------------------------------------------------------------
+// Non-temporal loads and stores for data that is read once, or written once and read back only after far more traffic
+// than the caches hold: they leave the cache replacement order alone.  U: any trivially copyable type of 1, 2, 4, 8 or 16 bytes.
+template <int kBytes> struct StreamWord;
+template <> struct StreamWord<1> { using type = uint8_t; };
+template <> struct StreamWord<2> { using type = uint16_t; };
+template <> struct StreamWord<4> { using type = uint32_t; };
+template <> struct StreamWord<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct StreamWord<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <typename U> __device__ __forceinline__ U load_streaming(const U *p) {
+    using W = typename StreamWord<sizeof(U)>::type;
+    return __builtin_bit_cast(U, __builtin_nontemporal_load(reinterpret_cast<const W *>(p)));
+}
+template <typename U> __device__ __forceinline__ void store_streaming(U *p, U v) {
+    using W = typename StreamWord<sizeof(U)>::type;
+    __builtin_nontemporal_store(__builtin_bit_cast(W, v), reinterpret_cast<W *>(p));
+}
+
 // ---- matrix cores -------------------------------------------------------------------------------------------
 // v_mfma_f32_32x32x8 (bf16 / f16 operands, fp32 accumulate): D (32 x 32) += A (32 x 8) * B (8 x 32).  Lane l supplies
 // A[l % 32][4*(l/32) .. +3] and B[4*(l/32) .. +3][l % 32] as two dwords of packed 16-bit values, and holds
