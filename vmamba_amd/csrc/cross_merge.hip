@@ -48,7 +48,12 @@ __device__ __forceinline__ T unit_get_reversed(typename MergePack<T, kVec>::type
 
 constexpr int kMergeUnroll = 4;
 
-template <typename T, int kOrder, int kVec>
+// kStream: operands and result as non-temporal accesses.  Chosen by the host when the four operands are more than the
+// last-level cache holds (they are read once, the result is written once: stage 1, fp32, 616 MB: 150 -> 131 us alone,
+// scan + merge 373 -> 352); smaller ones are found in the cache by ordinary loads (stage 3, 154 MB: 30 us against 36).
+constexpr int64_t kStreamOperandBytes = (int64_t)256 << 20;
+
+template <typename T, int kOrder, int kVec, bool kStream>
 __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__restrict__ ys, T *__restrict__ out, int C,
                                                                   int H, int W, int G, int groups_per_image,
                                                                   FastDiv divL, FastDiv divH, FastDiv divW, int Wp) {
@@ -72,8 +77,10 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
     const T *y3 = y2 + CL;
     T *o = out + ((size_t)b * C + c0) * L;
 
-    // (the four operands are read once and the result is written once: streaming accesses.  Stage 1, fp32: 150 -> 130 us
-    // alone, scan + merge 373 -> 352)
+    auto get = [](const unit_t *src) {
+        if constexpr (kStream) return load_streaming(src);
+        else return *src;
+    };
     // column-major operands -> LDS, transposed
     for (uint32_t base = threadIdx.x; base < units; base += kBlock * kMergeUnroll) {
         unit_t a[kMergeUnroll], c[kMergeUnroll];
@@ -83,8 +90,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
             const uint32_t q = base + k * kBlock;
             if (q < units) {
                 divmod(q * kVec, divL, mm[k], tt[k]);
-                a[k] = load_streaming(reinterpret_cast<const unit_t *>(y1) + q);
-                c[k] = load_streaming(reinterpret_cast<const unit_t *>(y3 + mm[k] * L + (L - kVec - tt[k])));
+                a[k] = get(reinterpret_cast<const unit_t *>(y1) + q);
+                c[k] = get(reinterpret_cast<const unit_t *>(y3 + mm[k] * L + (L - kVec - tt[k])));
             }
         }
 #pragma unroll
@@ -117,8 +124,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
             const uint32_t q = base + k * kBlock;
             if (q < units) {
                 divmod(q * kVec, divL, mm[k], rr[k]);
-                a[k] = load_streaming(reinterpret_cast<const unit_t *>(y0) + q);
-                c[k] = load_streaming(reinterpret_cast<const unit_t *>(y2 + mm[k] * L + (L - kVec - rr[k])));
+                a[k] = get(reinterpret_cast<const unit_t *>(y0) + q);
+                c[k] = get(reinterpret_cast<const unit_t *>(y2 + mm[k] * L + (L - kVec - rr[k])));
             }
         }
 #pragma unroll
@@ -139,12 +146,13 @@ __global__ __launch_bounds__(kBlock) void cross_merge_maps_kernel(const T *__res
                 }
                 if (++w == (uint32_t)W) { w = 0; ++h; }
             }
-            store_streaming(reinterpret_cast<unit_t *>(o) + q, unit_make<T, kVec>(res));
+            if constexpr (kStream) store_streaming(reinterpret_cast<unit_t *>(o) + q, unit_make<T, kVec>(res));
+            else reinterpret_cast<unit_t *>(o)[q] = unit_make<T, kVec>(res);
         }
     }
 }
 
-template <typename T, int kOrder>
+template <typename T, int kOrder, bool kStream>
 __global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__restrict__ ys, T *__restrict__ out, int C,
                                                                   int H, int W, int tiles_h, int tiles_w) {
     __shared__ T lds[(kOrder == SS2D_MERGE_PAIRWISE ? 1 : 2) * kMTile * kMTilePitch];
@@ -167,8 +175,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__res
         const uint32_t w = w0 + cc, h = h0 + lane;
         if (h < (uint32_t)H && w < (uint32_t)W) {
             const size_t t = (size_t)w * H + h;
-            const T a = load_streaming(y1 + t);
-            const T d = load_streaming(y3 + (L - 1 - t));
+            const T a = kStream ? load_streaming(y1 + t) : y1[t];
+            const T d = kStream ? load_streaming(y3 + (L - 1 - t)) : y3[L - 1 - t];
             if (kOrder == SS2D_MERGE_PAIRWISE) {
                 lds[lane * kMTilePitch + cc] = add_rn(a, d);
             } else {
@@ -182,8 +190,8 @@ __global__ __launch_bounds__(kBlock) void cross_merge_tile_kernel(const T *__res
         const uint32_t h = h0 + rr, w = w0 + lane;
         if (h < (uint32_t)H && w < (uint32_t)W) {
             const size_t r = (size_t)h * W + w;
-            const T a = load_streaming(y0 + r);
-            const T d = load_streaming(y2 + (L - 1 - r));
+            const T a = kStream ? load_streaming(y0 + r) : y0[r];
+            const T d = kStream ? load_streaming(y2 + (L - 1 - r)) : y2[L - 1 - r];
             const uint32_t li = rr * kMTilePitch + lane;
             if (kOrder == SS2D_MERGE_PAIRWISE) {
                 o[r] = add_rn(add_rn(a, d), lds[li]);
@@ -200,6 +208,7 @@ static int launch_cross_merge(const void *ys, void *out, int B, int C, int H, in
     const int Wp = W | 1;
     const int planes = kOrder == SS2D_MERGE_PAIRWISE ? 1 : 2;
     const int64_t map_lds = (int64_t)planes * H * Wp * (int64_t)sizeof(T);
+    const bool stream_ops = 4 * (int64_t)B * C * L * (int64_t)sizeof(T) > kStreamOperandBytes;
     if (map_lds <= kMergeLdsBytes) {
         int G = (int)((kMergeTargetElems + L - 1) / L);
         G = G < 1 ? 1 : G;
@@ -217,29 +226,33 @@ static int launch_cross_merge(const void *ys, void *out, int B, int C, int H, in
         if constexpr (sizeof(T) == 4) {
             quads = (L % 4 == 0) && ((reinterpret_cast<uintptr_t>(ys) | reinterpret_cast<uintptr_t>(out)) % 16 == 0);
         }
+#define SS2D_LAUNCH_MERGE_MAPS(VEC, ST)                                                                                        \
+    hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, VEC, ST>), dim3((uint32_t)n_wg), dim3(kBlock), (size_t)(G * map_lds), \
+                       stream, (const T *)ys, (T *)out, C, H, W, G, groups, make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), \
+                       make_fastdiv((uint32_t)W), Wp)
         if (quads) {
             if constexpr (sizeof(T) == 4) {
-                hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 4>), dim3((uint32_t)n_wg), dim3(kBlock),
-                                   (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
-                                   make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+                if (stream_ops) SS2D_LAUNCH_MERGE_MAPS(4, true); else SS2D_LAUNCH_MERGE_MAPS(4, false);
             }
         } else if (pairs) {
             if constexpr (sizeof(T) == 2) {
-                hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 2>), dim3((uint32_t)n_wg), dim3(kBlock),
-                                   (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
-                                   make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+                if (stream_ops) SS2D_LAUNCH_MERGE_MAPS(2, true); else SS2D_LAUNCH_MERGE_MAPS(2, false);
             }
         } else {
-            hipLaunchKernelGGL((cross_merge_maps_kernel<T, kOrder, 1>), dim3((uint32_t)n_wg), dim3(kBlock),
-                               (size_t)(G * map_lds), stream, (const T *)ys, (T *)out, C, H, W, G, groups,
-                               make_fastdiv((uint32_t)L), make_fastdiv((uint32_t)H), make_fastdiv((uint32_t)W), Wp);
+            if (stream_ops) SS2D_LAUNCH_MERGE_MAPS(1, true); else SS2D_LAUNCH_MERGE_MAPS(1, false);
         }
+#undef SS2D_LAUNCH_MERGE_MAPS
     } else {
         const int tiles_h = (H + kMTile - 1) / kMTile, tiles_w = (W + kMTile - 1) / kMTile;
         const int64_t n_wg = (int64_t)B * C * tiles_h * tiles_w;
         if (n_wg > 0x7fffffff) return SS2D_ENOTSUP;
-        hipLaunchKernelGGL((cross_merge_tile_kernel<T, kOrder>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
-                           (const T *)ys, (T *)out, C, H, W, tiles_h, tiles_w);
+        if (stream_ops) {
+            hipLaunchKernelGGL((cross_merge_tile_kernel<T, kOrder, true>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                               (const T *)ys, (T *)out, C, H, W, tiles_h, tiles_w);
+        } else {
+            hipLaunchKernelGGL((cross_merge_tile_kernel<T, kOrder, false>), dim3((uint32_t)n_wg), dim3(kBlock), 0, stream,
+                               (const T *)ys, (T *)out, C, H, W, tiles_h, tiles_w);
+        }
     }
     return launch_status();
 }
